@@ -1,0 +1,117 @@
+/*
+ * mdcn.h -- C ABI of libmdcn_hip.so: modulated deformable convolution (DCNv2)
+ * forward for AMD MI355X (gfx950), written directly in HIP.
+ *
+ * Plain C types only: device pointers and sizes, no torch types.  None of the
+ * calls below allocates device memory, synchronises the stream or throws; all
+ * device work is enqueued on the HIP stream the caller passes.
+ *
+ * What this replaces in the reference (mmcv v2.2.0):
+ *   mmcv/ops/csrc/pytorch/modulated_deform_conv.cpp:62-138   host op: output
+ *       zeroing, the columns scratch, the per-sample im2col launch, the per-group
+ *       addmm_ and the bias add,
+ *   mmcv/ops/csrc/pytorch/cuda/modulated_deform_conv_cuda.cu:5-32 and
+ *   mmcv/ops/csrc/common/cuda/modulated_deform_conv_cuda_kernel.cuh:80-108,186-245
+ *       the im2col device kernel and its sampler,
+ * i.e. everything below `modulated_deform_conv_forward`
+ * (mmcv/ops/csrc/pytorch/pybind.cpp:157-162) once `input.is_cuda()`.
+ */
+#ifndef MDCN_H_
+#define MDCN_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MDCN_ABI_VERSION 1
+
+/* Element type of every tensor of a call (the Python wrapper unifies them to
+ * offset's dtype, mmcv/ops/modulated_deform_conv.py:136-139). */
+enum mdcn_dtype { MDCN_F32 = 0, MDCN_F16 = 1, MDCN_BF16 = 2 };
+
+/* Which device path runs. */
+enum mdcn_path {
+  MDCN_PATH_AUTO = 0,   /* fused MFMA kernel when the shape allows, else direct */
+  MDCN_PATH_FUSED = 1,  /* fused implicit-GEMM MFMA kernel; error if not eligible */
+  MDCN_PATH_DIRECT = 2  /* one thread per output element; any shape */
+};
+
+enum mdcn_status {
+  MDCN_OK = 0,
+  MDCN_ERR_NULL = -1,       /* a required pointer is NULL */
+  MDCN_ERR_SHAPE = -2,      /* non-positive size, or Cin/Cout not divisible by groups / deform groups */
+  MDCN_ERR_DTYPE = -3,      /* dtype is not one of mdcn_dtype */
+  MDCN_ERR_WORKSPACE = -4,  /* workspace missing, misaligned or smaller than mdcn_workspace_bytes() */
+  MDCN_ERR_PATH = -5,       /* MDCN_PATH_FUSED asked for a shape it does not cover */
+  MDCN_ERR_TOO_LARGE = -6,  /* one padded image exceeds the 32-bit byte offsets used on the device */
+  MDCN_ERR_LAUNCH = -7      /* HIP reported a launch error */
+};
+
+/*
+ * One forward call.  All tensors are dense, of element type `dtype`, on the
+ * device that is current when the call is made:
+ *   input  (N, Cin, H, W)                      NCHW
+ *   offset (N, dgroups*2*kh*kw, Ho, Wo)        channel 2t = dy, 2t+1 = dx of tap t = i*kw + j
+ *   mask   (N, dgroups*kh*kw, Ho, Wo)
+ *   weight (Cout, Cin/groups, kh, kw)
+ *   bias   (Cout) or NULL                      NULL <=> with_bias == false
+ *   output (N, Cout, Ho, Wo)                   written in full, need not be initialised
+ * with Ho = (H + 2*ph - (dh*(kh-1)+1))/sh + 1 and Wo likewise
+ * (mmcv/ops/csrc/pytorch/modulated_deform_conv.cpp:87-90).  Sampling positions and
+ * bilinear weights are always computed in fp32; products are accumulated in
+ * fp32 and rounded once to `dtype` after the bias add.
+ */
+typedef struct mdcn_params {
+  const void *input;
+  const void *offset;
+  const void *mask;
+  const void *weight;
+  const void *bias;
+  void *output;
+  void *workspace;        /* device scratch, 256-byte aligned; may be NULL when mdcn_workspace_bytes() == 0 */
+  size_t workspace_bytes;
+  int32_t dtype;          /* enum mdcn_dtype */
+  int32_t path;           /* enum mdcn_path */
+  int32_t N, Cin, H, W;
+  int32_t Cout, kh, kw;
+  int32_t sh, sw, ph, pw, dh, dw;
+  int32_t groups, dgroups;
+} mdcn_params;
+
+/* ABI version of the loaded library (== MDCN_ABI_VERSION it was built with). */
+int mdcn_abi_version(void);
+
+/* Static text for a status code. */
+const char *mdcn_status_string(int status);
+
+/* Output height/width for the shape in *p; returns MDCN_OK or MDCN_ERR_SHAPE. */
+int mdcn_output_size(const mdcn_params *p, int32_t *Ho, int32_t *Wo);
+
+/* 1 when the fused MFMA kernel covers the shape/dtype in *p, else 0. */
+int mdcn_fused_eligible(const mdcn_params *p);
+
+/* Bytes of device scratch mdcn_forward() needs for *p (pointer fields are not
+ * read).  The fused path keeps a zero-bordered channels-last copy of the input
+ * and the repacked weights there; the direct path needs none.  Returns 0 for an
+ * invalid *p (mdcn_forward then reports the error). */
+size_t mdcn_workspace_bytes(const mdcn_params *p);
+
+/* Enqueue the forward on `hip_stream` (a hipStream_t; NULL = the null stream).
+ * Returns an mdcn_status.  Replaces the body of
+ * modulated_deform_conv_forward_fallthrough for device tensors
+ * (mmcv/ops/csrc/pytorch/modulated_deform_conv.cpp:62-138). */
+int mdcn_forward(const mdcn_params *p, void *hip_stream);
+
+/* Same work as mdcn_forward(), with HIP events recorded on `hip_stream` around
+ * each stage; waits for the stream and reports milliseconds per stage:
+ *   ms[0] input re-layout, ms[1] weight repack, ms[2] main kernel, ms[3] total.
+ * Stages a path does not run report 0.  For measurement only. */
+int mdcn_forward_timed(const mdcn_params *p, void *hip_stream, float ms[4]);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MDCN_H_ */

@@ -1,0 +1,75 @@
+"""Builds the native parts of mmcv_amd in-tree.
+
+``libmdcn_hip.so``  hand-written HIP for gfx950 behind the C ABI of include/mdcn.h
+                    (hipcc cross-compiles it without a GPU),
+``_ext*.so``        the PyTorch-ROCm extension module ``mmcv_amd._ext`` (host
+                    compiler only) that mmcv's Python op layer binds to.
+
+Run ``python -m mmcv_amd.build``.
+"""
+import os
+import subprocess
+import sys
+import sysconfig
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG)
+CSRC = os.path.join(PKG, 'csrc')
+LIBDIR = os.path.join(PKG, 'lib')
+HIP_LIB = os.path.join(LIBDIR, 'libmdcn_hip.so')
+EXT_LIB = os.path.join(PKG, '_ext' + sysconfig.get_config_var('EXT_SUFFIX'))
+ROCM = os.environ.get('ROCM_PATH', '/opt/rocm')
+
+HIPCC_FLAGS = [
+    '--offload-arch=gfx950', '-O3', '-std=c++17', '-fPIC', '-shared',
+    # packed-fp32 VALU forms are kept out of the generated code
+    '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
+    '-Wno-unused-command-line-argument',
+]
+
+
+def _run(cmd):
+    print(' '.join(cmd), flush=True)
+    subprocess.check_call(cmd)
+
+
+def build_hip(extra=()):
+    os.makedirs(LIBDIR, exist_ok=True)
+    hipcc = os.path.join(ROCM, 'bin', 'hipcc')
+    _run([hipcc, *HIPCC_FLAGS, *extra, '-I', os.path.join(ROOT, 'include'),
+          '-o', HIP_LIB, os.path.join(CSRC, 'mdcn_api.hip')])
+    return HIP_LIB
+
+
+def build_ext():
+    import torch
+    tdir = os.path.dirname(torch.__file__)
+    tlib = os.path.join(tdir, 'lib')
+    cmd = [
+        'g++', '-O2', '-std=c++17', '-fPIC', '-shared', '-w',
+        '-D__HIP_PLATFORM_AMD__=1', '-DUSE_ROCM=1',
+        '-DTORCH_EXTENSION_NAME=_ext', '-DTORCH_API_INCLUDE_EXTENSION_H',
+        '-D_GLIBCXX_USE_CXX11_ABI=1',
+        '-I', os.path.join(ROOT, 'include'),
+        '-I', os.path.join(tdir, 'include'),
+        '-I', os.path.join(tdir, 'include', 'torch', 'csrc', 'api', 'include'),
+        '-I', os.path.join(ROCM, 'include'),
+        '-I', sysconfig.get_paths()['include'],
+        os.path.join(CSRC, 'ext.cpp'), '-o', EXT_LIB,
+        '-L', LIBDIR, '-lmdcn_hip', '-Wl,-rpath,$ORIGIN/lib',
+        '-L', tlib, '-Wl,-rpath,' + tlib,
+        '-lc10', '-lc10_hip', '-ltorch', '-ltorch_cpu', '-ltorch_hip',
+        '-ltorch_python',
+    ]
+    _run(cmd)
+    return EXT_LIB
+
+
+def build_all():
+    build_hip()
+    build_ext()
+
+
+if __name__ == '__main__':
+    build_all()
+    sys.exit(0)

@@ -1,0 +1,79 @@
+"""ctypes binding of the C ABI in ``include/mdcn.h`` (``lib/libmdcn_hip.so``).
+
+This is the binding a non-PyTorch caller would write; the tests use it to drive
+the library with raw device pointers.  ``import torch`` first so that the process
+holds a single HIP runtime."""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, 'lib', 'libmdcn_hip.so')
+
+MDCN_F32, MDCN_F16, MDCN_BF16 = 0, 1, 2
+PATH_AUTO, PATH_FUSED, PATH_DIRECT = 0, 1, 2
+MDCN_OK = 0
+
+EXPORTS = ('mdcn_abi_version', 'mdcn_status_string', 'mdcn_output_size',
+           'mdcn_fused_eligible', 'mdcn_workspace_bytes', 'mdcn_forward',
+           'mdcn_forward_timed')
+
+
+class MdcnParams(ctypes.Structure):
+    _fields_ = ([(n, ctypes.c_void_p) for n in
+                 ('input', 'offset', 'mask', 'weight', 'bias', 'output',
+                  'workspace')] +
+                [('workspace_bytes', ctypes.c_size_t)] +
+                [(n, ctypes.c_int32) for n in
+                 ('dtype', 'path', 'N', 'Cin', 'H', 'W', 'Cout', 'kh', 'kw',
+                  'sh', 'sw', 'ph', 'pw', 'dh', 'dw', 'groups', 'dgroups')])
+
+
+_lib = None
+
+
+def load():
+    """dlopen the library (raises OSError when it is not built)."""
+    global _lib
+    if _lib is None:
+        lib = ctypes.CDLL(LIB_PATH)
+        P = ctypes.POINTER(MdcnParams)
+        lib.mdcn_abi_version.restype = ctypes.c_int
+        lib.mdcn_abi_version.argtypes = []
+        lib.mdcn_status_string.restype = ctypes.c_char_p
+        lib.mdcn_status_string.argtypes = [ctypes.c_int]
+        lib.mdcn_output_size.restype = ctypes.c_int
+        lib.mdcn_output_size.argtypes = [P, ctypes.POINTER(ctypes.c_int32),
+                                         ctypes.POINTER(ctypes.c_int32)]
+        lib.mdcn_fused_eligible.restype = ctypes.c_int
+        lib.mdcn_fused_eligible.argtypes = [P]
+        lib.mdcn_workspace_bytes.restype = ctypes.c_size_t
+        lib.mdcn_workspace_bytes.argtypes = [P]
+        lib.mdcn_forward.restype = ctypes.c_int
+        lib.mdcn_forward.argtypes = [P, ctypes.c_void_p]
+        lib.mdcn_forward_timed.restype = ctypes.c_int
+        lib.mdcn_forward_timed.argtypes = [P, ctypes.c_void_p,
+                                           ctypes.POINTER(ctypes.c_float)]
+        _lib = lib
+    return _lib
+
+
+def status_string(rc):
+    return load().mdcn_status_string(rc).decode()
+
+
+def make_params(dtype, N, Cin, H, W, Cout, kh, kw, stride=(1, 1), padding=(0, 0),
+                dilation=(1, 1), groups=1, deform_groups=1, path=PATH_AUTO):
+    p = MdcnParams()
+    p.dtype, p.path = dtype, path
+    p.N, p.Cin, p.H, p.W, p.Cout, p.kh, p.kw = N, Cin, H, W, Cout, kh, kw
+    p.sh, p.sw = stride
+    p.ph, p.pw = padding
+    p.dh, p.dw = dilation
+    p.groups, p.dgroups = groups, deform_groups
+    return p
+
+
+def output_size(p):
+    ho, wo = ctypes.c_int32(0), ctypes.c_int32(0)
+    rc = load().mdcn_output_size(ctypes.byref(p), ctypes.byref(ho), ctypes.byref(wo))
+    return rc, ho.value, wo.value

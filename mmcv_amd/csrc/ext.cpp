@@ -1,0 +1,217 @@
+// mmcv_amd._ext: the PyTorch-ROCm side of the drop-in boundary.  It exports the
+// two ops mmcv's Python layer asserts on
+// (mmcv/ops/modulated_deform_conv.py:17-19, mmcv/utils/ext_loader.py:12-16) with
+// the signature and keyword names of mmcv/ops/csrc/pytorch/pybind.cpp:157-170,
+// 641-657, and forwards device tensors to the C ABI of libmdcn_hip.so.
+//
+// There is no CPU implementation here on purpose: a call with CPU tensors
+// raises, the way the reference's device registry does for a device nobody
+// registered (mmcv/ops/csrc/common/pytorch_device_registry.hpp:120-126).
+#include <c10/hip/HIPStream.h>
+#include <torch/extension.h>
+
+#include <string>
+#include <vector>
+
+#include "mdcn.h"
+
+namespace {
+
+using at::Tensor;
+
+int g_path = MDCN_PATH_AUTO;
+
+std::string device_str(const at::Device &d) {
+  std::string s = c10::DeviceTypeName(d.type(), /*lower_case=*/true);
+  if (d.has_index()) s += ":" + std::to_string(d.index());
+  return s;
+}
+
+int mdcn_dtype_of(const Tensor &t) {
+  switch (t.scalar_type()) {
+    case at::kFloat: return MDCN_F32;
+    case at::kHalf: return MDCN_F16;
+    case at::kBFloat16: return MDCN_BF16;
+    default:
+      TORCH_CHECK(false, "\"modulated_deform_conv_forward\" not implemented for '",
+                  c10::toString(t.scalar_type()), "'");
+  }
+}
+
+struct Prepared {
+  mdcn_params p;
+  std::vector<Tensor> keep;  // contiguous copies and the workspace
+};
+
+// Checks in the order of the reference host op
+// (mmcv/ops/csrc/pytorch/modulated_deform_conv.cpp:68-90), then the dispatch
+// checks (pytorch_device_registry.hpp:115-128).
+void prepare(Prepared &pr, const Tensor &input, const Tensor &weight,
+             const Tensor &bias, const Tensor &offset, const Tensor &mask,
+             Tensor &output, int kernel_h, int kernel_w, int stride_h,
+             int stride_w, int pad_h, int pad_w, int dilation_h, int dilation_w,
+             int group, int deformable_group, bool with_bias) {
+  TORCH_CHECK(input.dim() == 4 && weight.dim() == 4 && offset.dim() == 4 &&
+                  mask.dim() == 4,
+              "modulated_deform_conv_forward expects 4-D input, weight, offset and mask");
+  const int64_t batch = input.size(0), channels = input.size(1);
+  const int64_t height = input.size(2), width = input.size(3);
+  const int64_t channels_out = weight.size(0), channels_kernel = weight.size(1);
+  TORCH_CHECK(weight.size(2) == kernel_h && weight.size(3) == kernel_w,
+              "Input shape and kernel shape won't match: (", kernel_h, " x ",
+              kernel_w, " vs ", weight.size(2), " x ", weight.size(3), ").");
+  TORCH_CHECK(channels == channels_kernel * group,
+              "Input shape and kernel channels won't match: (", channels, " vs ",
+              channels_kernel * group, ").");
+
+  const at::Device dev = input.device();
+  TORCH_CHECK(dev.is_cuda(),
+              "modulated_deformable_im2col_impl: implementation for device ",
+              device_str(dev), " not found.");
+  const Tensor *all[] = {&input, &weight, &bias, &offset, &mask, &output};
+  const char *names[] = {"input", "weight", "bias", "offset", "mask", "output"};
+  for (int i = 1; i < 6; ++i)
+    TORCH_CHECK(all[i]->device() == dev, "modulated_deform_conv_forward: at param ",
+                names[i], ", inconsistent device: ", device_str(all[i]->device()),
+                " vs ", device_str(dev));
+  const auto st = input.scalar_type();
+  for (int i = 1; i < 6; ++i)
+    TORCH_CHECK(all[i]->scalar_type() == st,
+                "modulated_deform_conv_forward: expected ", names[i],
+                " to have dtype ", c10::toString(st), " but got ",
+                c10::toString(all[i]->scalar_type()));
+
+  mdcn_params &p = pr.p;
+  p = mdcn_params{};
+  p.dtype = mdcn_dtype_of(input);
+  p.path = g_path;
+  p.N = (int)batch; p.Cin = (int)channels; p.H = (int)height; p.W = (int)width;
+  p.Cout = (int)channels_out; p.kh = kernel_h; p.kw = kernel_w;
+  p.sh = stride_h; p.sw = stride_w; p.ph = pad_h; p.pw = pad_w;
+  p.dh = dilation_h; p.dw = dilation_w;
+  p.groups = group; p.dgroups = deformable_group;
+
+  int32_t Ho = 0, Wo = 0;
+  const int rc = mdcn_output_size(&p, &Ho, &Wo);
+  TORCH_CHECK(rc == MDCN_OK, "modulated_deform_conv_forward: ", mdcn_status_string(rc));
+  const int64_t taps = (int64_t)kernel_h * kernel_w;
+  TORCH_CHECK(offset.size(0) == batch && offset.size(1) == deformable_group * 2 * taps &&
+                  offset.size(2) == Ho && offset.size(3) == Wo,
+              "modulated_deform_conv_forward: offset must be (", batch, ", ",
+              deformable_group * 2 * taps, ", ", Ho, ", ", Wo, "), got ", offset.sizes());
+  TORCH_CHECK(mask.size(0) == batch && mask.size(1) == deformable_group * taps &&
+                  mask.size(2) == Ho && mask.size(3) == Wo,
+              "modulated_deform_conv_forward: mask must be (", batch, ", ",
+              deformable_group * taps, ", ", Ho, ", ", Wo, "), got ", mask.sizes());
+  TORCH_CHECK(output.numel() == batch * channels_out * Ho * Wo && output.is_contiguous(),
+              "modulated_deform_conv_forward: output must be a dense (", batch, ", ",
+              channels_out, ", ", Ho, ", ", Wo, ") tensor, got ", output.sizes());
+  if (with_bias)
+    TORCH_CHECK(bias.numel() == channels_out,
+                "modulated_deform_conv_forward: bias must have ", channels_out,
+                " elements, got ", bias.numel());
+
+  auto dense = [&](const Tensor &t) {
+    pr.keep.push_back(t.contiguous());
+    return pr.keep.back().data_ptr();
+  };
+  p.input = dense(input);
+  p.offset = dense(offset);
+  p.mask = dense(mask);
+  p.weight = dense(weight);
+  p.bias = with_bias ? dense(bias) : nullptr;
+  p.output = output.data_ptr();
+
+  const size_t ws = mdcn_workspace_bytes(&p);
+  if (ws > 0) {
+    // torch's caching allocator: stream-ordered with the launches below
+    pr.keep.push_back(at::empty({(int64_t)ws}, input.options().dtype(at::kByte)));
+    p.workspace = pr.keep.back().data_ptr();
+    p.workspace_bytes = ws;
+  }
+}
+
+void modulated_deform_conv_forward(
+    Tensor input, Tensor weight, Tensor bias, Tensor ones, Tensor offset,
+    Tensor mask, Tensor output, Tensor columns, int kernel_h, int kernel_w,
+    const int stride_h, const int stride_w, const int pad_h, const int pad_w,
+    const int dilation_h, const int dilation_w, const int group,
+    const int deformable_group, const bool with_bias) {
+  // `ones` and `columns` are the reference's scratch placeholders
+  // (mmcv/ops/modulated_deform_conv.py:149); the fused path has no use for them.
+  (void)ones;
+  (void)columns;
+  c10::DeviceGuard guard(input.device());
+  Prepared pr;
+  prepare(pr, input, weight, bias, offset, mask, output, kernel_h, kernel_w,
+          stride_h, stride_w, pad_h, pad_w, dilation_h, dilation_w, group,
+          deformable_group, with_bias);
+  void *stream = (void *)c10::hip::getCurrentHIPStream().stream();
+  const int rc = mdcn_forward(&pr.p, stream);
+  TORCH_CHECK(rc == MDCN_OK, "modulated_deform_conv_forward: ", mdcn_status_string(rc));
+}
+
+// Same call, timed stage by stage with HIP events on the current stream.
+std::vector<double> modulated_deform_conv_forward_timed(
+    Tensor input, Tensor weight, Tensor bias, Tensor offset, Tensor mask,
+    Tensor output, int kernel_h, int kernel_w, int stride_h, int stride_w,
+    int pad_h, int pad_w, int dilation_h, int dilation_w, int group,
+    int deformable_group, bool with_bias) {
+  c10::DeviceGuard guard(input.device());
+  Prepared pr;
+  prepare(pr, input, weight, bias, offset, mask, output, kernel_h, kernel_w,
+          stride_h, stride_w, pad_h, pad_w, dilation_h, dilation_w, group,
+          deformable_group, with_bias);
+  void *stream = (void *)c10::hip::getCurrentHIPStream().stream();
+  float ms[4] = {0, 0, 0, 0};
+  const int rc = mdcn_forward_timed(&pr.p, stream, ms);
+  TORCH_CHECK(rc == MDCN_OK, "modulated_deform_conv_forward: ", mdcn_status_string(rc));
+  return {ms[0], ms[1], ms[2], ms[3]};
+}
+
+void modulated_deform_conv_backward(
+    Tensor input, Tensor weight, Tensor bias, Tensor ones, Tensor offset,
+    Tensor mask, Tensor columns, Tensor grad_input, Tensor grad_weight,
+    Tensor grad_bias, Tensor grad_offset, Tensor grad_mask, Tensor grad_output,
+    int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h,
+    int pad_w, int dilation_h, int dilation_w, int group, int deformable_group,
+    const bool with_bias) {
+  TORCH_CHECK(false,
+              "modulated_deform_conv_backward: this build implements the forward "
+              "pass only");
+}
+
+}  // namespace
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.def("modulated_deform_conv_forward", &modulated_deform_conv_forward,
+        "modulated deform conv forward", py::arg("input"), py::arg("weight"),
+        py::arg("bias"), py::arg("ones"), py::arg("offset"), py::arg("mask"),
+        py::arg("output"), py::arg("columns"), py::arg("kernel_h"),
+        py::arg("kernel_w"), py::arg("stride_h"), py::arg("stride_w"),
+        py::arg("pad_h"), py::arg("pad_w"), py::arg("dilation_h"),
+        py::arg("dilation_w"), py::arg("group"), py::arg("deformable_group"),
+        py::arg("with_bias"));
+  m.def("modulated_deform_conv_backward", &modulated_deform_conv_backward,
+        "modulated deform conv backward", py::arg("input"), py::arg("weight"),
+        py::arg("bias"), py::arg("ones"), py::arg("offset"), py::arg("mask"),
+        py::arg("columns"), py::arg("grad_input"), py::arg("grad_weight"),
+        py::arg("grad_bias"), py::arg("grad_offset"), py::arg("grad_mask"),
+        py::arg("grad_output"), py::arg("kernel_h"), py::arg("kernel_w"),
+        py::arg("stride_h"), py::arg("stride_w"), py::arg("pad_h"),
+        py::arg("pad_w"), py::arg("dilation_h"), py::arg("dilation_w"),
+        py::arg("group"), py::arg("deformable_group"), py::arg("with_bias"));
+  m.def("modulated_deform_conv_forward_timed", &modulated_deform_conv_forward_timed,
+        "forward with per-stage HIP-event timing; returns [relayout, pack, main, total] ms",
+        py::arg("input"), py::arg("weight"), py::arg("bias"), py::arg("offset"),
+        py::arg("mask"), py::arg("output"), py::arg("kernel_h"), py::arg("kernel_w"),
+        py::arg("stride_h"), py::arg("stride_w"), py::arg("pad_h"), py::arg("pad_w"),
+        py::arg("dilation_h"), py::arg("dilation_w"), py::arg("group"),
+        py::arg("deformable_group"), py::arg("with_bias"));
+  m.def("set_path", [](int path) {
+          TORCH_CHECK(path >= MDCN_PATH_AUTO && path <= MDCN_PATH_DIRECT, "path must be 0 (auto), 1 (fused) or 2 (direct)");
+          g_path = path;
+        }, "choose the device path: 0 auto, 1 fused MFMA kernel, 2 direct kernel", py::arg("path"));
+  m.def("get_path", []() { return g_path; });
+  m.def("abi_version", []() { return mdcn_abi_version(); });
+}

@@ -1,0 +1,299 @@
+// C ABI of libmdcn_hip.so (see include/mdcn.h): parameter checks, path choice,
+// workspace carving and kernel launches.  No allocation, no synchronisation
+// (mdcn_forward_timed excepted, which exists to measure).
+#include "../../include/mdcn.h"
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+
+#include "mdcn_common.h"
+#include "mdcn_direct.h"
+#include "mdcn_fused.h"
+#include "mdcn_prepass.h"
+
+namespace {
+
+using namespace mdcn;
+
+constexpr size_t kAlign = 256;
+constexpr size_t kMaxLds = 160 * 1024;
+// Device byte offsets into the channels-last copy are 32-bit.
+constexpr uint64_t kMaxXtBytes = 0xF0000000ull;
+
+inline size_t align_up(size_t v) { return (v + kAlign - 1) / kAlign * kAlign; }
+
+inline size_t elem_size(int dtype) { return dtype == MDCN_F32 ? 4 : 2; }
+
+int check_params(const mdcn_params *p, Geom *g, bool need_ptrs) {
+  if (!p) return MDCN_ERR_NULL;
+  if (p->dtype != MDCN_F32 && p->dtype != MDCN_F16 && p->dtype != MDCN_BF16)
+    return MDCN_ERR_DTYPE;
+  if (p->N <= 0 || p->Cin <= 0 || p->H <= 0 || p->W <= 0 || p->Cout <= 0 ||
+      p->kh <= 0 || p->kw <= 0 || p->sh <= 0 || p->sw <= 0 || p->ph < 0 ||
+      p->pw < 0 || p->dh <= 0 || p->dw <= 0 || p->groups <= 0 || p->dgroups <= 0)
+    return MDCN_ERR_SHAPE;
+  if (p->Cin % p->groups || p->Cout % p->groups || p->Cin % p->dgroups)
+    return MDCN_ERR_SHAPE;
+  const long Ho = ((long)p->H + 2L * p->ph - ((long)p->dh * (p->kh - 1) + 1)) / p->sh + 1;
+  const long Wo = ((long)p->W + 2L * p->pw - ((long)p->dw * (p->kw - 1) + 1)) / p->sw + 1;
+  if ((long)p->H + 2L * p->ph < (long)p->dh * (p->kh - 1) + 1 ||
+      (long)p->W + 2L * p->pw < (long)p->dw * (p->kw - 1) + 1 || Ho <= 0 || Wo <= 0)
+    return MDCN_ERR_SHAPE;
+  if (need_ptrs && (!p->input || !p->offset || !p->mask || !p->weight || !p->output))
+    return MDCN_ERR_NULL;
+  g->N = p->N; g->Cin = p->Cin; g->H = p->H; g->W = p->W;
+  g->Cout = p->Cout; g->kh = p->kh; g->kw = p->kw;
+  g->sh = p->sh; g->sw = p->sw; g->ph = p->ph; g->pw = p->pw;
+  g->dh = p->dh; g->dw = p->dw; g->G = p->groups; g->DG = p->dgroups;
+  g->Ho = (int)Ho; g->Wo = (int)Wo;
+  g->cin_g = p->Cin / p->groups;
+  g->cout_g = p->Cout / p->groups;
+  g->ch_per_dg = p->Cin / p->dgroups;
+  g->taps = p->kh * p->kw;
+  g->Hp = p->H + 2; g->Wp = p->W + 2;
+  return MDCN_OK;
+}
+
+inline int slab_channels(int dtype) { return dtype == MDCN_F32 ? 16 : 32; }
+
+// Output-channel tile of the fused kernel for a group of cout_g channels.
+inline int pick_ct(int cout_g) { return cout_g > 128 ? 256 : (cout_g > 64 ? 128 : 64); }
+
+inline size_t fused_lds(int dtype, int CT, int taps) {
+  return dtype == MDCN_F32 ? fused_lds_bytes<float>(CT, taps)
+                           : fused_lds_bytes<bf16_t>(CT, taps);
+}
+
+bool fused_ok(const mdcn_params *p, const Geom &g) {
+  const int KC = slab_channels(p->dtype);
+  if (g.cin_g % KC || g.ch_per_dg % KC) return false;
+  if (fused_lds(p->dtype, pick_ct(g.cout_g), g.taps) > kMaxLds) return false;
+  // one padded image must fit the 32-bit offsets
+  const uint64_t img = (uint64_t)g.Hp * g.Wp * g.Cin * elem_size(p->dtype);
+  if (img > kMaxXtBytes) return false;
+  if ((uint64_t)g.N * g.Ho * g.Wo > 0x7fffffffull * 1ull) return false;
+  return true;
+}
+
+struct Plan {
+  bool fused;
+  int CT, KC, n_ctiles, slabs;
+  int n_chunk;       // images per launch of the fused path
+  size_t xt_bytes;   // channels-last copy of one chunk
+  size_t wp_bytes;   // packed weights
+};
+
+int make_plan(const mdcn_params *p, const Geom &g, Plan *pl) {
+  const bool ok = fused_ok(p, g);
+  if (p->path == MDCN_PATH_FUSED && !ok) return MDCN_ERR_PATH;
+  pl->fused = ok && p->path != MDCN_PATH_DIRECT;
+  pl->CT = pl->KC = pl->n_ctiles = pl->slabs = pl->n_chunk = 0;
+  pl->xt_bytes = pl->wp_bytes = 0;
+  if (!pl->fused) return MDCN_OK;
+  const size_t es = elem_size(p->dtype);
+  pl->KC = slab_channels(p->dtype);
+  pl->CT = pick_ct(g.cout_g);
+  pl->n_ctiles = (g.cout_g + pl->CT - 1) / pl->CT;
+  pl->slabs = g.cin_g / pl->KC;
+  const uint64_t img = (uint64_t)g.Hp * g.Wp * g.Cin * es;
+  pl->n_chunk = (int)std::min<uint64_t>((uint64_t)g.N, std::max<uint64_t>(1, kMaxXtBytes / img));
+  pl->xt_bytes = align_up((size_t)img * pl->n_chunk);
+  pl->wp_bytes = align_up((size_t)g.G * pl->n_ctiles * pl->slabs * g.taps * pl->CT * pl->KC * es);
+  return MDCN_OK;
+}
+
+template <typename E, int CT>
+hipError_t launch_fused_ct(const FusedArgs &fa, size_t lds, hipStream_t st) {
+  auto kern = fused_kernel<E, CT>;
+  static bool attr_set = false;  // idempotent; a race only repeats the call
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void *)kern,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)kMaxLds);
+    if (e != hipSuccess) return e;
+    attr_set = true;
+  }
+  const int total_wg = fa.n_ptiles * fa.n_ctiles * fa.g.G;
+  const int grid = ((total_wg + 7) / 8) * 8;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, st, fa);
+  return hipGetLastError();
+}
+
+template <typename E>
+hipError_t launch_fused(const FusedArgs &fa, int CT, size_t lds, hipStream_t st) {
+  switch (CT) {
+    case 64: return launch_fused_ct<E, 64>(fa, lds, st);
+    case 128: return launch_fused_ct<E, 128>(fa, lds, st);
+    default: return launch_fused_ct<E, 256>(fa, lds, st);
+  }
+}
+
+struct StageEvents {
+  hipEvent_t ev[4];  // start, after relayout, after pack, after main
+  bool on;
+};
+
+template <typename E>
+int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t st,
+              float *ms) {
+  hipEvent_t ev[2] = {nullptr, nullptr};
+  auto tic = [&]() { if (ms) hipEventRecord(ev[0], st); };
+  auto toc = [&](int slot) {
+    if (!ms) return;
+    hipEventRecord(ev[1], st);
+    hipEventSynchronize(ev[1]);
+    float t = 0.f;
+    hipEventElapsedTime(&t, ev[0], ev[1]);
+    ms[slot] += t;
+  };
+  if (ms) {
+    ms[0] = ms[1] = ms[2] = ms[3] = 0.f;
+    if (hipEventCreate(&ev[0]) != hipSuccess || hipEventCreate(&ev[1]) != hipSuccess)
+      return MDCN_ERR_LAUNCH;
+  }
+  int rc = MDCN_OK;
+  const size_t es = sizeof(E);
+  const long plane_out = (long)g.Ho * g.Wo;
+
+  if (!pl.fused) {
+    const long total = (long)g.N * g.Cout * plane_out;
+    const int grid = (int)std::min<long>((total + 255) / 256, 1L << 20);
+    tic();
+    hipLaunchKernelGGL(direct_kernel<E>, dim3(grid), dim3(256), 0, st, g,
+                       (const E *)p->input, (const E *)p->offset,
+                       (const E *)p->mask, (const E *)p->weight,
+                       (const E *)p->bias, (E *)p->output, total);
+    if (hipGetLastError() != hipSuccess) rc = MDCN_ERR_LAUNCH;
+    toc(2);
+  } else {
+    unsigned char *ws = (unsigned char *)p->workspace;
+    E *xt = (E *)ws;
+    E *wp = (E *)(ws + pl.xt_bytes);
+
+    // weights: once per call
+    {
+      const long total = (long)g.G * pl.n_ctiles * pl.slabs * g.taps * pl.CT * pl.KC;
+      const int grid = (int)std::min<long>((total + 255) / 256, 1L << 16);
+      tic();
+      hipLaunchKernelGGL(pack_weight_kernel<E>, dim3(grid), dim3(256), 0, st, g,
+                         (const E *)p->weight, wp, pl.CT, pl.KC, pl.n_ctiles,
+                         pl.slabs, total);
+      if (hipGetLastError() != hipSuccess) rc = MDCN_ERR_LAUNCH;
+      toc(1);
+    }
+    const size_t lds = fused_lds_bytes<E>(pl.CT, g.taps);
+    for (int n0 = 0; n0 < g.N && rc == MDCN_OK; n0 += pl.n_chunk) {
+      Geom gc = g;
+      gc.N = std::min(pl.n_chunk, g.N - n0);
+      const E *in = (const E *)p->input + (size_t)n0 * g.Cin * g.H * g.W;
+      {
+        const int n_xtiles = (gc.Wp + 63) / 64, n_ctl = (gc.Cin + 63) / 64;
+        const long blocks = (long)gc.N * gc.Hp * n_xtiles * n_ctl;
+        tic();
+        hipLaunchKernelGGL(relayout_kernel<E>, dim3((unsigned)blocks), dim3(256),
+                           0, st, gc, in, xt, n_xtiles, n_ctl);
+        if (hipGetLastError() != hipSuccess) rc = MDCN_ERR_LAUNCH;
+        toc(0);
+      }
+      FusedArgs fa;
+      fa.g = gc;
+      fa.xt = xt;
+      fa.wp = wp;
+      fa.offset = (const E *)p->offset + (size_t)n0 * g.DG * 2 * g.taps * plane_out;
+      fa.mask = (const E *)p->mask + (size_t)n0 * g.DG * g.taps * plane_out;
+      fa.bias = p->bias;
+      fa.out = (E *)p->output + (size_t)n0 * g.Cout * plane_out;
+      fa.total_px = (long)gc.N * plane_out;
+      fa.n_ptiles = (int)((fa.total_px + kPT - 1) / kPT);
+      fa.n_ctiles = pl.n_ctiles;
+      fa.slabs = pl.slabs;
+      fa.pix_bytes = (uint32_t)(g.Cin * es);
+      fa.row_bytes = (uint32_t)((size_t)g.Wp * g.Cin * es);
+      tic();
+      if (launch_fused<E>(fa, pl.CT, lds, st) != hipSuccess) rc = MDCN_ERR_LAUNCH;
+      toc(2);
+    }
+  }
+  if (ms) {
+    ms[3] = ms[0] + ms[1] + ms[2];
+    hipEventDestroy(ev[0]);
+    hipEventDestroy(ev[1]);
+  }
+  return rc;
+}
+
+int run(const mdcn_params *p, void *stream, float *ms) {
+  Geom g;
+  int rc = check_params(p, &g, true);
+  if (rc != MDCN_OK) return rc;
+  Plan pl;
+  rc = make_plan(p, g, &pl);
+  if (rc != MDCN_OK) return rc;
+  if (pl.fused) {
+    const size_t need = pl.xt_bytes + pl.wp_bytes;
+    if (!p->workspace || p->workspace_bytes < need ||
+        ((uintptr_t)p->workspace % kAlign) != 0)
+      return MDCN_ERR_WORKSPACE;
+  }
+  hipStream_t st = (hipStream_t)stream;
+  switch (p->dtype) {
+    case MDCN_F32: return run_typed<float>(p, g, pl, st, ms);
+    case MDCN_F16: return run_typed<f16_t>(p, g, pl, st, ms);
+    default: return run_typed<bf16_t>(p, g, pl, st, ms);
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+int mdcn_abi_version(void) { return MDCN_ABI_VERSION; }
+
+const char *mdcn_status_string(int status) {
+  switch (status) {
+    case MDCN_OK: return "ok";
+    case MDCN_ERR_NULL: return "a required pointer is NULL";
+    case MDCN_ERR_SHAPE: return "invalid shape (non-positive size or channels not divisible by groups)";
+    case MDCN_ERR_DTYPE: return "unsupported dtype";
+    case MDCN_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
+    case MDCN_ERR_PATH: return "shape not covered by the fused path";
+    case MDCN_ERR_TOO_LARGE: return "tensor too large for 32-bit device offsets";
+    case MDCN_ERR_LAUNCH: return "HIP launch error";
+    default: return "unknown status";
+  }
+}
+
+int mdcn_output_size(const mdcn_params *p, int32_t *Ho, int32_t *Wo) {
+  Geom g;
+  const int rc = check_params(p, &g, false);
+  if (rc != MDCN_OK) return rc;
+  if (Ho) *Ho = g.Ho;
+  if (Wo) *Wo = g.Wo;
+  return MDCN_OK;
+}
+
+int mdcn_fused_eligible(const mdcn_params *p) {
+  Geom g;
+  if (check_params(p, &g, false) != MDCN_OK) return 0;
+  return fused_ok(p, g) ? 1 : 0;
+}
+
+size_t mdcn_workspace_bytes(const mdcn_params *p) {
+  Geom g;
+  if (check_params(p, &g, false) != MDCN_OK) return 0;
+  Plan pl;
+  if (make_plan(p, g, &pl) != MDCN_OK) return 0;
+  return pl.fused ? pl.xt_bytes + pl.wp_bytes : 0;
+}
+
+int mdcn_forward(const mdcn_params *p, void *hip_stream) {
+  return run(p, hip_stream, nullptr);
+}
+
+int mdcn_forward_timed(const mdcn_params *p, void *hip_stream, float ms[4]) {
+  if (!ms) return MDCN_ERR_NULL;
+  return run(p, hip_stream, ms);
+}
+
+}  // extern "C"

@@ -1,0 +1,105 @@
+"""Helpers shared by the tests: seeded inputs, the error metric and a thin
+caller of the C ABI with torch device tensors."""
+import ctypes
+import math
+
+import numpy as np
+import torch
+
+from mmcv_amd import capi
+
+TOL = {torch.float32: 1e-4, torch.float16: 2e-2, torch.bfloat16: 2e-2}
+DT = {torch.float32: capi.MDCN_F32, torch.float16: capi.MDCN_F16,
+      torch.bfloat16: capi.MDCN_BF16}
+
+
+def pair(v):
+    return (v, v) if isinstance(v, int) else tuple(v)
+
+
+def out_hw(H, W, kh, kw, stride, padding, dilation):
+    (sh, sw), (ph, pw), (dh, dw) = pair(stride), pair(padding), pair(dilation)
+    return ((H + 2 * ph - (dh * (kh - 1) + 1)) // sh + 1,
+            (W + 2 * pw - (dw * (kw - 1) + 1)) // sw + 1)
+
+
+def make_case(seed, N, Cin, Cout, H, W, k=3, stride=1, padding=1, dilation=1,
+              groups=1, deform_groups=1, sigma=2.0, bias=True):
+    """Seeded fp32 CPU tensors in the fixed order input, offset, mask logits,
+    weight, bias: input ~ N(0,1); offset ~ N(0, sigma) pixels;
+    mask = sigmoid(N(0,1)); weight Kaiming-normal (fan-in, ReLU gain);
+    bias ~ N(0, 0.01)."""
+    kh, kw = pair(k)
+    Ho, Wo = out_hw(H, W, kh, kw, stride, padding, dilation)
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(N, Cin, H, W, generator=g)
+    offset = torch.randn(N, deform_groups * 2 * kh * kw, Ho, Wo, generator=g) * sigma
+    mask = torch.sigmoid(torch.randn(N, deform_groups * kh * kw, Ho, Wo, generator=g))
+    fan_in = Cin // groups * kh * kw
+    weight = torch.randn(Cout, Cin // groups, kh, kw, generator=g) * math.sqrt(2.0 / fan_in)
+    b = torch.randn(Cout, generator=g) * 0.01 if bias else None
+    return dict(input=x, offset=offset, mask=mask, weight=weight, bias=b,
+                stride=pair(stride), padding=pair(padding), dilation=pair(dilation),
+                groups=groups, deform_groups=deform_groups)
+
+
+def rel_err(y, ref):
+    """max|y - ref| / max|ref| over the whole tensor."""
+    y = np.asarray(y, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    return float(np.abs(y - ref).max() / max(np.abs(ref).max(), 1e-30))
+
+
+def oracle_forward(case, dtype=np.float32):
+    """CPU oracle on the (possibly rounded) inputs of `case`."""
+    import oracle
+    f = lambda t: None if t is None else t.detach().cpu().to(torch.float64 if dtype == np.float64 else torch.float32).numpy()
+    return oracle.forward(f(case['input']), f(case['offset']), f(case['mask']),
+                          f(case['weight']), f(case['bias']), case['stride'],
+                          case['padding'], case['dilation'], case['groups'],
+                          case['deform_groups'])
+
+
+def cast_case(case, dtype, device=None):
+    """Round every tensor once to `dtype` (and move it)."""
+    out = dict(case)
+    for k in ('input', 'offset', 'mask', 'weight', 'bias'):
+        if case[k] is not None:
+            t = case[k].to(dtype)
+            out[k] = t.to(device) if device is not None else t
+    return out
+
+
+def capi_forward(case, path=capi.PATH_AUTO, timed=False):
+    """Run the C ABI on device tensors of `case`; returns the output tensor
+    (and the per-stage milliseconds when `timed`)."""
+    lib = capi.load()
+    x, off, msk, w, b = (case[k] for k in ('input', 'offset', 'mask', 'weight', 'bias'))
+    assert x.is_cuda
+    N, Cin, H, W = x.shape
+    Cout, _, kh, kw = w.shape
+    p = capi.make_params(DT[x.dtype], N, Cin, H, W, Cout, kh, kw, case['stride'],
+                         case['padding'], case['dilation'], case['groups'],
+                         case['deform_groups'], path)
+    rc, Ho, Wo = capi.output_size(p)
+    assert rc == 0, capi.status_string(rc)
+    out = torch.empty(N, Cout, Ho, Wo, dtype=x.dtype, device=x.device)
+    ws_bytes = lib.mdcn_workspace_bytes(ctypes.byref(p))
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=x.device)
+    keep = [t.contiguous() for t in (x, off, msk, w)]
+    p.input, p.offset, p.mask, p.weight = (t.data_ptr() for t in keep)
+    p.bias = b.contiguous().data_ptr() if b is not None else None
+    p.output = out.data_ptr()
+    p.workspace = ws.data_ptr() if ws_bytes else None
+    p.workspace_bytes = ws_bytes
+    stream = torch.cuda.current_stream().cuda_stream
+    if timed:
+        ms = (ctypes.c_float * 4)()
+        rc = lib.mdcn_forward_timed(ctypes.byref(p), ctypes.c_void_p(stream), ms)
+        assert rc == 0, capi.status_string(rc)
+        torch.cuda.synchronize()
+        return out, list(ms)
+    rc = lib.mdcn_forward(ctypes.byref(p), ctypes.c_void_p(stream))
+    assert rc == 0, capi.status_string(rc)
+    torch.cuda.synchronize()
+    return out
