@@ -1,0 +1,195 @@
+"""Host-side checks that need no GPU: the C-ABI library loads and exports what
+include/mdcn.h declares, its parameter validation, and the Python op layer's
+mmcv-compatible behaviour (names, errors, registry, state-dict upgrade)."""
+import ctypes
+import os
+import re
+import warnings
+
+import pytest
+import torch
+
+from mmcv_amd import capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, 'include', 'mdcn.h')).read()
+    text = re.sub(r'/\*.*?\*/', '', text, flags=re.S)
+    return sorted(set(re.findall(r'\b(mdcn_[a-z_]+)\s*\(', text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = capi.load()
+    names = declared_functions()
+    assert sorted(names) == sorted(capi.EXPORTS)
+    for n in names:
+        assert hasattr(lib, n), n
+    assert lib.mdcn_abi_version() == 1
+    assert capi.status_string(0) == 'ok'
+    assert 'workspace' in capi.status_string(-4)
+
+
+def test_params_struct_matches_header_order():
+    text = open(os.path.join(ROOT, 'include', 'mdcn.h')).read()
+    body = re.search(r'typedef struct mdcn_params \{(.*?)\} mdcn_params;', text, re.S).group(1)
+    body = re.sub(r'/\*.*?\*/', '', body, flags=re.S)
+    fields = []
+    for decl in body.split(';'):
+        decl = decl.strip()
+        if not decl:
+            continue
+        for name in decl.split(','):
+            fields.append(name.strip().split()[-1].lstrip('*'))
+    assert fields == [f[0] for f in capi.MdcnParams._fields_]
+
+
+def test_output_size_and_shape_errors():
+    p = capi.make_params(capi.MDCN_F32, 16, 512, 50, 50, 512, 3, 3, (2, 2), (1, 1),
+                         (1, 1), 1, 4)
+    assert capi.output_size(p) == (0, 25, 25)
+    p = capi.make_params(capi.MDCN_F32, 1, 4, 2, 2, 4, 3, 3)  # 2x2 input, 3x3 kernel, no pad
+    assert capi.output_size(p)[0] == -2
+    p = capi.make_params(capi.MDCN_F32, 1, 6, 8, 8, 4, 3, 3, groups=4)
+    assert capi.output_size(p)[0] == -2  # Cin % groups
+    p = capi.make_params(capi.MDCN_F32, 1, 6, 8, 8, 6, 3, 3, deform_groups=4)
+    assert capi.output_size(p)[0] == -2
+    p = capi.make_params(7, 1, 4, 8, 8, 4, 3, 3)
+    assert capi.output_size(p)[0] == -3
+    assert capi.load().mdcn_output_size(None, None, None) == -1
+
+
+def test_eligibility_and_workspace():
+    lib = capi.load()
+    # N=16, C=256, 100x152 bf16: fused; copy (102*154*256*2 B per image) + weights
+    p = capi.make_params(capi.MDCN_BF16, 16, 256, 100, 152, 256, 3, 3, (1, 1), (1, 1))
+    assert lib.mdcn_fused_eligible(ctypes.byref(p)) == 1
+    ws = lib.mdcn_workspace_bytes(ctypes.byref(p))
+    assert ws >= 16 * 102 * 154 * 256 * 2 + 256 * 256 * 9 * 2
+    assert ws < 1.02 * (16 * 102 * 154 * 256 * 2 + 256 * 256 * 9 * 2) + 4096
+    # fp32 needs Cin/groups and Cin/deform_groups to be multiples of 16, 16-bit of 32
+    p = capi.make_params(capi.MDCN_F32, 1, 16, 8, 8, 4, 3, 3)
+    assert lib.mdcn_fused_eligible(ctypes.byref(p)) == 1
+    p = capi.make_params(capi.MDCN_F16, 1, 16, 8, 8, 4, 3, 3)
+    assert lib.mdcn_fused_eligible(ctypes.byref(p)) == 0
+    p = capi.make_params(capi.MDCN_F32, 1, 64, 8, 8, 4, 3, 3, deform_groups=8)
+    assert lib.mdcn_fused_eligible(ctypes.byref(p)) == 0
+    assert lib.mdcn_workspace_bytes(ctypes.byref(p)) == 0
+    p.path = capi.PATH_DIRECT
+    assert lib.mdcn_workspace_bytes(ctypes.byref(p)) == 0
+
+
+def test_forward_rejects_bad_calls_before_touching_the_device():
+    lib = capi.load()
+    p = capi.make_params(capi.MDCN_F32, 1, 16, 8, 8, 4, 3, 3, (1, 1), (1, 1))
+    assert lib.mdcn_forward(ctypes.byref(p), None) == -1  # null tensors
+    buf = ctypes.create_string_buffer(64)
+    addr = ctypes.addressof(buf)
+    p.input = p.offset = p.mask = p.weight = p.output = addr
+    assert lib.mdcn_forward(ctypes.byref(p), None) == -4  # fused path, no workspace
+    p.workspace, p.workspace_bytes = addr + 1, 1 << 30
+    assert lib.mdcn_forward(ctypes.byref(p), None) == -4  # misaligned
+    p2 = capi.make_params(capi.MDCN_F32, 1, 3, 8, 8, 4, 3, 3, path=capi.PATH_FUSED)
+    p2.input = p2.offset = p2.mask = p2.weight = p2.output = addr
+    assert lib.mdcn_forward(ctypes.byref(p2), None) == -5
+    assert lib.mdcn_forward_timed(ctypes.byref(p), None, None) == -1
+
+
+# ---- Python op layer ----------------------------------------------------------
+
+def test_ext_module_exports():
+    from mmcv_amd.utils import ext_loader
+    ext = ext_loader.load_ext('_ext', ['modulated_deform_conv_forward',
+                                       'modulated_deform_conv_backward'])
+    assert ext.abi_version() == 1
+    with pytest.raises(AssertionError):
+        ext_loader.load_ext('_ext', ['no_such_op'])
+    with pytest.raises(ImportError):
+        ext_loader.load_ext('_missing', [])
+
+
+def test_public_names():
+    import mmcv_amd.ops as ops
+    for n in ('ModulatedDeformConv2d', 'ModulatedDeformConv2dPack', 'modulated_deform_conv2d'):
+        assert hasattr(ops, n)
+    assert ops.MODELS.get('DCNv2') is ops.ModulatedDeformConv2dPack
+    layer = ops.build_conv_layer(dict(type='DCNv2', deform_groups=2), 8, 6, 3, stride=2, padding=1)
+    assert isinstance(layer, ops.ModulatedDeformConv2dPack)
+    assert layer.conv_offset.out_channels == 2 * 3 * 9
+    assert layer.conv_offset.stride == (2, 2)
+    assert layer.weight.shape == (6, 8, 3, 3) and layer.bias.shape == (6,)
+    assert layer.transposed is False and layer.output_padding == (0,)
+    assert float(layer.conv_offset.weight.detach().abs().sum()) == 0.0
+    bound = 1.0 / (8 * 9) ** 0.5
+    assert float(layer.weight.detach().abs().max()) <= bound and float(layer.bias.detach().abs().sum()) == 0.0
+
+
+def test_deprecated_kwarg():
+    from mmcv_amd.ops import ModulatedDeformConv2d
+    with warnings.catch_warnings(record=True) as w:
+        warnings.simplefilter('always')
+        m = ModulatedDeformConv2d(4, 4, 3, deformable_groups=2, bias=False)
+    assert m.deform_groups == 2 and m.bias is None
+    assert any(issubclass(x.category, DeprecationWarning) for x in w)
+    with pytest.raises(AssertionError):
+        ModulatedDeformConv2d(4, 4, 3, deformable_groups=2, deform_groups=2)
+
+
+def test_python_errors():
+    from mmcv_amd.ops import modulated_deform_conv2d
+    w = torch.zeros(4, 4, 3, 3)
+    with pytest.raises(ValueError, match='Expected 4D tensor'):
+        modulated_deform_conv2d(torch.zeros(4, 8, 8), torch.zeros(1, 18, 8, 8),
+                                torch.zeros(1, 9, 8, 8), w)
+    with pytest.raises(ValueError, match='too small'):
+        modulated_deform_conv2d(torch.zeros(1, 4, 2, 2), torch.zeros(1, 18, 1, 1),
+                                torch.zeros(1, 9, 1, 1), w)
+    # there is no CPU implementation behind this extension: loud error, no fallback
+    with pytest.raises(RuntimeError, match='implementation for device cpu not found'):
+        modulated_deform_conv2d(torch.zeros(1, 4, 8, 8), torch.zeros(1, 18, 8, 8),
+                                torch.zeros(1, 9, 8, 8), w, None, 1, 1)
+    with pytest.raises(RuntimeError, match="kernel channels won't match"):
+        modulated_deform_conv2d(torch.zeros(1, 6, 8, 8), torch.zeros(1, 18, 8, 8),
+                                torch.zeros(1, 9, 8, 8), w, None, 1, 1)
+
+
+def test_state_dict_upgrade():
+    from mmcv_amd.ops import ModulatedDeformConv2dPack
+
+    class Net(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.conv2 = ModulatedDeformConv2dPack(4, 4, 3, padding=1)
+
+    net = Net()
+    sd = net.state_dict()
+    old = {}
+    for k, v in sd.items():
+        old[k.replace('conv2.conv_offset.', 'conv2_offset.')] = torch.full_like(v, 0.5)
+    assert 'conv2_offset.weight' in old
+    # mmengine-style loaders hand every module the whole dict (torch's own
+    # load_state_dict filters it by prefix first, which hides the legacy keys)
+    missing, unexpected, errors = [], [], []
+    net.conv2._load_from_state_dict(old, 'conv2.', {'version': 1}, True, missing,
+                                    unexpected, errors)
+    assert not missing and not errors
+    assert 'conv2.conv_offset.weight' in old and 'conv2_offset.weight' not in old
+    net.conv2.conv_offset._load_from_state_dict(old, 'conv2.conv_offset.', {}, True,
+                                                missing, unexpected, errors)
+    assert float(net.conv2.conv_offset.weight.mean()) == 0.5
+    assert float(net.conv2.conv_offset.bias.mean()) == 0.5
+    # current-format dicts load unchanged through torch's own loader
+    net.load_state_dict(Net().state_dict())
+
+
+def test_onnx_symbolic_name():
+    from mmcv_amd.ops import ModulatedDeformConv2dFunction
+
+    class G:
+        def op(self, name, *args, **kw):
+            return name, len(args), kw
+
+    name, nargs, kw = ModulatedDeformConv2dFunction.symbolic(G(), 1, 2, 3, 4, None, 1, 1, 1, 1, 1)
+    assert name == 'mmcv::MMCVModulatedDeformConv2d' and nargs == 4
+    assert set(kw) == {'stride_i', 'padding_i', 'dilation_i', 'groups_i', 'deform_groups_i'}
