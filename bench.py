@@ -1,0 +1,197 @@
+"""Benchmark of the DCNv2 forward hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg4]
+
+One "step" is one call of the extension op ``modulated_deform_conv_forward`` (the
+drop-in boundary) on synthetic inputs that are already resident in HBM, at the
+configuration the headline metric is quoted on: bf16, N=16, Cin=Cout=256,
+100x152, 3x3, stride 1, pad 1.  Prints ONE JSON line on stdout; progress and the
+per-stage breakdown go to stderr.
+
+  value       whole-op TFLOP/s (2*N*Ho*Wo*Cout*Cin/groups*kh*kw divided by the
+              time of one step, re-layout and weight repack included)
+  roofline    the fused main kernel alone against the dense bf16 MFMA peak,
+              its launch time measured with HIP events on the stream it runs on
+  cpu_baseline  the reference's own CPU path (compiled from its sources into
+              oracle/_ref) or, when that is absent, the C restatement, timed on
+              this host on a bounded number of samples of the same workload
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, 'tests'))
+
+PEAK_TFLOPS = {'bf16': 2500.0, 'f16': 2500.0, 'f32': 157.3}
+HBM_PEAK_GBS = 8000.0
+
+WORKLOADS = {
+    'cfg1': dict(N=1, Cin=64, Cout=64, H=56, W=56, sigma=2.0, dtype='f32'),
+    'cfg2': dict(N=8, Cin=256, Cout=256, H=64, W=64, sigma=4.0, dtype='f32'),
+    'cfg3': dict(N=16, Cin=512, Cout=512, H=50, W=50, stride=2, deform_groups=4,
+                 sigma=3.0, dtype='f32'),
+    'cfg4': dict(N=16, Cin=256, Cout=256, H=100, W=152, sigma=2.0, dtype='bf16'),
+    'cfg4_f16': dict(N=16, Cin=256, Cout=256, H=100, W=152, sigma=2.0, dtype='f16'),
+}
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def cpu_baseline(case, flops_per_sample, budget_s=20.0):
+    """Time the CPU path on as many samples of the workload as fit the budget."""
+    import torch
+    import oracle
+    N = case['input'].shape[0]
+    args = lambda n: dict(stride=case['stride'], padding=case['padding'],
+                          dilation=case['dilation'], groups=case['groups'],
+                          deform_groups=case['deform_groups'])
+    use_ref = oracle.load_reference_ext() is not None
+
+    def run(n):
+        t = {k: case[k][:n] for k in ('input', 'offset', 'mask')}
+        t0 = time.perf_counter()
+        if use_ref:
+            oracle.reference_forward(t['input'], t['offset'], t['mask'], case['weight'],
+                                     case['bias'], **args(n))
+        else:
+            oracle.forward(t['input'].numpy(), t['offset'].numpy(), t['mask'].numpy(),
+                           case['weight'].numpy(), case['bias'].numpy(), **args(n))
+        return time.perf_counter() - t0
+
+    t1 = run(1)  # also the warm-up
+    n = int(max(1, min(N, budget_s // max(t1, 1e-3))))
+    tn = run(n)
+    threads = torch.get_num_threads() if use_ref else int(os.environ.get('OMP_NUM_THREADS', os.cpu_count()))
+    return {
+        'value': round(flops_per_sample * n / tn / 1e12, 5),
+        'unit': 'TFLOP/s',
+        'cores': threads,
+        'kind': 'reference' if use_ref else 'port',
+        'sample': (f'{n} of {N} samples of the same workload in fp32, {tn:.2f} s '
+                   f'({tn / n * 1e3:.0f} ms/sample; im2col stage is single-threaded, '
+                   f'GEMM uses {threads} threads)'),
+        'ms_per_layer_extrapolated': round(tn / n * N * 1e3, 1),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=50)
+    ap.add_argument('--warmup', type=int, default=10)
+    ap.add_argument('--workload', default='cfg4', choices=sorted(WORKLOADS))
+    ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
+    a = ap.parse_args()
+    if a.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
+        log('bench.py: this path is built and measured on ONE GPU; '
+            'samples and pixel tiles are independent, so more GPUs only split the batch. '
+            'Run with --gpus 1.')
+        sys.exit(2)
+
+    import torch
+    from common import make_case, cast_case
+    from mmcv_amd.ops.modulated_deform_conv import ext_module
+
+    assert torch.cuda.is_available(), 'bench.py needs a GPU'
+    torch.cuda.set_device(0)
+    wl = dict(WORKLOADS[a.workload])
+    dname = wl.pop('dtype')
+    dtype = {'bf16': torch.bfloat16, 'f16': torch.float16, 'f32': torch.float32}[dname]
+    seed = 20240 + int(a.workload[3])
+    case = make_case(seed, **wl)
+    dev = cast_case(case, dtype, 'cuda')
+    N, Cin, H, W = case['input'].shape
+    Cout, cin_g, kh, kw = case['weight'].shape
+    x, off, msk, w, b = (dev[k] for k in ('input', 'offset', 'mask', 'weight', 'bias'))
+    (sh, sw), (ph, pw), (dh, dw) = case['stride'], case['padding'], case['dilation']
+    Ho = (H + 2 * ph - (dh * (kh - 1) + 1)) // sh + 1
+    Wo = (W + 2 * pw - (dw * (kw - 1) + 1)) // sw + 1
+    out = torch.empty(N, Cout, Ho, Wo, dtype=dtype, device='cuda')
+    empty = x.new_empty(0)
+    kwargs = dict(kernel_h=kh, kernel_w=kw, stride_h=sh, stride_w=sw, pad_h=ph, pad_w=pw,
+                  dilation_h=dh, dilation_w=dw, group=case['groups'],
+                  deformable_group=case['deform_groups'], with_bias=True)
+    flops = 2.0 * N * Ho * Wo * Cout * cin_g * kh * kw
+    es = 4 if dname == 'f32' else 2
+    alg_bytes = es * (x.numel() + off.numel() + msk.numel() + w.numel() + b.numel() + out.numel())
+
+    def step():
+        ext_module.modulated_deform_conv_forward(x, w, b, empty, off, msk, out, empty, **kwargs)
+
+    for _ in range(a.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(a.steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / a.steps
+    ev_ms = e0.elapsed_time(e1) / a.steps
+    ms_per_step = max(wall_ms, ev_ms)
+
+    # dominant kernel: HIP events recorded by the library on the stream it launches on
+    stage = [0.0, 0.0, 0.0, 0.0]
+    for _ in range(a.steps):
+        ms = ext_module.modulated_deform_conv_forward_timed(x, w, b, off, msk, out, **kwargs)
+        stage = [s + m for s, m in zip(stage, ms)]
+    stage = [s / a.steps for s in stage]
+    main_ms = stage[2]
+    log(f'{a.workload} {dname}: step {ms_per_step:.4f} ms (events {ev_ms:.4f}, wall {wall_ms:.4f}); '
+        f'stages relayout {stage[0]:.4f} pack {stage[1]:.4f} main {stage[2]:.4f} ms')
+
+    value = flops / (ms_per_step * 1e-3) / 1e12
+    achieved = flops / (main_ms * 1e-3) / 1e12
+    peak = PEAK_TFLOPS[dname]
+    rec = {
+        'metric': 'DCNv2 fwd TFLOP/s + ms/layer (N=16,C=256,100x152 bf16); % MFMA peak',
+        'value': round(value, 2),
+        'unit': 'TFLOP/s',
+        'n_gpus': 1,
+        'steps': a.steps,
+        'warmup': a.warmup,
+        'ms_per_step': round(ms_per_step, 4),
+        'higher_is_better': True,
+        'scaling': 'weak',
+        'vs_baseline': None,
+        'dtype': dname,
+        'data': 'synthetic',
+        'config': {
+            'workload': (f'{a.workload}: ModulatedDeformConv2d fwd N={N} Cin={Cin} Cout={Cout} '
+                         f'{H}x{W} k{kh}x{kw} s{sh} p{ph} d{dh} groups={case["groups"]} '
+                         f'deform_groups={case["deform_groups"]}, offsets N(0,{wl["sigma"]}) px'),
+            'entry': 'mmcv_amd._ext.modulated_deform_conv_forward',
+            'flops_per_step': flops,
+            'algorithmic_bytes_per_step': alg_bytes,
+        },
+        'ms_per_layer': round(ms_per_step, 4),
+        'pct_mfma_peak': round(100.0 * value / peak, 2),
+        'stage_ms': {'relayout': round(stage[0], 4), 'weight_pack': round(stage[1], 4),
+                     'main': round(stage[2], 4)},
+        'hbm_GBs_algorithmic': round(alg_bytes / (ms_per_step * 1e-3) / 1e9, 1),
+        'roofline': {
+            'bound': 'mfma',
+            'kernel': f'fused_kernel<{dname}>',
+            'achieved': round(achieved, 2),
+            'peak': peak,
+            'unit': 'TFLOP/s',
+            'frac': round(achieved / peak, 4),
+            'traffic': None,
+        },
+    }
+    if not a.no_cpu:
+        log('timing the CPU baseline ...')
+        rec['cpu_baseline'] = cpu_baseline(case, flops / N)
+    print(json.dumps(rec), flush=True)
+
+
+if __name__ == '__main__':
+    main()
