@@ -68,12 +68,28 @@ inline size_t fused_lds(int dtype, int CT, int taps) {
 bool fused_ok(const mdcn_params *p, const Geom &g) {
   const int KC = slab_channels(p->dtype);
   if (g.cin_g % KC || g.ch_per_dg % KC) return false;
+  // with several deformable groups the gather pipeline must stay inside one
+  // group's table while it fills
+  if (g.DG > 1 && (g.ch_per_dg / KC) * g.taps < kGatherAhead + 1) return false;
   if (fused_lds(p->dtype, pick_ct(g.cout_g), g.taps) > kMaxLds) return false;
   // one padded image must fit the 32-bit offsets
   const uint64_t img = (uint64_t)g.Hp * g.Wp * g.Cin * elem_size(p->dtype);
   if (img > kMaxXtBytes) return false;
-  if ((uint64_t)g.N * g.Ho * g.Wo > 0x7fffffffull * 1ull) return false;
+  if ((uint64_t)g.N * g.Ho * g.Wo > 0x7fffffffull) return false;
   return true;
+}
+
+int num_cus() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
 }
 
 struct Plan {
@@ -104,19 +120,22 @@ int make_plan(const mdcn_params *p, const Geom &g, Plan *pl) {
 }
 
 template <typename E, int CT>
-hipError_t launch_fused_ct(const FusedArgs &fa, size_t lds, hipStream_t st) {
+hipError_t launch_fused_ct(const FusedArgs &fa, size_t dyn_lds, hipStream_t st) {
   auto kern = fused_kernel<E, CT>;
-  static bool attr_set = false;  // idempotent; a race only repeats the call
-  if (!attr_set) {
+  static bool attr_set[64] = {false};  // per device; a race only repeats the call
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+  if (!attr_set[dev]) {
     hipError_t e = hipFuncSetAttribute((const void *)kern,
                                        hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)kMaxLds);
+                                       (int)(kMaxLds - fused_static_lds_bytes(CT)));
     if (e != hipSuccess) return e;
-    attr_set = true;
+    attr_set[dev] = true;
   }
+  // persistent workgroups: one per CU, a multiple of the 8 XCDs
   const int total_wg = fa.n_ptiles * fa.n_ctiles * fa.g.G;
-  const int grid = ((total_wg + 7) / 8) * 8;
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, st, fa);
+  const int per_xcd = std::max(1, std::min((total_wg + 7) / 8, num_cus() / 8));
+  hipLaunchKernelGGL(kern, dim3(per_xcd * 8), dim3(kThreads), dyn_lds, st, fa);
   return hipGetLastError();
 }
 
@@ -129,22 +148,17 @@ hipError_t launch_fused(const FusedArgs &fa, int CT, size_t lds, hipStream_t st)
   }
 }
 
-struct StageEvents {
-  hipEvent_t ev[4];  // start, after relayout, after pack, after main
-  bool on;
-};
-
 template <typename E>
 int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t st,
               float *ms) {
   hipEvent_t ev[2] = {nullptr, nullptr};
-  auto tic = [&]() { if (ms) hipEventRecord(ev[0], st); };
+  auto tic = [&]() { if (ms) (void)hipEventRecord(ev[0], st); };
   auto toc = [&](int slot) {
     if (!ms) return;
-    hipEventRecord(ev[1], st);
-    hipEventSynchronize(ev[1]);
+    (void)hipEventRecord(ev[1], st);
+    (void)hipEventSynchronize(ev[1]);
     float t = 0.f;
-    hipEventElapsedTime(&t, ev[0], ev[1]);
+    (void)hipEventElapsedTime(&t, ev[0], ev[1]);
     ms[slot] += t;
   };
   if (ms) {
@@ -182,7 +196,7 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
       if (hipGetLastError() != hipSuccess) rc = MDCN_ERR_LAUNCH;
       toc(1);
     }
-    const size_t lds = fused_lds_bytes<E>(pl.CT, g.taps);
+    const size_t lds = fused_dyn_lds_bytes<E>(g.taps);
     for (int n0 = 0; n0 < g.N && rc == MDCN_OK; n0 += pl.n_chunk) {
       Geom gc = g;
       gc.N = std::min(pl.n_chunk, g.N - n0);
@@ -191,8 +205,8 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
         const int n_xtiles = (gc.Wp + 63) / 64, n_ctl = (gc.Cin + 63) / 64;
         const long blocks = (long)gc.N * gc.Hp * n_xtiles * n_ctl;
         tic();
-        hipLaunchKernelGGL(relayout_kernel<E>, dim3((unsigned)blocks), dim3(256),
-                           0, st, gc, in, xt, n_xtiles, n_ctl);
+        hipLaunchKernelGGL((relayout_kernel<E, ElemTraits<E>::KC>), dim3((unsigned)blocks),
+                           dim3(256), 0, st, gc, in, xt, n_xtiles, n_ctl);
         if (hipGetLastError() != hipSuccess) rc = MDCN_ERR_LAUNCH;
         toc(0);
       }
@@ -208,8 +222,10 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
       fa.n_ptiles = (int)((fa.total_px + kPT - 1) / kPT);
       fa.n_ctiles = pl.n_ctiles;
       fa.slabs = pl.slabs;
-      fa.pix_bytes = (uint32_t)(g.Cin * es);
-      fa.row_bytes = (uint32_t)((size_t)g.Wp * g.Cin * es);
+      fa.slabs_total = g.Cin / pl.KC;
+      fa.plane_px = g.Hp * g.Wp;
+      fa.row_bytes = (uint32_t)g.Wp * 64u;
+      fa.out_vec_ok = (plane_out % (long)(16 / es) == 0) && (((uintptr_t)fa.out % 16) == 0);
       tic();
       if (launch_fused<E>(fa, pl.CT, lds, st) != hipSuccess) rc = MDCN_ERR_LAUNCH;
       toc(2);
@@ -217,8 +233,8 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
   }
   if (ms) {
     ms[3] = ms[0] + ms[1] + ms[2];
-    hipEventDestroy(ev[0]);
-    hipEventDestroy(ev[1]);
+    (void)hipEventDestroy(ev[0]);
+    (void)hipEventDestroy(ev[1]);
   }
   return rc;
 }

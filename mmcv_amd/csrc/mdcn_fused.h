@@ -1,112 +1,123 @@
-// Fused DCNv2 forward for gfx950: implicit GEMM  out[cout, pixel] = W[cout, k] * S[k, pixel]
+// Fused DCNv2 forward for gfx950: implicit GEMM  out[pixel, cout] = S[pixel, k] * W[k, cout]
 // where S (the "columns" of the reference's two-pass design,
 // mmcv/ops/csrc/pytorch/modulated_deform_conv.cpp:101-124) is produced on the
-// fly -- offset/mask-modulated bilinear samples computed by the wavefronts and
+// fly -- offset/mask-modulated bilinear samples computed by wavefronts and
 // written straight into LDS tiles that feed MFMA -- and never exists in HBM.
 //
-// Work split.  One workgroup (4 wavefronts, 256 lanes) owns a tile of PT = 128
-// consecutive output pixels (flattened n*Ho*Wo + ho*Wo + wo) x CT output
-// channels of one group.  K runs over (channel slab of KC channels) x (tap),
-// slab outer, tap inner, so that the KC-channel slice of the neighbourhood a
-// tile samples stays cache resident across the kh*kw taps.
+// Work split.  A persistent workgroup of 8 wavefronts owns, one after another,
+// tiles of PT = 128 consecutive output pixels (flattened n*Ho*Wo + ho*Wo + wo)
+// x CT output channels of one group.  K runs over (slab of KC channels) x
+// (tap), slab outer, tap inner; the input copy is stored slab-major
+// ([N][Cin/KC][H+2][W+2][KC], 64 bytes per pixel and slab) so that the KC
+// channels of the neighbourhood a tile samples are compact in memory and stay
+// cache resident across the kh*kw taps.
 //
-// Per tile, once per deformable group: a table in LDS holds, for every
-// (pixel, tap), the pixel index of the top-left bilinear corner inside the
-// zero-bordered channels-last input copy and the four mask-scaled bilinear
-// weights.  Positions and weights are computed in fp32.
+// The wavefronts are specialised:
+//   waves 4..7  PRODUCERS.  Once per tile (and deformable group) they fill a
+//     table in LDS with, for every (pixel, tap), the index of the top-left
+//     bilinear corner in the zero-bordered input copy and the four mask-scaled
+//     bilinear weights (positions and weights in fp32).  Per K step, each lane
+//     gathers for two pixels 16 bytes of channels at each of the four corners
+//     (8 x global_load_dwordx4, issued kGatherAhead steps ahead, held in
+//     registers), blends them (v_dot2_f32_{bf16,f16} on the raw 16-bit pairs,
+//     FMA for fp32) and writes 2 x 16 bytes of the sample tile.  They also
+//     start the direct-to-LDS copy of the weight tile kWeightAhead steps ahead.
+//   waves 0..3  CONSUMERS.  2 x 2 over the tile (64 pixels x CT/2 channels
+//     each): read sample and weight fragments from LDS, run MFMA
+//     (32x32x16 bf16/f16, 32x32x2 fp32) into fp32 accumulators; at the end of
+//     the tile add the bias, round once, transpose through LDS and store
+//     16 bytes per lane along W of the NCHW output.
+// One workgroup barrier per K step keeps the two roles in step; the sample
+// tile is double buffered, the weight tiles sit in a ring of kWeightAhead + 2.
 //
-// Per K step: each lane gathers, for one pixel, 32 contiguous bytes of channels
-// at each of the four corners (global_load_dwordx4 x 8), blends them, and
-// writes 32 bytes of the sample tile; the weight tile is copied from its
-// pre-packed form.  Loads for step k+1 are issued before the MFMAs of step k;
-// LDS tiles are double buffered, one barrier per step.
-//
-// MFMA mapping: the "A" operand is the weight tile (rows = output channels),
-// the "B" operand the sample tile (columns = pixels), so that in the 32x32
-// accumulator block lane%32 indexes the pixel and stores of one register are
-// contiguous along W in the NCHW output.
+// LDS tiles have 64-byte rows (one pixel resp. one output channel, KC elements
+// of K); the 16-byte chunk c of row r is stored at chunk c ^ ((r >> 2) & 3), so
+// that both the 16-byte fragment reads (32 consecutive rows, one chunk) and the
+// writes (4 lanes per row) touch every bank once.
 #pragma once
 
 #include "mdcn_common.h"
 
 namespace mdcn {
 
-constexpr int kPT = 128;    // pixels per workgroup tile
-constexpr int kRowB = 80;   // LDS bytes per tile row: 64 data + 16 pad (keeps 16-byte
-                            // reads of 16 consecutive rows on distinct banks)
+constexpr int kPT = 128;           // pixels per tile
+constexpr int kGatherAhead = 3;    // K steps a gather is in flight
+constexpr int kWeightAhead = 2;    // K steps a weight-tile copy is in flight
+constexpr int kWeightSlots = kWeightAhead + 2;
+constexpr int kThreads = 512;
 
 struct FusedArgs {
   Geom g;
-  const void *xt;      // zero-bordered channels-last input copy
+  const void *xt;      // zero-bordered slab-major input copy
   const void *wp;      // packed weights
   const void *offset;
   const void *mask;
   const void *bias;    // may be null
   void *out;
   long total_px;       // N * Ho * Wo
-  int n_ptiles, n_ctiles, slabs;
-  uint32_t pix_bytes;  // Cin * sizeof(E)
-  uint32_t row_bytes;  // Wp * Cin * sizeof(E)
+  int n_ptiles, n_ctiles, slabs;   // slabs = (Cin/G) / KC
+  int slabs_total;     // Cin / KC
+  int plane_px;        // Hp * Wp
+  int out_vec_ok;      // (Ho*Wo) % (16/sizeof(E)) == 0 and the output pointer is 16-byte aligned
+  uint32_t row_bytes;  // Wp * 64
 };
+
+typedef const __attribute__((address_space(1))) void *gptr_t;
+typedef __attribute__((address_space(3))) void *lptr_t;
+
+// s_waitcnt on the vector-memory counter only (gfx9 encoding).
+#define MDCN_WAIT_VMCNT(n) \
+  __builtin_amdgcn_s_waitcnt(((n) & 15) | (7 << 4) | (15 << 8) | (((n) >> 4) << 14))
 
 template <typename E>
 struct ElemTraits;
 
-// ---- 16-bit element types: v_dot2c blend, 32x32x16 MFMA --------------------
+// ---- 16-bit element types ---------------------------------------------------
+// A 32-bit word of gathered data holds two channels and is fed to the blend
+// instruction unchanged (no unpacking); the first corner uses the constant 0 as
+// accumulator, so nothing is cleared beforehand.
 template <typename E>
 struct Half16Traits {
-  static constexpr int KC = 32;    // channels per K step (64 bytes)
-  static constexpr int NACC = 16;  // samples per lane per K step
-  static constexpr int TW = 2;     // table dwords per (pixel, tap) for the weights
+  static constexpr int KC = 32;  // channels per K step (64 bytes)
+  static constexpr int NS = 8;   // samples per lane, pixel and K step (16 bytes)
 
-  static __device__ __forceinline__ uint32_t pack2(float lo, float hi);
-  static __device__ __forceinline__ float dot2(uint32_t d, uint32_t w, float acc);
-
-  static __device__ __forceinline__ void store_weights(const TapSample &s,
-                                                       uint32_t (&tw)[TW]) {
-    tw[0] = ElemTraits<E>::pack2(s.w00, s.w01);
-    tw[1] = ElemTraits<E>::pack2(s.w10, s.w11);
+  static __device__ __forceinline__ void table_weights(const TapSample &s, uint32_t (&tw)[4]) {
+    tw[0] = ElemTraits<E>::pack2(s.w00, 0.0f);
+    tw[1] = ElemTraits<E>::pack2(s.w01, 0.0f);
+    tw[2] = ElemTraits<E>::pack2(s.w10, 0.0f);
+    tw[3] = ElemTraits<E>::pack2(s.w11, 0.0f);
   }
 
-  // acc[2d], acc[2d+1] += w * (low, high) element of dword d.  The dword is fed
-  // to v_dot2c unchanged, paired with (w, 0) resp. (0, w).
-  static __device__ __forceinline__ void blend(float (&acc)[NACC],
-                                               const uint4 (&v)[4][2],
-                                               const uint32_t (&tw)[TW]) {
-    const uint32_t wlo[4] = {tw[0] & 0xffffu, tw[0] >> 16, tw[1] & 0xffffu,
-                             tw[1] >> 16};
-    const uint32_t whi[4] = {tw[0] << 16, tw[0] & 0xffff0000u, tw[1] << 16,
-                             tw[1] & 0xffff0000u};
-#pragma unroll
-    for (int i = 0; i < NACC; ++i) acc[i] = 0.0f;
+  // four consecutive pixels of one output channel, rounded, to the staging row
+  static __device__ __forceinline__ void store4(unsigned char *dst, float a, float b, float c,
+                                                float d) {
+    *(uint2 *)dst = make_uint2(ElemTraits<E>::pack2(a, b), ElemTraits<E>::pack2(c, d));
+  }
+
+  static __device__ __forceinline__ uint4 blend(const uint4 (&v)[4], const uint4 &w) {
+    const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+    float acc[NS];
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
+      const uint32_t d[4] = {v[q].x, v[q].y, v[q].z, v[q].w};
 #pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const uint32_t d[4] = {v[q][h].x, v[q][h].y, v[q][h].z, v[q][h].w};
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int k = (h * 4 + j) * 2;
-          acc[k] = ElemTraits<E>::dot2(d[j], wlo[q], acc[k]);
-          acc[k + 1] = ElemTraits<E>::dot2(d[j], whi[q], acc[k + 1]);
+      for (int j = 0; j < 4; ++j) {
+        if (q == 0) {
+          acc[2 * j] = ElemTraits<E>::dot_lo0(d[j], ww[q]);
+          acc[2 * j + 1] = ElemTraits<E>::dot_hi0(d[j], ww[q]);
+        } else {
+          acc[2 * j] = ElemTraits<E>::dot_lo(d[j], ww[q], acc[2 * j]);
+          acc[2 * j + 1] = ElemTraits<E>::dot_hi(d[j], ww[q], acc[2 * j + 1]);
         }
       }
     }
-  }
-
-  static __device__ __forceinline__ void pack_samples(const float (&acc)[NACC],
-                                                      uint4 (&o)[2]) {
-    o[0] = make_uint4(ElemTraits<E>::pack2(acc[0], acc[1]),
-                      ElemTraits<E>::pack2(acc[2], acc[3]),
-                      ElemTraits<E>::pack2(acc[4], acc[5]),
-                      ElemTraits<E>::pack2(acc[6], acc[7]));
-    o[1] = make_uint4(ElemTraits<E>::pack2(acc[8], acc[9]),
-                      ElemTraits<E>::pack2(acc[10], acc[11]),
-                      ElemTraits<E>::pack2(acc[12], acc[13]),
-                      ElemTraits<E>::pack2(acc[14], acc[15]));
+    return make_uint4(ElemTraits<E>::pack2(acc[0], acc[1]), ElemTraits<E>::pack2(acc[2], acc[3]),
+                      ElemTraits<E>::pack2(acc[4], acc[5]), ElemTraits<E>::pack2(acc[6], acc[7]));
   }
 };
 
+// bf16: v_dot2_f32_bf16 on the raw pair.  The table keeps the weight word
+// (w, 0); the word for the high channel, (0, w), is that shifted left by 16.
 template <>
 struct ElemTraits<bf16_t> : Half16Traits<bf16_t> {
   static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
@@ -115,20 +126,30 @@ struct ElemTraits<bf16_t> : Half16Traits<bf16_t> {
     p.y = (bf16_t)hi;
     return __builtin_bit_cast(uint32_t, p);
   }
-  static __device__ __forceinline__ float dot2(uint32_t d, uint32_t w, float acc) {
+  // (builtins, not inline assembly: the compiler must see the DOT instruction
+  // to insert the wait states its result needs before another VALU reads it)
+  static __device__ __forceinline__ float dot_lo(uint32_t d, uint32_t w, float c) {
     return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, d),
-                                           __builtin_bit_cast(bf16x2, w), acc,
-                                           false);
+                                           __builtin_bit_cast(bf16x2, w), c, false);
+  }
+  static __device__ __forceinline__ float dot_hi(uint32_t d, uint32_t w, float c) {
+    return dot_lo(d, w << 16, c);
+  }
+  static __device__ __forceinline__ float dot_lo0(uint32_t d, uint32_t w) {
+    return dot_lo(d, w, 0.0f);
+  }
+  static __device__ __forceinline__ float dot_hi0(uint32_t d, uint32_t w) {
+    return dot_lo(d, w << 16, 0.0f);
   }
   // 16 bytes = 8 consecutive K elements of one row per lane.
-  static __device__ __forceinline__ void mma(f32x16 &c, const uint4 &a,
-                                             const uint4 &b) {
+  static __device__ __forceinline__ void mma(f32x16 &c, const uint4 &a, const uint4 &b) {
     c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
-                                                __builtin_bit_cast(bf16x8, b),
-                                                c, 0, 0, 0);
+                                                __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
   }
 };
 
+// fp16: mixed-precision FMA (v_fma_mix_f32): one source is read as the low or
+// high fp16 half of the gathered word, the bilinear weight stays fp32.
 template <>
 struct ElemTraits<f16_t> : Half16Traits<f16_t> {
   static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
@@ -137,299 +158,396 @@ struct ElemTraits<f16_t> : Half16Traits<f16_t> {
     p.y = (f16_t)hi;
     return __builtin_bit_cast(uint32_t, p);
   }
-  static __device__ __forceinline__ float dot2(uint32_t d, uint32_t w, float acc) {
-    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, d),
-                                  __builtin_bit_cast(f16x2, w), acc, false);
+  static __device__ __forceinline__ void table_weights(const TapSample &s, uint32_t (&tw)[4]) {
+    tw[0] = __float_as_uint(s.w00);
+    tw[1] = __float_as_uint(s.w01);
+    tw[2] = __float_as_uint(s.w10);
+    tw[3] = __float_as_uint(s.w11);
   }
-  static __device__ __forceinline__ void mma(f32x16 &c, const uint4 &a,
-                                             const uint4 &b) {
+  // fma(fpext(half), w, c): the compiler selects v_fma_mix_f32 with op_sel
+  static __device__ __forceinline__ float dot_lo(uint32_t d, uint32_t w, float c) {
+    return __builtin_fmaf((float)__builtin_bit_cast(f16x2, d).x, __uint_as_float(w), c);
+  }
+  static __device__ __forceinline__ float dot_hi(uint32_t d, uint32_t w, float c) {
+    return __builtin_fmaf((float)__builtin_bit_cast(f16x2, d).y, __uint_as_float(w), c);
+  }
+  static __device__ __forceinline__ float dot_lo0(uint32_t d, uint32_t w) {
+    return (float)__builtin_bit_cast(f16x2, d).x * __uint_as_float(w);
+  }
+  static __device__ __forceinline__ float dot_hi0(uint32_t d, uint32_t w) {
+    return (float)__builtin_bit_cast(f16x2, d).y * __uint_as_float(w);
+  }
+  static __device__ __forceinline__ void mma(f32x16 &c, const uint4 &a, const uint4 &b) {
     c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
-                                               __builtin_bit_cast(f16x8, b), c,
-                                               0, 0, 0);
+                                               __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
   }
 };
 
-// ---- fp32: scalar FMA blend, 32x32x2 fp32 MFMA ------------------------------
+// ---- fp32 --------------------------------------------------------------------
 template <>
 struct ElemTraits<float> {
   static constexpr int KC = 16;
-  static constexpr int NACC = 8;
-  static constexpr int TW = 4;
+  static constexpr int NS = 4;
 
-  static __device__ __forceinline__ void store_weights(const TapSample &s,
-                                                       uint32_t (&tw)[TW]) {
+  static __device__ __forceinline__ void table_weights(const TapSample &s, uint32_t (&tw)[4]) {
     tw[0] = __float_as_uint(s.w00);
     tw[1] = __float_as_uint(s.w01);
     tw[2] = __float_as_uint(s.w10);
     tw[3] = __float_as_uint(s.w11);
   }
 
-  static __device__ __forceinline__ void blend(float (&acc)[NACC],
-                                               const uint4 (&v)[4][2],
-                                               const uint32_t (&tw)[TW]) {
-#pragma unroll
-    for (int i = 0; i < NACC; ++i) acc[i] = 0.0f;
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const float w = __uint_as_float(tw[q]);
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        acc[h * 4 + 0] += w * __uint_as_float(v[q][h].x);
-        acc[h * 4 + 1] += w * __uint_as_float(v[q][h].y);
-        acc[h * 4 + 2] += w * __uint_as_float(v[q][h].z);
-        acc[h * 4 + 3] += w * __uint_as_float(v[q][h].w);
-      }
-    }
+  static __device__ __forceinline__ void store4(unsigned char *dst, float a, float b, float c,
+                                                float d) {
+    *(uint4 *)dst = make_uint4(__float_as_uint(a), __float_as_uint(b), __float_as_uint(c),
+                               __float_as_uint(d));
   }
 
-  static __device__ __forceinline__ void pack_samples(const float (&acc)[NACC],
-                                                      uint4 (&o)[2]) {
-    o[0] = make_uint4(__float_as_uint(acc[0]), __float_as_uint(acc[1]),
-                      __float_as_uint(acc[2]), __float_as_uint(acc[3]));
-    o[1] = make_uint4(__float_as_uint(acc[4]), __float_as_uint(acc[5]),
-                      __float_as_uint(acc[6]), __float_as_uint(acc[7]));
+  static __device__ __forceinline__ uint4 blend(const uint4 (&v)[4], const uint4 &w) {
+    const float ww[4] = {__uint_as_float(w.x), __uint_as_float(w.y), __uint_as_float(w.z),
+                         __uint_as_float(w.w)};
+    float acc[NS];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const float d[4] = {__uint_as_float(v[q].x), __uint_as_float(v[q].y),
+                          __uint_as_float(v[q].z), __uint_as_float(v[q].w)};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[j] = (q == 0) ? ww[q] * d[j] : acc[j] + ww[q] * d[j];
+    }
+    return make_uint4(__float_as_uint(acc[0]), __float_as_uint(acc[1]), __float_as_uint(acc[2]),
+                      __float_as_uint(acc[3]));
   }
 
   // 16 bytes = 4 consecutive K elements of one row per lane; element j of both
   // operands goes to the j-th 32x32x2 MFMA.
-  static __device__ __forceinline__ void mma(f32x16 &c, const uint4 &a,
-                                             const uint4 &b) {
-    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.x),
-                                             __uint_as_float(b.x), c, 0, 0, 0);
-    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.y),
-                                             __uint_as_float(b.y), c, 0, 0, 0);
-    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.z),
-                                             __uint_as_float(b.z), c, 0, 0, 0);
-    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.w),
-                                             __uint_as_float(b.w), c, 0, 0, 0);
+  static __device__ __forceinline__ void mma(f32x16 &c, const uint4 &a, const uint4 &b) {
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.x), __uint_as_float(b.x), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.y), __uint_as_float(b.y), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.z), __uint_as_float(b.z), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.w), __uint_as_float(b.w), c, 0, 0, 0);
   }
 };
 
-// LDS bytes of one workgroup of fused_kernel<E, CT>.
+// Bytes per row of the epilogue staging area: 64 pixels + 16 bytes of padding.
+template <typename E>
+constexpr int stage_row_bytes() {
+  return 64 * (int)sizeof(E) + 16;
+}
+
+// Dynamic LDS of fused_kernel: the (pixel, tap) table, reused as the epilogue
+// staging area (4 consumer waves x 32 output channels x one padded row).
+template <typename E>
+constexpr size_t fused_dyn_lds_bytes(int taps) {
+  const size_t table = (size_t)kPT * taps * 20;
+  const size_t stage = (size_t)4 * 32 * stage_row_bytes<E>();
+  return table > stage ? table : stage;
+}
+
+// Static LDS of one workgroup: two sample tiles and the ring of weight tiles.
+constexpr size_t fused_static_lds_bytes(int CT) {
+  return (size_t)2 * kPT * 64 + (size_t)kWeightSlots * CT * 64;
+}
+
+// Static + dynamic LDS of one workgroup.
 template <typename E>
 constexpr size_t fused_lds_bytes(int CT, int taps) {
-  return (size_t)2 * kPT * kRowB + (size_t)2 * CT * kRowB +
-         (size_t)kPT * taps * 4 * (1 + ElemTraits<E>::TW);
+  return fused_static_lds_bytes(CT) + fused_dyn_lds_bytes<E>(taps);
 }
 
 template <typename E, int CT>
-__global__ __launch_bounds__(256, 2) void fused_kernel(FusedArgs a) {
+__global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
   using TR = ElemTraits<E>;
   constexpr int PT = kPT;
   constexpr int KC = TR::KC;
-  constexpr int TW = TR::TW;
-  constexpr int MB = CT / 64;  // 32-row accumulator blocks per wave along Cout
-  constexpr int NB = 2;        // ... along pixels (64 pixels per wave)
-  constexpr int WREG = CT / 64;  // 16-byte weight-tile pieces per lane
+  constexpr int ES = (int)sizeof(E);
+  constexpr int MB = CT / 64;        // 32-channel accumulator blocks per consumer wave
+  constexpr int NB = 2;              // 32-pixel blocks per consumer wave
+  constexpr int WDMA = CT / 64;      // 1 KiB direct-to-LDS copies per producer wave and K step
+  constexpr int OPS = 8 + WDMA;      // vector-memory ops a producer lane issues per K step
+
+  __shared__ uint4 Xs[2][PT * 4];                // sample tiles
+  __shared__ uint4 Ws[kWeightSlots][CT * 4];     // weight tiles
+  extern __shared__ __align__(16) unsigned char dyn[];
 
   const Geom &g = a.g;
   const int taps = g.taps;
-
-  // XCD-aware tile order: consecutive workgroup ids go to different XCDs, so
-  // give each XCD one contiguous run of tiles (shared halo rows stay in its L2).
-  const int total_wg = a.n_ptiles * a.n_ctiles * g.G;
-  const int chunk = (total_wg + 7) >> 3;
-  int L = (int)(blockIdx.x & 7) * chunk + (int)(blockIdx.x >> 3);
-  if (L >= total_wg) return;
-  const int ctile = L % a.n_ctiles;
-  L /= a.n_ctiles;
-  const int grp = L % g.G;
-  const int ptile = L / g.G;
-
-  extern __shared__ __align__(16) unsigned char smem[];
-  unsigned char *Xs = smem;                        // [2][PT][kRowB]
-  unsigned char *Ws = Xs + 2 * PT * kRowB;         // [2][CT][kRowB]
-  int32_t *tpix = (int32_t *)(Ws + 2 * CT * kRowB);  // [taps][PT]
-  uint32_t *tws = (uint32_t *)(tpix + PT * taps);    // [TW][taps][PT]
+  const int nk = a.slabs * taps;
+  const long plane_out = (long)g.Ho * g.Wo;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int wave_c = wave >> 1;  // which half of the Cout tile
-  const int wave_p = wave & 1;   // which half of the pixel tile
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const bool producer = wave >= 4;
 
-  const long plane_out = (long)g.Ho * g.Wo;
-  const long p0 = (long)ptile * PT;
+  int32_t *tpix = (int32_t *)dyn;                    // [taps][PT]
+  uint4 *tws = (uint4 *)(dyn + (size_t)PT * taps * 4);  // [taps][PT]
 
-  // ---- (pixel, tap) table for one deformable group ------------------------
-  // Entry e = tap*PT + pixel; this lane always serves pixel tid%128.
-  const int tb_pl = tid & (PT - 1);
-  const long tb_p = p0 + tb_pl;
-  const bool tb_valid = tb_p < a.total_px;
-  int tb_n = 0, tb_ho = 0, tb_wo = 0;
-  long tb_rem = 0;
-  if (tb_valid) {
-    tb_n = (int)(tb_p / plane_out);
-    tb_rem = tb_p - (long)tb_n * plane_out;
-    tb_ho = (int)(tb_rem / g.Wo);
-    tb_wo = (int)(tb_rem - (long)tb_ho * g.Wo);
-  }
-  auto build_table = [&](int dgi) {
-    const E *off = (const E *)a.offset +
-                   ((long)tb_n * g.DG + dgi) * 2 * taps * plane_out + tb_rem;
-    const E *msk = (const E *)a.mask +
-                   ((long)tb_n * g.DG + dgi) * taps * plane_out + tb_rem;
-    for (int tap = tid >> 7; tap < taps; tap += 2) {
-      int32_t pix = 0;
-      uint32_t tw[TW];
-#pragma unroll
-      for (int i = 0; i < TW; ++i) tw[i] = 0u;
+  // XCD-aware persistent schedule: consecutive workgroup ids sit on different
+  // XCDs; each XCD walks one contiguous run of tiles so that the halo rows
+  // neighbouring tiles share stay in its L2.
+  const int total_tiles = a.n_ptiles * a.n_ctiles * g.G;
+  const int xcd = (int)(blockIdx.x & 7);
+  const int wg_in_xcd = (int)(blockIdx.x >> 3);
+  const int wgs_per_xcd = (int)(gridDim.x >> 3);
+  const int chunk = (total_tiles + 7) >> 3;
+  const int tile_end = min((xcd + 1) * chunk, total_tiles);
+
+  for (int tile = xcd * chunk + wg_in_xcd; tile < tile_end; tile += wgs_per_xcd) {
+    int L = tile;
+    const int ctile = L % a.n_ctiles;
+    L /= a.n_ctiles;
+    const int grp = L % g.G;
+    const int ptile = L / g.G;
+    const long p0 = (long)ptile * PT;
+    const int ch0 = grp * g.cin_g;  // first input channel of the group
+
+    if (producer) {
+      // =================== PRODUCER ===================
+      const int ptid = tid - 256;
+      const int q = ptid & 3;          // 16-byte chunk of the 64-byte slab row
+      const int pxl = ptid >> 2;       // pixels pxl and pxl + 64 of the tile
+      const unsigned char *xt = (const unsigned char *)a.xt;
+      const int slab0 = ch0 / KC;
+
+      // -- (pixel, tap) table of one deformable group; lane serves pixel ptid%128
+      const int tb_pl = ptid & (PT - 1);
+      const long tb_p = p0 + tb_pl;
+      const bool tb_valid = tb_p < a.total_px;
+      int tb_n = 0, tb_ho = 0, tb_wo = 0;
+      long tb_rem = 0;
       if (tb_valid) {
-        const float dy = to_f32(off[(long)(2 * tap) * plane_out]);
-        const float dx = to_f32(off[(long)(2 * tap + 1) * plane_out]);
-        const float m = to_f32(msk[(long)tap * plane_out]);
-        const int i = tap / g.kw, j = tap - i * g.kw;
-        const TapSample s =
-            make_tap_sample(tb_ho * g.sh - g.ph + i * g.dh,
-                            tb_wo * g.sw - g.pw + j * g.dw, dy, dx, m, g.H, g.W);
-        // +1: coordinates in the zero-bordered copy.  y0, x0 are in [-1, H-1] x
-        // [-1, W-1] when inside, 0 otherwise (weights are 0 then).
-        pix = (tb_n * g.Hp + (s.y0 + 1)) * g.Wp + (s.x0 + 1);
-        TR::store_weights(s, tw);
+        tb_n = (int)(tb_p / plane_out);
+        tb_rem = tb_p - (long)tb_n * plane_out;
+        tb_ho = (int)(tb_rem / g.Wo);
+        tb_wo = (int)(tb_rem - (long)tb_ho * g.Wo);
       }
-      const int e = tap * PT + tb_pl;
-      tpix[e] = pix;
-#pragma unroll
-      for (int i = 0; i < TW; ++i) tws[i * (PT * taps) + e] = tw[i];
-    }
-  };
+      auto build_table = [&](int dgi) {
+        const E *off = (const E *)a.offset + ((long)tb_n * g.DG + dgi) * 2 * taps * plane_out + tb_rem;
+        const E *msk = (const E *)a.mask + ((long)tb_n * g.DG + dgi) * taps * plane_out + tb_rem;
+        for (int tap = ptid >> 7; tap < taps; tap += 2) {
+          int32_t pix = 0;
+          uint32_t tw[4] = {0u, 0u, 0u, 0u};
+          if (tb_valid) {
+            const float dy = to_f32(off[(long)(2 * tap) * plane_out]);
+            const float dx = to_f32(off[(long)(2 * tap + 1) * plane_out]);
+            const float m = to_f32(msk[(long)tap * plane_out]);
+            const int i = tap / g.kw, j = tap - i * g.kw;
+            const TapSample s = make_tap_sample(tb_ho * g.sh - g.ph + i * g.dh,
+                                                tb_wo * g.sw - g.pw + j * g.dw, dy, dx, m, g.H, g.W);
+            // +1: coordinates in the zero-bordered copy (y0, x0 >= -1 when inside,
+            // 0 with zero weights otherwise); slab 0 of image tb_n.
+            pix = tb_n * a.slabs_total * a.plane_px + (s.y0 + 1) * g.Wp + (s.x0 + 1);
+            TR::table_weights(s, tw);
+          }
+          tpix[tap * PT + tb_pl] = pix;
+          tws[tap * PT + tb_pl] = make_uint4(tw[0], tw[1], tw[2], tw[3]);
+        }
+      };
 
-  // ---- producer state: this lane gathers pixel g_px, 32 bytes per corner --
-  const int g_px = tid >> 1;
-  const uint32_t g_half = (uint32_t)(tid & 1) * 32u;
-  const unsigned char *xt = (const unsigned char *)a.xt;
-  const uint32_t grp_ch_bytes = (uint32_t)(grp * g.cin_g) * (uint32_t)sizeof(E);
+      // -- gather state: kGatherAhead register sets, set m % kGatherAhead holds step m
+      uint4 gv[kGatherAhead][2][4];
+      uint4 gw[kGatherAhead][2];
 
-  uint4 gv[4][2];       // gathered corner data of the step in flight
-  uint32_t gtw[TW];     // its blend weights
-  uint4 wreg[WREG];     // its weight-tile pieces
+      auto issue_gather = [&](int ks, uint4 (&v)[2][4], uint4 (&w)[2]) {
+        const int kk = min(ks, nk - 1);  // past the end: repeat the last step (never consumed)
+        const int slab = kk / taps;
+        const int tap = kk - slab * taps;
+        const int sbase = (slab0 + slab) * a.plane_px;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const int e = tap * PT + pxl + 64 * h;
+          const uint32_t o = ((uint32_t)(tpix[e] + sbase) << 6) + (uint32_t)q * 16u;
+          w[h] = tws[e];
+          const unsigned char *top = xt + o;
+          const unsigned char *bot = top + a.row_bytes;
+          v[h][0] = *(const uint4 *)(top);
+          v[h][1] = *(const uint4 *)(top + 64);
+          v[h][2] = *(const uint4 *)(bot);
+          v[h][3] = *(const uint4 *)(bot + 64);
+        }
+      };
 
-  const int nk = a.slabs * taps;
-  const unsigned char *wp_tile =
-      (const unsigned char *)a.wp +
-      ((size_t)(grp * a.n_ctiles + ctile) * nk) * (size_t)(CT * 64);
+      // weight tile of step ks -> ring slot ks % kWeightSlots, straight into LDS:
+      // lane i of copy c writes chunk c*64+i of the slot and reads the source
+      // chunk that the swizzle assigns to it.
+      const unsigned char *wp_tile = (const unsigned char *)a.wp +
+                                     ((size_t)(grp * a.n_ctiles + ctile) * nk) * (size_t)(CT * 64);
+      auto issue_weights = [&](int ks) {
+        const int kk = min(ks, nk - 1);
+        const unsigned char *src = wp_tile + (size_t)kk * (CT * 64);
+        const int slot = ks % kWeightSlots;
+#pragma unroll
+        for (int c = 0; c < WDMA; ++c) {
+          const int blk = (wave - 4) * WDMA + c;   // 1 KiB block of the tile
+          const int d = blk * 64 + lane;           // destination chunk
+          const int row = d >> 2;
+          const int sc = (d & 3) ^ ((row >> 2) & 3);
+          __builtin_amdgcn_global_load_lds((gptr_t)(src + row * 64 + sc * 16),
+                                           (lptr_t)(&Ws[slot][blk * 64]), 16, 0, 0);
+        }
+      };
 
-  auto issue_loads = [&](int ks) {
-    const int slab = ks / taps;
-    const int tap = ks - slab * taps;
-    const int e = tap * PT + g_px;
-    const uint32_t pix = (uint32_t)tpix[e];
+      auto commit = [&](int buf, const uint4 (&v)[2][4], const uint4 (&w)[2]) {
 #pragma unroll
-    for (int i = 0; i < TW; ++i) gtw[i] = tws[i * (PT * taps) + e];
-    const uint32_t o = pix * a.pix_bytes + grp_ch_bytes +
-                       (uint32_t)(slab * KC) * (uint32_t)sizeof(E) + g_half;
-    const uint32_t co[4] = {o, o + a.pix_bytes, o + a.row_bytes,
-                            o + a.row_bytes + a.pix_bytes};
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const uint4 *p = (const uint4 *)(xt + co[q]);
-      gv[q][0] = p[0];
-      gv[q][1] = p[1];
-    }
-    const uint4 *wt = (const uint4 *)(wp_tile + (size_t)ks * (CT * 64));
-#pragma unroll
-    for (int i = 0; i < WREG; ++i) wreg[i] = wt[tid + 256 * i];
-  };
+        for (int h = 0; h < 2; ++h) {
+          const int row = pxl + 64 * h;
+          Xs[buf][row * 4 + (q ^ ((row >> 2) & 3))] = TR::blend(v[h], w[h]);
+        }
+      };
 
-  auto commit_tiles = [&](int buf) {
-    float acc[TR::NACC];
-    TR::blend(acc, gv, gtw);
-    uint4 o[2];
-    TR::pack_samples(acc, o);
-    uint4 *xs = (uint4 *)(Xs + (buf * PT + g_px) * kRowB + g_half);
-    xs[0] = o[0];
-    xs[1] = o[1];
-#pragma unroll
-    for (int i = 0; i < WREG; ++i) {
-      const int q = tid + 256 * i;
-      *(uint4 *)(Ws + (buf * CT + (q >> 2)) * kRowB + (q & 3) * 16) = wreg[i];
-    }
-  };
+      // Deformable group of the (clamped) K step ks; the table holds one group.
+      auto dg_of = [&](int ks) { return (ch0 + (min(ks, nk - 1) / taps) * KC) / g.ch_per_dg; };
+      build_table(dg_of(0));
+      __syncthreads();  // B0: table visible
 
-  f32x16 acc[MB][NB];
+      // Issue order is that of the steady state extended to "virtual" steps
+      // v = -1-kGatherAhead .. -1: step v issues gather(v+1+kGatherAhead) and then
+      // weights(v+1+kWeightAhead).  Every step from -1-kWeightAhead on issues
+      // exactly OPS vector-memory operations, so "at most kWeightAhead*OPS
+      // outstanding" always means the weight tile of the next step has landed.
 #pragma unroll
-  for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[mb][nb][r] = 0.0f;
-
-  const int frag_row = lane & 31;
-  const int frag_off = (lane >> 5) * 16;
-
-  auto mma_phase = [&](int buf) {
-#pragma unroll
-    for (int ksub = 0; ksub < 2; ++ksub) {
-      uint4 wf[MB], xf[NB];
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb)
-        wf[mb] = *(const uint4 *)(Ws +
-                                  (buf * CT + wave_c * (CT / 2) + mb * 32 + frag_row) * kRowB +
-                                  ksub * 32 + frag_off);
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-        xf[nb] = *(const uint4 *)(Xs +
-                                  (buf * PT + wave_p * 64 + nb * 32 + frag_row) * kRowB +
-                                  ksub * 32 + frag_off);
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) TR::mma(acc[mb][nb], wf[mb], xf[nb]);
-    }
-  };
-
-  // ---- main loop ----------------------------------------------------------
-  const int ch0 = grp * g.cin_g;  // first input channel of this group
-  int cur_dg = ch0 / g.ch_per_dg;
-  build_table(cur_dg);
-  __syncthreads();
-  issue_loads(0);
-  commit_tiles(0);
-  __syncthreads();
-
-  for (int ks = 0; ks < nk; ++ks) {
-    const int buf = ks & 1;
-    const bool has_next = (ks + 1) < nk;
-    if (has_next) {
-      const int nslab = (ks + 1) / taps;
-      const int ndg = (ch0 + nslab * KC) / g.ch_per_dg;
-      if (ndg != cur_dg) {  // uniform over the workgroup
-        // Every lane read the table for step ks before the barrier that ended
-        // the previous iteration, so it can be overwritten now.
-        cur_dg = ndg;
-        build_table(cur_dg);
-        __syncthreads();
+      for (int v = -1 - kGatherAhead; v < -1; ++v) {
+        issue_gather(v + 1 + kGatherAhead, gv[v + 1 + kGatherAhead], gw[v + 1 + kGatherAhead]);
+        if (v + 1 + kWeightAhead >= 0) issue_weights(v + 1 + kWeightAhead);
       }
-      issue_loads(ks + 1);
-    }
-    mma_phase(buf);
-    if (has_next) commit_tiles(buf ^ 1);
-    __syncthreads();
-  }
+      commit(0, gv[0], gw[0]);
+      issue_gather(kGatherAhead, gv[0], gw[0]);
+      issue_weights(kWeightAhead);
+      MDCN_WAIT_VMCNT(kWeightAhead * OPS);
+      __syncthreads();  // B1: X[0], W[0] visible
 
-  // ---- epilogue: bias, round once, NCHW store -----------------------------
-  // Accumulator block: register r of lane l holds
-  //   row (cout) = (r/4)*8 + (l/32)*4 + r%4,  column (pixel) = l%32.
-  E *out = (E *)a.out;
+      for (int ks0 = 0; ks0 < nk; ks0 += kGatherAhead) {
 #pragma unroll
-  for (int nb = 0; nb < NB; ++nb) {
-    const long p = p0 + wave_p * 64 + nb * 32 + (lane & 31);
-    if (p >= a.total_px) continue;
-    const int n = (int)(p / plane_out);
-    const long rem = p - (long)n * plane_out;
-    E *obase = out + ((long)n * g.Cout + (long)grp * g.cout_g) * plane_out + rem;
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int col = ctile * CT + wave_c * (CT / 2) + mb * 32 + (r >> 2) * 8 +
-                        (lane >> 5) * 4 + (r & 3);
-        if (col < g.cout_g) {
-          float v = acc[mb][nb][r];
-          if (a.bias) v += to_f32(((const E *)a.bias)[grp * g.cout_g + col]);
-          obase[(long)col * plane_out] = from_f32<E>(v);
+        for (int j = 0; j < kGatherAhead; ++j) {
+          const int ks = ks0 + j;
+          if (ks < nk) {
+            const int set = (j + 1) % kGatherAhead;  // holds step ks + 1
+            commit((ks + 1) & 1, gv[set], gw[set]);
+            if (dg_of(ks + 1 + kGatherAhead) != dg_of(ks + kGatherAhead)) {
+              // Next step to issue samples with another deformable group's offsets.
+              // Every producer issued step ks + kGatherAhead before the barrier that
+              // ended the previous step, and took its weights into registers.
+              build_table(dg_of(ks + 1 + kGatherAhead));
+              __syncthreads();  // R: new table visible (consumers join, see below)
+            }
+            issue_gather(ks + 1 + kGatherAhead, gv[set], gw[set]);
+            issue_weights(ks + 1 + kWeightAhead);
+            MDCN_WAIT_VMCNT(kWeightAhead * OPS);
+            __syncthreads();  // end of step ks: X[ks+1], W[ks+1] visible
+          }
         }
       }
+      MDCN_WAIT_VMCNT(0);  // the copies issued past the end must land before LDS is reused
+      __syncthreads();     // E0: consumers own the dynamic LDS (staging) from here
+      __syncthreads();     // E1: epilogue done, the table may be rebuilt
+    } else {
+      // =================== CONSUMER ===================
+      const int wave_p = wave & 1;   // which 64 pixels
+      const int wave_c = wave >> 1;  // which CT/2 output channels
+      f32x16 acc[NB][MB];
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[nb][mb][r] = 0.0f;
+
+      const int frow = lane & 31;
+      const int fhalf = lane >> 5;
+      auto dg_of = [&](int ks) { return (ch0 + (min(ks, nk - 1) / taps) * KC) / g.ch_per_dg; };
+      __syncthreads();  // B0
+      __syncthreads();  // B1
+
+      for (int ks = 0; ks < nk; ++ks) {
+        const uint4 *X = Xs[ks & 1];
+        const uint4 *W = Ws[ks % kWeightSlots];
+#pragma unroll
+        for (int ksub = 0; ksub < 2; ++ksub) {
+          const int ch = ksub * 2 + fhalf;
+          uint4 xf[NB], wf[MB];
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb) {
+            const int row = wave_p * 64 + nb * 32 + frow;
+            xf[nb] = X[row * 4 + (ch ^ ((row >> 2) & 3))];
+          }
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb) {
+            const int row = wave_c * (CT / 2) + mb * 32 + frow;
+            wf[mb] = W[row * 4 + (ch ^ ((row >> 2) & 3))];
+          }
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) TR::mma(acc[nb][mb], xf[nb], wf[mb]);
+        }
+        if (dg_of(ks + 1 + kGatherAhead) != dg_of(ks + kGatherAhead))
+          __syncthreads();  // R: producers publish the next deformable group's table
+        __syncthreads();  // end of step ks
+      }
+      __syncthreads();  // E0
+
+      // ---- epilogue: bias, round once, transpose through LDS, NCHW store ----
+      // Accumulator block (A = samples, B = weights): register r of lane l holds
+      //   pixel = (r/4)*8 + (l/32)*4 + r%4,  channel = l%32.
+      constexpr int RB = stage_row_bytes<E>();
+      constexpr int CHUNK_PX = 16 / ES;           // pixels per 16-byte chunk
+      constexpr int CHUNKS = 64 / CHUNK_PX;       // chunks per staged row
+      unsigned char *stage = dyn + (size_t)wave * 32 * RB;
+      E *out = (E *)a.out;
+      const long pw0 = p0 + wave_p * 64;          // first pixel of this wave
+      const bool vec_ok = a.out_vec_ok != 0;  // 16-byte chunks never straddle images and are aligned
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        const int col0 = ctile * CT + wave_c * (CT / 2) + mb * 32;  // channel within the group
+        const int mycol = col0 + frow;
+        float bv = 0.0f;
+        if (a.bias && mycol < g.cout_g) bv = to_f32(((const E *)a.bias)[grp * g.cout_g + mycol]);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+          for (int r4 = 0; r4 < 4; ++r4) {
+            const int px = nb * 32 + r4 * 8 + fhalf * 4;
+            TR::store4(stage + frow * RB + px * ES, acc[nb][mb][r4 * 4 + 0] + bv,
+                       acc[nb][mb][r4 * 4 + 1] + bv, acc[nb][mb][r4 * 4 + 2] + bv,
+                       acc[nb][mb][r4 * 4 + 3] + bv);
+          }
+        }
+        // same wave wrote and reads: LDS operations of a wave complete in order
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int it = 0; it < 32 * CHUNKS / 64; ++it) {
+          const int idx = it * 64 + lane;
+          const int row = idx / CHUNKS;        // channel of the block
+          const int chunk = idx % CHUNKS;
+          const int col = col0 + row;
+          const long p = pw0 + chunk * CHUNK_PX;
+          if (col < g.cout_g && p < a.total_px) {
+            const uint4 val = *(const uint4 *)(stage + row * RB + chunk * 16);
+            const int n = (int)(p / plane_out);
+            const long rem = p - (long)n * plane_out;
+            E *o = out + ((long)n * g.Cout + (long)grp * g.cout_g + col) * plane_out + rem;
+            if (vec_ok && p + CHUNK_PX <= a.total_px) {
+              *(uint4 *)o = val;   // chunk lies in one image and is 16-byte aligned
+            } else {
+              const E *ve = (const E *)&val;
+#pragma unroll
+              for (int i = 0; i < CHUNK_PX; ++i) {
+                const long pi = p + i;
+                if (pi < a.total_px) {
+                  const int ni = (int)(pi / plane_out);
+                  const long ri = pi - (long)ni * plane_out;
+                  out[((long)ni * g.Cout + (long)grp * g.cout_g + col) * plane_out + ri] = ve[i];
+                }
+              }
+            }
+          }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      }
+      __syncthreads();  // E1
     }
   }
 }

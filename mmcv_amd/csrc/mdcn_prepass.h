@@ -5,15 +5,16 @@
 
 namespace mdcn {
 
-// NCHW input -> zero-bordered channels-last copy xt[N][H+2][W+2][Cin].
-// The one-pixel zero border makes every bilinear corner of an in-range
-// position a plain load: a corner outside the image reads a stored zero,
-// which is exactly the per-corner rule of the reference sampler
-// (mmcv/ops/csrc/pytorch/cpu/modulated_deform_conv.cpp:17-27).
+// NCHW input -> zero-bordered slab-major copy xt[N][Cin/KC][H+2][W+2][KC]
+// (KC channels = 64 bytes per pixel and slab).  The one-pixel zero border makes
+// every bilinear corner of an in-range position a plain load: a corner outside
+// the image reads a stored zero, which is exactly the per-corner rule of the
+// reference sampler (mmcv/ops/csrc/pytorch/cpu/modulated_deform_conv.cpp:17-27).
 //
 // One block moves a 64-channel x 64-column tile of one padded row through LDS:
-// reads run along W (contiguous in NCHW), writes along C (contiguous in xt).
-template <typename E>
+// reads run along W (contiguous in NCHW), writes along the KC channels of a
+// pixel and on to the next pixel (contiguous in xt).
+template <typename E, int KC>
 __global__ __launch_bounds__(256) void relayout_kernel(
     Geom g, const E *__restrict__ in, E *__restrict__ xt, int n_xtiles,
     int n_ctiles) {
@@ -25,6 +26,7 @@ __global__ __launch_bounds__(256) void relayout_kernel(
   b /= n_ctiles;
   const int yp = b % g.Hp;
   const int n = b / g.Hp;
+  const int slabs_total = g.Cin / KC;
 
   const int tid = threadIdx.x;
   const bool row_inside = (yp >= 1) && (yp <= g.H);
@@ -44,14 +46,21 @@ __global__ __launch_bounds__(256) void relayout_kernel(
   }
   __syncthreads();
   {
-    const int cl = tid & 63;
-    const int c = ctile * 64 + cl;
+    // lanes run over the KC channels of a slab, then over pixels
+    const int kc = tid % KC;
+    constexpr int PX_PER_PASS = 256 / KC;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int xl = (tid >> 6) + 4 * i;
-      const int xp = xtile * 64 + xl;
-      if (xp < g.Wp && c < g.Cin)
-        xt[(((long)n * g.Hp + yp) * g.Wp + xp) * g.Cin + c] = tile[cl][xl];
+    for (int sl = 0; sl < 64 / KC; ++sl) {
+      const int cl = sl * KC + kc;
+      const int c = ctile * 64 + cl;
+      const int slab = c / KC;
+#pragma unroll
+      for (int i = 0; i < 64 / PX_PER_PASS; ++i) {
+        const int xl = tid / KC + PX_PER_PASS * i;
+        const int xp = xtile * 64 + xl;
+        if (xp < g.Wp && c < g.Cin)
+          xt[((((long)n * slabs_total + slab) * g.Hp + yp) * g.Wp + xp) * KC + kc] = tile[cl][xl];
+      }
     }
   }
 }
