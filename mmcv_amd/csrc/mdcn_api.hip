@@ -60,9 +60,11 @@ inline int slab_channels(int dtype) { return dtype == MDCN_F32 ? 16 : 32; }
 // Output-channel tile of the fused kernel for a group of cout_g channels.
 inline int pick_ct(int cout_g) { return cout_g > 128 ? 256 : (cout_g > 64 ? 128 : 64); }
 
+inline int table_capacity(int taps) { return taps <= kTapsSmall ? kTapsSmall : kTapsLarge; }
+
 inline size_t fused_lds(int dtype, int CT, int taps) {
-  return dtype == MDCN_F32 ? fused_lds_bytes<float>(CT, taps)
-                           : fused_lds_bytes<bf16_t>(CT, taps);
+  const int tmax = table_capacity(taps);
+  return dtype == MDCN_F32 ? fused_lds_bytes<float>(CT, tmax) : fused_lds_bytes<bf16_t>(CT, tmax);
 }
 
 bool fused_ok(const mdcn_params *p, const Geom &g) {
@@ -71,6 +73,7 @@ bool fused_ok(const mdcn_params *p, const Geom &g) {
   // with several deformable groups the gather pipeline must stay inside one
   // group's table while it fills
   if (g.DG > 1 && (g.ch_per_dg / KC) * g.taps < kGatherAhead + 1) return false;
+  if (g.taps > kTapsLarge) return false;
   if (fused_lds(p->dtype, pick_ct(g.cout_g), g.taps) > kMaxLds) return false;
   // one padded image must fit the 32-bit offsets
   const uint64_t img = (uint64_t)g.Hp * g.Wp * g.Cin * elem_size(p->dtype);
@@ -119,32 +122,25 @@ int make_plan(const mdcn_params *p, const Geom &g, Plan *pl) {
   return MDCN_OK;
 }
 
-template <typename E, int CT>
-hipError_t launch_fused_ct(const FusedArgs &fa, size_t dyn_lds, hipStream_t st) {
-  auto kern = fused_kernel<E, CT>;
-  static bool attr_set[64] = {false};  // per device; a race only repeats the call
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
-  if (!attr_set[dev]) {
-    hipError_t e = hipFuncSetAttribute((const void *)kern,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)(kMaxLds - fused_static_lds_bytes(CT)));
-    if (e != hipSuccess) return e;
-    attr_set[dev] = true;
-  }
+template <typename E, int CT, int TMAX>
+hipError_t launch_fused_ct(const FusedArgs &fa, hipStream_t st) {
   // persistent workgroups: one per CU, a multiple of the 8 XCDs
   const int total_wg = fa.n_ptiles * fa.n_ctiles * fa.g.G;
   const int per_xcd = std::max(1, std::min((total_wg + 7) / 8, num_cus() / 8));
-  hipLaunchKernelGGL(kern, dim3(per_xcd * 8), dim3(kThreads), dyn_lds, st, fa);
+  hipLaunchKernelGGL((fused_kernel<E, CT, TMAX>), dim3(per_xcd * 8), dim3(kThreads), 0, st, fa);
   return hipGetLastError();
 }
 
 template <typename E>
-hipError_t launch_fused(const FusedArgs &fa, int CT, size_t lds, hipStream_t st) {
+hipError_t launch_fused(const FusedArgs &fa, int CT, hipStream_t st) {
+  const bool small = fa.g.taps <= kTapsSmall;
   switch (CT) {
-    case 64: return launch_fused_ct<E, 64>(fa, lds, st);
-    case 128: return launch_fused_ct<E, 128>(fa, lds, st);
-    default: return launch_fused_ct<E, 256>(fa, lds, st);
+    case 64:
+      return small ? launch_fused_ct<E, 64, kTapsSmall>(fa, st) : launch_fused_ct<E, 64, kTapsLarge>(fa, st);
+    case 128:
+      return small ? launch_fused_ct<E, 128, kTapsSmall>(fa, st) : launch_fused_ct<E, 128, kTapsLarge>(fa, st);
+    default:
+      return small ? launch_fused_ct<E, 256, kTapsSmall>(fa, st) : launch_fused_ct<E, 256, kTapsLarge>(fa, st);
   }
 }
 
@@ -196,7 +192,6 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
       if (hipGetLastError() != hipSuccess) rc = MDCN_ERR_LAUNCH;
       toc(1);
     }
-    const size_t lds = fused_dyn_lds_bytes<E>(g.taps);
     for (int n0 = 0; n0 < g.N && rc == MDCN_OK; n0 += pl.n_chunk) {
       Geom gc = g;
       gc.N = std::min(pl.n_chunk, g.N - n0);
@@ -227,7 +222,7 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
       fa.row_bytes = (uint32_t)g.Wp * 64u;
       fa.out_vec_ok = (plane_out % (long)(16 / es) == 0) && (((uintptr_t)fa.out % 16) == 0);
       tic();
-      if (launch_fused<E>(fa, pl.CT, lds, st) != hipSuccess) rc = MDCN_ERR_LAUNCH;
+      if (launch_fused<E>(fa, pl.CT, st) != hipSuccess) rc = MDCN_ERR_LAUNCH;
       toc(2);
     }
   }

@@ -44,6 +44,7 @@ constexpr int kPT = 128;           // pixels per tile
 constexpr int kGatherAhead = 3;    // K steps a gather is in flight
 constexpr int kWeightAhead = 2;    // K steps a weight-tile copy is in flight
 constexpr int kWeightSlots = kWeightAhead + 2;
+static_assert((kWeightSlots & (kWeightSlots - 1)) == 0, "the slot index is taken with a mask");
 constexpr int kThreads = 512;
 
 struct FusedArgs {
@@ -233,27 +234,64 @@ constexpr int stage_row_bytes() {
   return 64 * (int)sizeof(E) + 16;
 }
 
-// Dynamic LDS of fused_kernel: the (pixel, tap) table, reused as the epilogue
-// staging area (4 consumer waves x 32 output channels x one padded row).
+// uint4 elements of the weight part of the (pixel, tap) table for up to `tmax`
+// taps; the same array is reused as the epilogue staging area (4 consumer
+// waves x 32 output channels x one padded row).
 template <typename E>
-constexpr size_t fused_dyn_lds_bytes(int taps) {
-  const size_t table = (size_t)kPT * taps * 20;
-  const size_t stage = (size_t)4 * 32 * stage_row_bytes<E>();
+constexpr int fused_tws_elems(int tmax) {
+  const int table = kPT * tmax;
+  const int stage = 4 * 32 * stage_row_bytes<E>() / 16;
   return table > stage ? table : stage;
 }
 
-// Static LDS of one workgroup: two sample tiles and the ring of weight tiles.
-constexpr size_t fused_static_lds_bytes(int CT) {
-  return (size_t)2 * kPT * 64 + (size_t)kWeightSlots * CT * 64;
-}
-
-// Static + dynamic LDS of one workgroup.
+// LDS of one workgroup: two sample tiles, the ring of weight tiles, the table.
 template <typename E>
-constexpr size_t fused_lds_bytes(int CT, int taps) {
-  return fused_static_lds_bytes(CT) + fused_dyn_lds_bytes<E>(taps);
+constexpr size_t fused_lds_bytes(int CT, int tmax) {
+  return (size_t)2 * kPT * 64 + (size_t)kWeightSlots * CT * 64 + (size_t)kPT * tmax * 4 +
+         (size_t)fused_tws_elems<E>(tmax) * 16;
 }
 
-template <typename E, int CT>
+// Table capacities the kernel is instantiated for (taps = kh * kw).
+constexpr int kTapsSmall = 9;
+constexpr int kTapsLarge = 25;
+
+// Workgroup barrier without the memory-model fence of __syncthreads(): that
+// fence would also wait for every outstanding direct-to-LDS copy (vmcnt(0)),
+// i.e. drain the weight prefetch at every K step.  Waits for this wave's own
+// LDS operations and for all but `VM` of its vector-memory operations.
+#define MDCN_BARRIER(VM) \
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(VM) : "memory")
+#define MDCN_BARRIER_LDS() asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory")
+
+// Walks the K steps of a tile in issue order (channel slab outer, tap inner) and
+// reports when a step starts a new deformable group.  Producers and consumers
+// run identical cursors, so both know when the table is rebuilt.
+struct StepCursor {
+  int step, slab, tap, dgrem;
+  bool new_dg;
+  __device__ __forceinline__ void init(int slab0, int spd) {
+    step = 0;
+    slab = 0;
+    tap = 0;
+    dgrem = slab0 % spd;
+    new_dg = false;
+  }
+  // Move to the next step; past the last step the cursor stays on it.
+  __device__ __forceinline__ void advance(int nk, int taps, int spd) {
+    if (step >= nk - 1) return;
+    ++step;
+    if (++tap == taps) {
+      tap = 0;
+      ++slab;
+      if (++dgrem == spd) {
+        dgrem = 0;
+        new_dg = true;
+      }
+    }
+  }
+};
+
+template <typename E, int CT, int TMAX>
 __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
   using TR = ElemTraits<E>;
   constexpr int PT = kPT;
@@ -263,23 +301,26 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
   constexpr int NB = 2;              // 32-pixel blocks per consumer wave
   constexpr int WDMA = CT / 64;      // 1 KiB direct-to-LDS copies per producer wave and K step
   constexpr int OPS = 8 + WDMA;      // vector-memory ops a producer lane issues per K step
+  constexpr int TPT = (TMAX + 1) / 2;  // table entries per producer lane
 
-  __shared__ uint4 Xs[2][PT * 4];                // sample tiles
-  __shared__ uint4 Ws[kWeightSlots][CT * 4];     // weight tiles
-  extern __shared__ __align__(16) unsigned char dyn[];
+  // All LDS arrays are separate static objects: the compiler then knows that
+  // the direct-to-LDS weight copies (into Ws) cannot alias the table reads.
+  __shared__ uint4 Xs[2][PT * 4];                  // sample tiles
+  __shared__ uint4 Ws[kWeightSlots][CT * 4];       // weight tiles
+  __shared__ int32_t tpix[PT * TMAX];              // (pixel, tap) table, [tap][PT]: corner index
+  __shared__ uint4 tws[fused_tws_elems<E>(TMAX)];  // ... and weights; also the epilogue staging
 
   const Geom &g = a.g;
   const int taps = g.taps;
   const int nk = a.slabs * taps;
-  const long plane_out = (long)g.Ho * g.Wo;
+  const int plane_out = g.Ho * g.Wo;
+  const int total_px = (int)a.total_px;
+  const int spd = g.ch_per_dg / KC;  // slabs per deformable group
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const bool producer = wave >= 4;
-
-  int32_t *tpix = (int32_t *)dyn;                    // [taps][PT]
-  uint4 *tws = (uint4 *)(dyn + (size_t)PT * taps * 4);  // [taps][PT]
 
   // XCD-aware persistent schedule: consecutive workgroup ids sit on different
   // XCDs; each XCD walks one contiguous run of tiles so that the halo rows
@@ -297,8 +338,12 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
     L /= a.n_ctiles;
     const int grp = L % g.G;
     const int ptile = L / g.G;
-    const long p0 = (long)ptile * PT;
+    const int p0 = ptile * PT;
     const int ch0 = grp * g.cin_g;  // first input channel of the group
+    const int slab0 = ch0 / KC;
+
+    StepCursor cur;  // the next step whose gather is issued
+    cur.init(slab0, spd);
 
     if (producer) {
       // =================== PRODUCER ===================
@@ -306,40 +351,52 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
       const int q = ptid & 3;          // 16-byte chunk of the 64-byte slab row
       const int pxl = ptid >> 2;       // pixels pxl and pxl + 64 of the tile
       const unsigned char *xt = (const unsigned char *)a.xt;
-      const int slab0 = ch0 / KC;
 
       // -- (pixel, tap) table of one deformable group; lane serves pixel ptid%128
       const int tb_pl = ptid & (PT - 1);
-      const long tb_p = p0 + tb_pl;
-      const bool tb_valid = tb_p < a.total_px;
-      int tb_n = 0, tb_ho = 0, tb_wo = 0;
-      long tb_rem = 0;
+      const int tb_p = p0 + tb_pl;
+      const bool tb_valid = tb_p < total_px;
+      int tb_n = 0, tb_ho = 0, tb_wo = 0, tb_rem = 0;
       if (tb_valid) {
-        tb_n = (int)(tb_p / plane_out);
-        tb_rem = tb_p - (long)tb_n * plane_out;
-        tb_ho = (int)(tb_rem / g.Wo);
-        tb_wo = (int)(tb_rem - (long)tb_ho * g.Wo);
+        tb_n = tb_p / plane_out;
+        tb_rem = tb_p - tb_n * plane_out;
+        tb_ho = tb_rem / g.Wo;
+        tb_wo = tb_rem - tb_ho * g.Wo;
       }
       auto build_table = [&](int dgi) {
         const E *off = (const E *)a.offset + ((long)tb_n * g.DG + dgi) * 2 * taps * plane_out + tb_rem;
         const E *msk = (const E *)a.mask + ((long)tb_n * g.DG + dgi) * taps * plane_out + tb_rem;
-        for (int tap = ptid >> 7; tap < taps; tap += 2) {
-          int32_t pix = 0;
-          uint32_t tw[4] = {0u, 0u, 0u, 0u};
-          if (tb_valid) {
-            const float dy = to_f32(off[(long)(2 * tap) * plane_out]);
-            const float dx = to_f32(off[(long)(2 * tap + 1) * plane_out]);
-            const float m = to_f32(msk[(long)tap * plane_out]);
-            const int i = tap / g.kw, j = tap - i * g.kw;
-            const TapSample s = make_tap_sample(tb_ho * g.sh - g.ph + i * g.dh,
-                                                tb_wo * g.sw - g.pw + j * g.dw, dy, dx, m, g.H, g.W);
-            // +1: coordinates in the zero-bordered copy (y0, x0 >= -1 when inside,
-            // 0 with zero weights otherwise); slab 0 of image tb_n.
-            pix = tb_n * a.slabs_total * a.plane_px + (s.y0 + 1) * g.Wp + (s.x0 + 1);
-            TR::table_weights(s, tw);
+        // all loads first, then the arithmetic
+        E rdy[TPT], rdx[TPT], rm[TPT];
+#pragma unroll
+        for (int i = 0; i < TPT; ++i) {
+          const int tap = (ptid >> 7) + 2 * i;
+          rdy[i] = rdx[i] = rm[i] = from_f32<E>(0.0f);
+          if (tb_valid && tap < taps) {
+            rdy[i] = off[(long)(2 * tap) * plane_out];
+            rdx[i] = off[(long)(2 * tap + 1) * plane_out];
+            rm[i] = msk[(long)tap * plane_out];
           }
-          tpix[tap * PT + tb_pl] = pix;
-          tws[tap * PT + tb_pl] = make_uint4(tw[0], tw[1], tw[2], tw[3]);
+        }
+#pragma unroll
+        for (int i = 0; i < TPT; ++i) {
+          const int tap = (ptid >> 7) + 2 * i;
+          if (tap < taps) {
+            int32_t pix = 0;
+            uint32_t tw[4] = {0u, 0u, 0u, 0u};
+            if (tb_valid) {
+              const int ti = tap / g.kw, tj = tap - ti * g.kw;
+              const TapSample sm =
+                  make_tap_sample(tb_ho * g.sh - g.ph + ti * g.dh, tb_wo * g.sw - g.pw + tj * g.dw,
+                                  to_f32(rdy[i]), to_f32(rdx[i]), to_f32(rm[i]), g.H, g.W);
+              // +1: coordinates in the zero-bordered copy (y0, x0 >= -1 when inside,
+              // 0 with zero weights otherwise); slab 0 of image tb_n.
+              pix = tb_n * a.slabs_total * a.plane_px + (sm.y0 + 1) * g.Wp + (sm.x0 + 1);
+              TR::table_weights(sm, tw);
+            }
+            tpix[tap * PT + tb_pl] = pix;
+            tws[tap * PT + tb_pl] = make_uint4(tw[0], tw[1], tw[2], tw[3]);
+          }
         }
       };
 
@@ -347,14 +404,20 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
       uint4 gv[kGatherAhead][2][4];
       uint4 gw[kGatherAhead][2];
 
-      auto issue_gather = [&](int ks, uint4 (&v)[2][4], uint4 (&w)[2]) {
-        const int kk = min(ks, nk - 1);  // past the end: repeat the last step (never consumed)
-        const int slab = kk / taps;
-        const int tap = kk - slab * taps;
-        const int sbase = (slab0 + slab) * a.plane_px;
+      // Gather of the cursor's step (rebuilding the table first when the step
+      // opens a new deformable group), then move the cursor on.
+      auto issue_gather = [&](uint4 (&v)[2][4], uint4 (&w)[2]) {
+        if (cur.new_dg) {
+          // Every producer issued the previous group's last step before the
+          // barrier that ended the previous K step, with its weights in registers.
+          cur.new_dg = false;
+          build_table((ch0 + cur.slab * KC) / g.ch_per_dg);
+          MDCN_BARRIER_LDS();  // R: new table visible (the consumers join)
+        }
+        const int sbase = (slab0 + cur.slab) * a.plane_px;
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-          const int e = tap * PT + pxl + 64 * h;
+          const int e = cur.tap * PT + pxl + 64 * h;
           const uint32_t o = ((uint32_t)(tpix[e] + sbase) << 6) + (uint32_t)q * 16u;
           w[h] = tws[e];
           const unsigned char *top = xt + o;
@@ -364,6 +427,7 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
           v[h][2] = *(const uint4 *)(bot);
           v[h][3] = *(const uint4 *)(bot + 64);
         }
+        cur.advance(nk, taps, spd);
       };
 
       // weight tile of step ks -> ring slot ks % kWeightSlots, straight into LDS:
@@ -371,18 +435,22 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
       // chunk that the swizzle assigns to it.
       const unsigned char *wp_tile = (const unsigned char *)a.wp +
                                      ((size_t)(grp * a.n_ctiles + ctile) * nk) * (size_t)(CT * 64);
+      uint32_t wlane[WDMA];  // byte offset of this lane's source chunk inside a tile
+#pragma unroll
+      for (int c = 0; c < WDMA; ++c) {
+        const int d = ((wave - 4) * WDMA + c) * 64 + lane;
+        const int row = d >> 2;
+        wlane[c] = (uint32_t)(row * 64 + (((d & 3) ^ ((row >> 2) & 3)) * 16));
+      }
       auto issue_weights = [&](int ks) {
-        const int kk = min(ks, nk - 1);
+        const int kk = min(ks, nk - 1);  // past the end: repeat the last tile (never read)
         const unsigned char *src = wp_tile + (size_t)kk * (CT * 64);
-        const int slot = ks % kWeightSlots;
+        const int slot = ks & (kWeightSlots - 1);
 #pragma unroll
         for (int c = 0; c < WDMA; ++c) {
-          const int blk = (wave - 4) * WDMA + c;   // 1 KiB block of the tile
-          const int d = blk * 64 + lane;           // destination chunk
-          const int row = d >> 2;
-          const int sc = (d & 3) ^ ((row >> 2) & 3);
-          __builtin_amdgcn_global_load_lds((gptr_t)(src + row * 64 + sc * 16),
-                                           (lptr_t)(&Ws[slot][blk * 64]), 16, 0, 0);
+          const int blk = (wave - 4) * WDMA + c;  // 1 KiB block of the tile
+          __builtin_amdgcn_global_load_lds((gptr_t)(src + wlane[c]), (lptr_t)(&Ws[slot][blk * 64]),
+                                           16, 0, 0);
         }
       };
 
@@ -394,10 +462,8 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
         }
       };
 
-      // Deformable group of the (clamped) K step ks; the table holds one group.
-      auto dg_of = [&](int ks) { return (ch0 + (min(ks, nk - 1) / taps) * KC) / g.ch_per_dg; };
-      build_table(dg_of(0));
-      __syncthreads();  // B0: table visible
+      build_table(ch0 / g.ch_per_dg);
+      MDCN_BARRIER_LDS();  // B0: table visible
 
       // Issue order is that of the steady state extended to "virtual" steps
       // v = -1-kGatherAhead .. -1: step v issues gather(v+1+kGatherAhead) and then
@@ -406,14 +472,13 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
       // outstanding" always means the weight tile of the next step has landed.
 #pragma unroll
       for (int v = -1 - kGatherAhead; v < -1; ++v) {
-        issue_gather(v + 1 + kGatherAhead, gv[v + 1 + kGatherAhead], gw[v + 1 + kGatherAhead]);
+        issue_gather(gv[v + 1 + kGatherAhead], gw[v + 1 + kGatherAhead]);
         if (v + 1 + kWeightAhead >= 0) issue_weights(v + 1 + kWeightAhead);
       }
       commit(0, gv[0], gw[0]);
-      issue_gather(kGatherAhead, gv[0], gw[0]);
+      issue_gather(gv[0], gw[0]);
       issue_weights(kWeightAhead);
-      MDCN_WAIT_VMCNT(kWeightAhead * OPS);
-      __syncthreads();  // B1: X[0], W[0] visible
+      MDCN_BARRIER(kWeightAhead * OPS);  // B1: X[0], W[0] visible
 
       for (int ks0 = 0; ks0 < nk; ks0 += kGatherAhead) {
 #pragma unroll
@@ -422,23 +487,14 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
           if (ks < nk) {
             const int set = (j + 1) % kGatherAhead;  // holds step ks + 1
             commit((ks + 1) & 1, gv[set], gw[set]);
-            if (dg_of(ks + 1 + kGatherAhead) != dg_of(ks + kGatherAhead)) {
-              // Next step to issue samples with another deformable group's offsets.
-              // Every producer issued step ks + kGatherAhead before the barrier that
-              // ended the previous step, and took its weights into registers.
-              build_table(dg_of(ks + 1 + kGatherAhead));
-              __syncthreads();  // R: new table visible (consumers join, see below)
-            }
-            issue_gather(ks + 1 + kGatherAhead, gv[set], gw[set]);
+            issue_gather(gv[set], gw[set]);          // step ks + 1 + kGatherAhead
             issue_weights(ks + 1 + kWeightAhead);
-            MDCN_WAIT_VMCNT(kWeightAhead * OPS);
-            __syncthreads();  // end of step ks: X[ks+1], W[ks+1] visible
+            MDCN_BARRIER(kWeightAhead * OPS);  // end of step ks: X[ks+1], W[ks+1] visible
           }
         }
       }
-      MDCN_WAIT_VMCNT(0);  // the copies issued past the end must land before LDS is reused
-      __syncthreads();     // E0: consumers own the dynamic LDS (staging) from here
-      __syncthreads();     // E1: epilogue done, the table may be rebuilt
+      MDCN_BARRIER(0);      // E0: copies issued past the end have landed; consumers take tws
+      MDCN_BARRIER_LDS();   // E1: epilogue done, the table may be rebuilt
     } else {
       // =================== CONSUMER ===================
       const int wave_p = wave & 1;   // which 64 pixels
@@ -453,13 +509,22 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
 
       const int frow = lane & 31;
       const int fhalf = lane >> 5;
-      auto dg_of = [&](int ks) { return (ch0 + (min(ks, nk - 1) / taps) * KC) / g.ch_per_dg; };
-      __syncthreads();  // B0
-      __syncthreads();  // B1
+      // mirror of the producers' issue sequence, for the table-rebuild barriers
+      auto mirror_issue = [&]() {
+        if (cur.new_dg) {
+          cur.new_dg = false;
+          MDCN_BARRIER_LDS();  // R
+        }
+        cur.advance(nk, taps, spd);
+      };
+      MDCN_BARRIER_LDS();  // B0
+#pragma unroll
+      for (int v = 0; v <= kGatherAhead; ++v) mirror_issue();
+      MDCN_BARRIER_LDS();  // B1
 
       for (int ks = 0; ks < nk; ++ks) {
         const uint4 *X = Xs[ks & 1];
-        const uint4 *W = Ws[ks % kWeightSlots];
+        const uint4 *W = Ws[ks & (kWeightSlots - 1)];
 #pragma unroll
         for (int ksub = 0; ksub < 2; ++ksub) {
           const int ch = ksub * 2 + fhalf;
@@ -479,11 +544,10 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) TR::mma(acc[nb][mb], xf[nb], wf[mb]);
         }
-        if (dg_of(ks + 1 + kGatherAhead) != dg_of(ks + kGatherAhead))
-          __syncthreads();  // R: producers publish the next deformable group's table
-        __syncthreads();  // end of step ks
+        mirror_issue();
+        MDCN_BARRIER_LDS();  // end of step ks
       }
-      __syncthreads();  // E0
+      MDCN_BARRIER_LDS();  // E0
 
       // ---- epilogue: bias, round once, transpose through LDS, NCHW store ----
       // Accumulator block (A = samples, B = weights): register r of lane l holds
@@ -491,10 +555,10 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
       constexpr int RB = stage_row_bytes<E>();
       constexpr int CHUNK_PX = 16 / ES;           // pixels per 16-byte chunk
       constexpr int CHUNKS = 64 / CHUNK_PX;       // chunks per staged row
-      unsigned char *stage = dyn + (size_t)wave * 32 * RB;
+      unsigned char *stage = (unsigned char *)tws + (size_t)wave * 32 * RB;
       E *out = (E *)a.out;
-      const long pw0 = p0 + wave_p * 64;          // first pixel of this wave
-      const bool vec_ok = a.out_vec_ok != 0;  // 16-byte chunks never straddle images and are aligned
+      const int pw0 = p0 + wave_p * 64;           // first pixel of this wave
+      const bool vec_ok = a.out_vec_ok != 0;      // 16-byte chunks never straddle images, aligned
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
         const int col0 = ctile * CT + wave_c * (CT / 2) + mb * 32;  // channel within the group
@@ -511,43 +575,39 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
                        acc[nb][mb][r4 * 4 + 3] + bv);
           }
         }
-        // same wave wrote and reads: LDS operations of a wave complete in order
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
+        // the same wave wrote and now reads: only its own LDS operations matter
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll 1
         for (int it = 0; it < 32 * CHUNKS / 64; ++it) {
           const int idx = it * 64 + lane;
           const int row = idx / CHUNKS;        // channel of the block
-          const int chunk = idx % CHUNKS;
+          const int chunk_i = idx % CHUNKS;
           const int col = col0 + row;
-          const long p = pw0 + chunk * CHUNK_PX;
-          if (col < g.cout_g && p < a.total_px) {
-            const uint4 val = *(const uint4 *)(stage + row * RB + chunk * 16);
-            const int n = (int)(p / plane_out);
-            const long rem = p - (long)n * plane_out;
-            E *o = out + ((long)n * g.Cout + (long)grp * g.cout_g + col) * plane_out + rem;
-            if (vec_ok && p + CHUNK_PX <= a.total_px) {
-              *(uint4 *)o = val;   // chunk lies in one image and is 16-byte aligned
+          const int p = pw0 + chunk_i * CHUNK_PX;
+          if (col < g.cout_g && p < total_px) {
+            const uint4 val = *(const uint4 *)(stage + row * RB + chunk_i * 16);
+            const long cbase = (long)grp * g.cout_g + col;
+            if (vec_ok && p + CHUNK_PX <= total_px) {
+              const int n = p / plane_out;
+              const int rem = p - n * plane_out;
+              *(uint4 *)(out + ((long)n * g.Cout + cbase) * plane_out + rem) = val;
             } else {
               const E *ve = (const E *)&val;
-#pragma unroll
+#pragma unroll 1
               for (int i = 0; i < CHUNK_PX; ++i) {
-                const long pi = p + i;
-                if (pi < a.total_px) {
-                  const int ni = (int)(pi / plane_out);
-                  const long ri = pi - (long)ni * plane_out;
-                  out[((long)ni * g.Cout + (long)grp * g.cout_g + col) * plane_out + ri] = ve[i];
+                const int pi = p + i;
+                if (pi < total_px) {
+                  const int ni = pi / plane_out;
+                  const int ri = pi - ni * plane_out;
+                  out[((long)ni * g.Cout + cbase) * plane_out + ri] = ve[i];
                 }
               }
             }
           }
         }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       }
-      __syncthreads();  // E1
+      MDCN_BARRIER_LDS();  // E1
     }
   }
 }
