@@ -122,25 +122,32 @@ int make_plan(const mdcn_params *p, const Geom &g, Plan *pl) {
   return MDCN_OK;
 }
 
-template <typename E, int CT, int TMAX>
+template <typename E, int CT, int TMAX, bool MULTI_DG>
 hipError_t launch_fused_ct(const FusedArgs &fa, hipStream_t st) {
   // persistent workgroups: one per CU, a multiple of the 8 XCDs
   const int total_wg = fa.n_ptiles * fa.n_ctiles * fa.g.G;
   const int per_xcd = std::max(1, std::min((total_wg + 7) / 8, num_cus() / 8));
-  hipLaunchKernelGGL((fused_kernel<E, CT, TMAX>), dim3(per_xcd * 8), dim3(kThreads), 0, st, fa);
+  hipLaunchKernelGGL((fused_kernel<E, CT, TMAX, MULTI_DG>), dim3(per_xcd * 8), dim3(kThreads), 0,
+                     st, fa);
   return hipGetLastError();
+}
+
+template <typename E, int CT>
+hipError_t launch_fused_tm(const FusedArgs &fa, hipStream_t st) {
+  const bool small = fa.g.taps <= kTapsSmall;
+  if (fa.g.DG > 1)
+    return small ? launch_fused_ct<E, CT, kTapsSmall, true>(fa, st)
+                 : launch_fused_ct<E, CT, kTapsLarge, true>(fa, st);
+  return small ? launch_fused_ct<E, CT, kTapsSmall, false>(fa, st)
+               : launch_fused_ct<E, CT, kTapsLarge, false>(fa, st);
 }
 
 template <typename E>
 hipError_t launch_fused(const FusedArgs &fa, int CT, hipStream_t st) {
-  const bool small = fa.g.taps <= kTapsSmall;
   switch (CT) {
-    case 64:
-      return small ? launch_fused_ct<E, 64, kTapsSmall>(fa, st) : launch_fused_ct<E, 64, kTapsLarge>(fa, st);
-    case 128:
-      return small ? launch_fused_ct<E, 128, kTapsSmall>(fa, st) : launch_fused_ct<E, 128, kTapsLarge>(fa, st);
-    default:
-      return small ? launch_fused_ct<E, 256, kTapsSmall>(fa, st) : launch_fused_ct<E, 256, kTapsLarge>(fa, st);
+    case 64: return launch_fused_tm<E, 64>(fa, st);
+    case 128: return launch_fused_tm<E, 128>(fa, st);
+    default: return launch_fused_tm<E, 256>(fa, st);
   }
 }
 

@@ -263,6 +263,21 @@ constexpr int kTapsLarge = 25;
   asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(VM) : "memory")
 #define MDCN_BARRIER_LDS() asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory")
 
+// 16 bytes per lane from global memory straight into LDS: lane i's data lands at
+// lds_base + 16*i (lds_base, in M0, is the same for the whole wave).  Written as
+// inline assembly on purpose: the compiler treats the builtin as a flat access
+// that may touch both memories and then answers every later register or LDS
+// dependency with vmcnt(0)/lgkmcnt(0), which would drain the gather prefetch at
+// every K step.  Unseen by the compiler, the copies only make its own vmcnt
+// waits stricter than necessary (they count as extra younger operations); their
+// completion is waited for explicitly (MDCN_BARRIER).
+__device__ __forceinline__ void copy16_global_to_lds(const void *src, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+               :
+               : "s"(lds_base), "v"(src)
+               : "memory");
+}
+
 // Walks the K steps of a tile in issue order (channel slab outer, tap inner) and
 // reports when a step starts a new deformable group.  Producers and consumers
 // run identical cursors, so both know when the table is rebuilt.
@@ -291,7 +306,11 @@ struct StepCursor {
   }
 };
 
-template <typename E, int CT, int TMAX>
+// MULTI_DG: more than one deformable group, i.e. the table is rebuilt inside the
+// K loop.  Kept out of the single-group instantiation because a conditional
+// block with loads inside the step loop makes the compiler drain the gather
+// prefetch (vmcnt(0)) at every step.
+template <typename E, int CT, int TMAX, bool MULTI_DG>
 __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
   using TR = ElemTraits<E>;
   constexpr int PT = kPT;
@@ -313,6 +332,7 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
   const Geom &g = a.g;
   const int taps = g.taps;
   const int nk = a.slabs * taps;
+  const int nk_pad = (nk + kGatherAhead - 1) / kGatherAhead * kGatherAhead;
   const int plane_out = g.Ho * g.Wo;
   const int total_px = (int)a.total_px;
   const int spd = g.ch_per_dg / KC;  // slabs per deformable group
@@ -407,7 +427,7 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
       // Gather of the cursor's step (rebuilding the table first when the step
       // opens a new deformable group), then move the cursor on.
       auto issue_gather = [&](uint4 (&v)[2][4], uint4 (&w)[2]) {
-        if (cur.new_dg) {
+        if (MULTI_DG && cur.new_dg) {
           // Every producer issued the previous group's last step before the
           // barrier that ended the previous K step, with its weights in registers.
           cur.new_dg = false;
@@ -449,8 +469,7 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
 #pragma unroll
         for (int c = 0; c < WDMA; ++c) {
           const int blk = (wave - 4) * WDMA + c;  // 1 KiB block of the tile
-          __builtin_amdgcn_global_load_lds((gptr_t)(src + wlane[c]), (lptr_t)(&Ws[slot][blk * 64]),
-                                           16, 0, 0);
+          copy16_global_to_lds(src + wlane[c], (uint32_t)(uintptr_t)(lptr_t)(&Ws[slot][blk * 64]));
         }
       };
 
@@ -480,17 +499,19 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
       issue_weights(kWeightAhead);
       MDCN_BARRIER(kWeightAhead * OPS);  // B1: X[0], W[0] visible
 
-      for (int ks0 = 0; ks0 < nk; ks0 += kGatherAhead) {
+      // The step loop runs in whole rounds of kGatherAhead steps (register sets are
+      // addressed statically and the body stays branch-free, so the compiler's
+      // vmcnt bookkeeping sees one fixed issue pattern); steps past nk repeat the
+      // last one and nobody reads what they produce.
+      for (int ks0 = 0; ks0 < nk_pad; ks0 += kGatherAhead) {
 #pragma unroll
         for (int j = 0; j < kGatherAhead; ++j) {
           const int ks = ks0 + j;
-          if (ks < nk) {
-            const int set = (j + 1) % kGatherAhead;  // holds step ks + 1
-            commit((ks + 1) & 1, gv[set], gw[set]);
-            issue_gather(gv[set], gw[set]);          // step ks + 1 + kGatherAhead
-            issue_weights(ks + 1 + kWeightAhead);
-            MDCN_BARRIER(kWeightAhead * OPS);  // end of step ks: X[ks+1], W[ks+1] visible
-          }
+          const int set = (j + 1) % kGatherAhead;  // holds step ks + 1
+          commit((ks + 1) & 1, gv[set], gw[set]);
+          issue_gather(gv[set], gw[set]);          // step ks + 1 + kGatherAhead
+          issue_weights(ks + 1 + kWeightAhead);
+          MDCN_BARRIER(kWeightAhead * OPS);  // end of step ks: X[ks+1], W[ks+1] visible
         }
       }
       MDCN_BARRIER(0);      // E0: copies issued past the end have landed; consumers take tws
@@ -511,7 +532,7 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
       const int fhalf = lane >> 5;
       // mirror of the producers' issue sequence, for the table-rebuild barriers
       auto mirror_issue = [&]() {
-        if (cur.new_dg) {
+        if (MULTI_DG && cur.new_dg) {
           cur.new_dg = false;
           MDCN_BARRIER_LDS();  // R
         }
@@ -522,9 +543,10 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
       for (int v = 0; v <= kGatherAhead; ++v) mirror_issue();
       MDCN_BARRIER_LDS();  // B1
 
-      for (int ks = 0; ks < nk; ++ks) {
+      for (int ks = 0; ks < nk_pad; ++ks) {
         const uint4 *X = Xs[ks & 1];
         const uint4 *W = Ws[ks & (kWeightSlots - 1)];
+        if (ks < nk) {
 #pragma unroll
         for (int ksub = 0; ksub < 2; ++ksub) {
           const int ch = ksub * 2 + fhalf;
@@ -543,6 +565,7 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
           for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) TR::mma(acc[nb][mb], xf[nb], wf[mb]);
+        }
         }
         mirror_issue();
         MDCN_BARRIER_LDS();  // end of step ks
