@@ -55,26 +55,23 @@ int check_params(const mdcn_params *p, Geom *g, bool need_ptrs) {
   return MDCN_OK;
 }
 
-inline int slab_channels(int dtype) { return dtype == MDCN_F32 ? 16 : 32; }
-
-// Output-channel tile of the fused kernel for a group of cout_g channels.
-inline int pick_ct(int cout_g) { return cout_g > 128 ? 256 : (cout_g > 64 ? 128 : 64); }
+// channels per K step: 128 bytes
+inline int slab_channels(int dtype) { return dtype == MDCN_F32 ? 32 : 64; }
 
 inline int table_capacity(int taps) { return taps <= kTapsSmall ? kTapsSmall : kTapsLarge; }
 
-inline size_t fused_lds(int dtype, int CT, int taps) {
-  const int tmax = table_capacity(taps);
-  return dtype == MDCN_F32 ? fused_lds_bytes<float>(CT, tmax) : fused_lds_bytes<bf16_t>(CT, tmax);
+// Output-channel tile of the fused kernel for a group of cout_g channels; the
+// 256-wide tile leaves LDS room for the 9-tap table only.
+inline int pick_ct(int cout_g, int taps) {
+  if (cout_g > 128 && taps <= kTapsSmall) return 256;
+  return cout_g > 64 ? 128 : 64;
 }
 
 bool fused_ok(const mdcn_params *p, const Geom &g) {
   const int KC = slab_channels(p->dtype);
   if (g.cin_g % KC || g.ch_per_dg % KC) return false;
-  // with several deformable groups the gather pipeline must stay inside one
-  // group's table while it fills
-  if (g.DG > 1 && (g.ch_per_dg / KC) * g.taps < kGatherAhead + 1) return false;
   if (g.taps > kTapsLarge) return false;
-  if (fused_lds(p->dtype, pick_ct(g.cout_g), g.taps) > kMaxLds) return false;
+  if (fused_lds_bytes(pick_ct(g.cout_g, g.taps), table_capacity(g.taps)) > kMaxLds) return false;
   // one padded image must fit the 32-bit offsets
   const uint64_t img = (uint64_t)g.Hp * g.Wp * g.Cin * elem_size(p->dtype);
   if (img > kMaxXtBytes) return false;
@@ -112,7 +109,7 @@ int make_plan(const mdcn_params *p, const Geom &g, Plan *pl) {
   if (!pl->fused) return MDCN_OK;
   const size_t es = elem_size(p->dtype);
   pl->KC = slab_channels(p->dtype);
-  pl->CT = pick_ct(g.cout_g);
+  pl->CT = pick_ct(g.cout_g, g.taps);
   pl->n_ctiles = (g.cout_g + pl->CT - 1) / pl->CT;
   pl->slabs = g.cin_g / pl->KC;
   const uint64_t img = (uint64_t)g.Hp * g.Wp * g.Cin * es;
@@ -135,11 +132,16 @@ hipError_t launch_fused_ct(const FusedArgs &fa, hipStream_t st) {
 template <typename E, int CT>
 hipError_t launch_fused_tm(const FusedArgs &fa, hipStream_t st) {
   const bool small = fa.g.taps <= kTapsSmall;
-  if (fa.g.DG > 1)
-    return small ? launch_fused_ct<E, CT, kTapsSmall, true>(fa, st)
-                 : launch_fused_ct<E, CT, kTapsLarge, true>(fa, st);
-  return small ? launch_fused_ct<E, CT, kTapsSmall, false>(fa, st)
-               : launch_fused_ct<E, CT, kTapsLarge, false>(fa, st);
+  if constexpr (CT == 256) {  // (pick_ct never pairs the 256-wide tile with the large table)
+    return fa.g.DG > 1 ? launch_fused_ct<E, CT, kTapsSmall, true>(fa, st)
+                       : launch_fused_ct<E, CT, kTapsSmall, false>(fa, st);
+  } else {
+    if (fa.g.DG > 1)
+      return small ? launch_fused_ct<E, CT, kTapsSmall, true>(fa, st)
+                   : launch_fused_ct<E, CT, kTapsLarge, true>(fa, st);
+    return small ? launch_fused_ct<E, CT, kTapsSmall, false>(fa, st)
+                 : launch_fused_ct<E, CT, kTapsLarge, false>(fa, st);
+  }
 }
 
 template <typename E>
@@ -226,7 +228,7 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
       fa.slabs = pl.slabs;
       fa.slabs_total = g.Cin / pl.KC;
       fa.plane_px = g.Hp * g.Wp;
-      fa.row_bytes = (uint32_t)g.Wp * 64u;
+      fa.row_bytes = (uint32_t)g.Wp * (uint32_t)kRowB;
       fa.out_vec_ok = (plane_out % (long)(16 / es) == 0) && (((uintptr_t)fa.out % 16) == 0);
       tic();
       if (launch_fused<E>(fa, pl.CT, st) != hipSuccess) rc = MDCN_ERR_LAUNCH;

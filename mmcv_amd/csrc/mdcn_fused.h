@@ -7,33 +7,34 @@
 // Work split.  A persistent workgroup of 8 wavefronts owns, one after another,
 // tiles of PT = 128 consecutive output pixels (flattened n*Ho*Wo + ho*Wo + wo)
 // x CT output channels of one group.  K runs over (slab of KC channels) x
-// (tap), slab outer, tap inner; the input copy is stored slab-major
-// ([N][Cin/KC][H+2][W+2][KC], 64 bytes per pixel and slab) so that the KC
-// channels of the neighbourhood a tile samples are compact in memory and stay
-// cache resident across the kh*kw taps.
+// (tap), slab outer, tap inner.  A slab is 128 bytes of channels (64 bf16/fp16,
+// 32 fp32), and the input copy is stored slab-major
+// ([N][Cin/KC][H+2][W+2][KC]): one bilinear corner of one slab is exactly one
+// aligned 128-byte cache line, so every byte a gather pulls from L2 is used.
 //
 // The wavefronts are specialised:
 //   waves 4..7  PRODUCERS.  Once per tile (and deformable group) they fill a
 //     table in LDS with, for every (pixel, tap), the index of the top-left
 //     bilinear corner in the zero-bordered input copy and the four mask-scaled
 //     bilinear weights (positions and weights in fp32).  Per K step, each lane
-//     gathers for two pixels 16 bytes of channels at each of the four corners
-//     (8 x global_load_dwordx4, issued kGatherAhead steps ahead, held in
-//     registers), blends them (v_dot2_f32_{bf16,f16} on the raw 16-bit pairs,
-//     FMA for fp32) and writes 2 x 16 bytes of the sample tile.  They also
-//     start the direct-to-LDS copy of the weight tile kWeightAhead steps ahead.
+//     gathers for two pixels 2 x 16 bytes of channels at each of the four corners
+//     (16 x global_load_dwordx4, issued kGatherAhead steps ahead, held in
+//     registers), blends them (v_dot2 on the raw bf16 pairs, mixed-precision FMA
+//     for fp16, FMA for fp32) and writes 4 x 16 bytes of the sample tile.  They
+//     also start the direct-to-LDS copy of the weight tile kWeightAhead steps
+//     ahead.
 //   waves 0..3  CONSUMERS.  2 x 2 over the tile (64 pixels x CT/2 channels
 //     each): read sample and weight fragments from LDS, run MFMA
 //     (32x32x16 bf16/f16, 32x32x2 fp32) into fp32 accumulators; at the end of
 //     the tile add the bias, round once, transpose through LDS and store
 //     16 bytes per lane along W of the NCHW output.
 // One workgroup barrier per K step keeps the two roles in step; the sample
-// tile is double buffered, the weight tiles sit in a ring of kWeightAhead + 2.
+// tile is double buffered, the weight tiles sit in a ring of kWeightSlots.
 //
-// LDS tiles have 64-byte rows (one pixel resp. one output channel, KC elements
-// of K); the 16-byte chunk c of row r is stored at chunk c ^ ((r >> 2) & 3), so
-// that both the 16-byte fragment reads (32 consecutive rows, one chunk) and the
-// writes (4 lanes per row) touch every bank once.
+// LDS tiles have 128-byte rows (one pixel resp. one output channel, KC elements
+// of K); the 16-byte chunks of a row are permuted (swz) so that both the
+// 16-byte fragment reads (32 consecutive rows, one chunk) and the writes
+// (4 lanes per row) spread over all banks.
 #pragma once
 
 #include "mdcn_common.h"
@@ -41,10 +42,11 @@
 namespace mdcn {
 
 constexpr int kPT = 128;           // pixels per tile
-constexpr int kGatherAhead = 3;    // K steps a gather is in flight
-constexpr int kWeightAhead = 2;    // K steps a weight-tile copy is in flight
+constexpr int kRowB = 128;         // bytes of K per tile row and K step
+constexpr int kRowChunks = kRowB / 16;
+constexpr int kGatherAhead = 2;    // K steps a gather is in flight
+constexpr int kWeightAhead = 1;    // K steps a weight-tile copy is in flight
 constexpr int kWeightSlots = kWeightAhead + 2;
-static_assert((kWeightSlots & (kWeightSlots - 1)) == 0, "the slot index is taken with a mask");
 constexpr int kThreads = 512;
 
 struct FusedArgs {
@@ -60,27 +62,20 @@ struct FusedArgs {
   int slabs_total;     // Cin / KC
   int plane_px;        // Hp * Wp
   int out_vec_ok;      // (Ho*Wo) % (16/sizeof(E)) == 0 and the output pointer is 16-byte aligned
-  uint32_t row_bytes;  // Wp * 64
+  uint32_t row_bytes;  // Wp * kRowB
 };
 
-typedef const __attribute__((address_space(1))) void *gptr_t;
 typedef __attribute__((address_space(3))) void *lptr_t;
-
-// s_waitcnt on the vector-memory counter only (gfx9 encoding).
-#define MDCN_WAIT_VMCNT(n) \
-  __builtin_amdgcn_s_waitcnt(((n) & 15) | (7 << 4) | (15 << 8) | (((n) >> 4) << 14))
 
 template <typename E>
 struct ElemTraits;
 
 // ---- 16-bit element types ---------------------------------------------------
 // A 32-bit word of gathered data holds two channels and is fed to the blend
-// instruction unchanged (no unpacking); the first corner uses the constant 0 as
-// accumulator, so nothing is cleared beforehand.
+// instruction unchanged (no unpacking).
 template <typename E>
 struct Half16Traits {
-  static constexpr int KC = 32;  // channels per K step (64 bytes)
-  static constexpr int NS = 8;   // samples per lane, pixel and K step (16 bytes)
+  static constexpr int KC = 64;  // channels per K step (128 bytes)
 
   static __device__ __forceinline__ void table_weights(const TapSample &s, uint32_t (&tw)[4]) {
     tw[0] = ElemTraits<E>::pack2(s.w00, 0.0f);
@@ -95,9 +90,12 @@ struct Half16Traits {
     *(uint2 *)dst = make_uint2(ElemTraits<E>::pack2(a, b), ElemTraits<E>::pack2(c, d));
   }
 
-  static __device__ __forceinline__ uint4 blend(const uint4 (&v)[4], const uint4 &w) {
+  // 16 bytes (8 channels) of one pixel from the same 16 bytes at its 4 corners
+  static __device__ __forceinline__ uint4 blend(const uint4 &v0, const uint4 &v1, const uint4 &v2,
+                                                const uint4 &v3, const uint4 &w) {
     const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
-    float acc[NS];
+    const uint4 v[4] = {v0, v1, v2, v3};
+    float acc[8];
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const uint32_t d[4] = {v[q].x, v[q].y, v[q].z, v[q].w};
@@ -117,8 +115,8 @@ struct Half16Traits {
   }
 };
 
-// bf16: v_dot2_f32_bf16 on the raw pair.  The table keeps the weight word
-// (w, 0); the word for the high channel, (0, w), is that shifted left by 16.
+// bf16: v_dot2 on the raw pair.  The table keeps the weight word (w, 0); the
+// word for the high channel, (0, w), is that shifted left by 16.
 template <>
 struct ElemTraits<bf16_t> : Half16Traits<bf16_t> {
   static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
@@ -187,8 +185,7 @@ struct ElemTraits<f16_t> : Half16Traits<f16_t> {
 // ---- fp32 --------------------------------------------------------------------
 template <>
 struct ElemTraits<float> {
-  static constexpr int KC = 16;
-  static constexpr int NS = 4;
+  static constexpr int KC = 32;
 
   static __device__ __forceinline__ void table_weights(const TapSample &s, uint32_t (&tw)[4]) {
     tw[0] = __float_as_uint(s.w00);
@@ -203,10 +200,12 @@ struct ElemTraits<float> {
                                __float_as_uint(d));
   }
 
-  static __device__ __forceinline__ uint4 blend(const uint4 (&v)[4], const uint4 &w) {
+  static __device__ __forceinline__ uint4 blend(const uint4 &v0, const uint4 &v1, const uint4 &v2,
+                                                const uint4 &v3, const uint4 &w) {
     const float ww[4] = {__uint_as_float(w.x), __uint_as_float(w.y), __uint_as_float(w.z),
                          __uint_as_float(w.w)};
-    float acc[NS];
+    const uint4 v[4] = {v0, v1, v2, v3};
+    float acc[4];
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const float d[4] = {__uint_as_float(v[q].x), __uint_as_float(v[q].y),
@@ -229,26 +228,20 @@ struct ElemTraits<float> {
 };
 
 // Bytes per row of the epilogue staging area: 64 pixels + 16 bytes of padding.
+// Each consumer wave stages 32 such rows; waves 0,1 use the sample tiles,
+// waves 2,3 the weight ring (both are idle once the K loop has ended).
 template <typename E>
 constexpr int stage_row_bytes() {
   return 64 * (int)sizeof(E) + 16;
 }
+static_assert(2 * 32 * (64 * 4 + 16) <= 2 * kPT * kRowB, "two staging areas fit the sample tiles");
+static_assert(2 * 32 * (64 * 4 + 16) <= kWeightSlots * 64 * kRowB,
+              "two staging areas fit the smallest weight ring");
 
-// uint4 elements of the weight part of the (pixel, tap) table for up to `tmax`
-// taps; the same array is reused as the epilogue staging area (4 consumer
-// waves x 32 output channels x one padded row).
-template <typename E>
-constexpr int fused_tws_elems(int tmax) {
-  const int table = kPT * tmax;
-  const int stage = 4 * 32 * stage_row_bytes<E>() / 16;
-  return table > stage ? table : stage;
-}
-
-// LDS of one workgroup: two sample tiles, the ring of weight tiles, the table.
-template <typename E>
+// LDS of one workgroup: two sample tiles, the ring of weight tiles, the
+// (pixel, tap) table (corner index + four weights per entry).
 constexpr size_t fused_lds_bytes(int CT, int tmax) {
-  return (size_t)2 * kPT * 64 + (size_t)kWeightSlots * CT * 64 + (size_t)kPT * tmax * 4 +
-         (size_t)fused_tws_elems<E>(tmax) * 16;
+  return (size_t)2 * kPT * kRowB + (size_t)kWeightSlots * CT * kRowB + (size_t)kPT * tmax * 20;
 }
 
 // Table capacities the kernel is instantiated for (taps = kh * kw).
@@ -256,9 +249,9 @@ constexpr int kTapsSmall = 9;
 constexpr int kTapsLarge = 25;
 
 // Workgroup barrier without the memory-model fence of __syncthreads(): that
-// fence would also wait for every outstanding direct-to-LDS copy (vmcnt(0)),
-// i.e. drain the weight prefetch at every K step.  Waits for this wave's own
-// LDS operations and for all but `VM` of its vector-memory operations.
+// fence would also wait for every outstanding vector-memory operation, i.e.
+// drain the prefetch at every K step.  Waits for this wave's own LDS operations
+// and for all but `VM` of its vector-memory operations.
 #define MDCN_BARRIER(VM) \
   asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(VM) : "memory")
 #define MDCN_BARRIER_LDS() asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory")
@@ -306,6 +299,14 @@ struct StepCursor {
   }
 };
 
+// Position of 16-byte chunk c of row r inside a tile: chunk c sits at c ^ swz(r).
+// swz runs through all 8 values over 16 consecutive rows (two rows share one and
+// sit in opposite halves of the 256-byte bank period), so the fragment reads
+// (16 consecutive rows, one chunk) are conflict free; rows 2 apart differ in
+// bit 2, so the writes (4 consecutive rows x chunks 0..3 or 4..7) are too.
+__device__ __forceinline__ int swz(int r) { return (((r >> 1) & 1) << 2) | ((r >> 2) & 3); }
+__device__ __forceinline__ int tile_chunk(int r, int c) { return r * kRowChunks + (c ^ swz(r)); }
+
 // MULTI_DG: more than one deformable group, i.e. the table is rebuilt inside the
 // K loop.  Kept out of the single-group instantiation because a conditional
 // block with loads inside the step loop makes the compiler drain the gather
@@ -318,16 +319,14 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
   constexpr int ES = (int)sizeof(E);
   constexpr int MB = CT / 64;        // 32-channel accumulator blocks per consumer wave
   constexpr int NB = 2;              // 32-pixel blocks per consumer wave
-  constexpr int WDMA = CT / 64;      // 1 KiB direct-to-LDS copies per producer wave and K step
-  constexpr int OPS = 8 + WDMA;      // vector-memory ops a producer lane issues per K step
+  constexpr int WDMA = CT / 32;      // 1 KiB direct-to-LDS copies per consumer wave and K step
   constexpr int TPT = (TMAX + 1) / 2;  // table entries per producer lane
+  static_assert(kWeightAhead * WDMA < 64, "vmcnt holds 6 bits");
 
-  // All LDS arrays are separate static objects: the compiler then knows that
-  // the direct-to-LDS weight copies (into Ws) cannot alias the table reads.
-  __shared__ uint4 Xs[2][PT * 4];                  // sample tiles
-  __shared__ uint4 Ws[kWeightSlots][CT * 4];       // weight tiles
-  __shared__ int32_t tpix[PT * TMAX];              // (pixel, tap) table, [tap][PT]: corner index
-  __shared__ uint4 tws[fused_tws_elems<E>(TMAX)];  // ... and weights; also the epilogue staging
+  __shared__ uint4 Xs[2][PT * kRowChunks];                // sample tiles
+  __shared__ uint4 Ws[kWeightSlots][CT * kRowChunks];     // weight tiles
+  __shared__ int32_t tpix[PT * TMAX];                     // (pixel, tap) table, [tap][PT]: corner
+  __shared__ uint4 tws[PT * TMAX];                        // ... and the four weights
 
   const Geom &g = a.g;
   const int taps = g.taps;
@@ -368,8 +367,8 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
     if (producer) {
       // =================== PRODUCER ===================
       const int ptid = tid - 256;
-      const int q = ptid & 3;          // 16-byte chunk of the 64-byte slab row
-      const int pxl = ptid >> 2;       // pixels pxl and pxl + 64 of the tile
+      const int q = ptid & 3;          // this lane handles 16-byte chunks q and q + 4 of a row
+      const int pxl = ptid >> 2;       // ... of pixels pxl and pxl + 64 of the tile
       const unsigned char *xt = (const unsigned char *)a.xt;
 
       // -- (pixel, tap) table of one deformable group; lane serves pixel ptid%128
@@ -384,35 +383,34 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
         tb_wo = tb_rem - tb_ho * g.Wo;
       }
       auto build_table = [&](int dgi) {
+        // (an invalid pixel reads the entries of pixel 0 of image 0 and stores zeros)
         const E *off = (const E *)a.offset + ((long)tb_n * g.DG + dgi) * 2 * taps * plane_out + tb_rem;
         const E *msk = (const E *)a.mask + ((long)tb_n * g.DG + dgi) * taps * plane_out + tb_rem;
-        // all loads first, then the arithmetic
+        // all loads first (unconditional, clamped), then the arithmetic
         E rdy[TPT], rdx[TPT], rm[TPT];
 #pragma unroll
         for (int i = 0; i < TPT; ++i) {
-          const int tap = (ptid >> 7) + 2 * i;
-          rdy[i] = rdx[i] = rm[i] = from_f32<E>(0.0f);
-          if (tb_valid && tap < taps) {
-            rdy[i] = off[(long)(2 * tap) * plane_out];
-            rdx[i] = off[(long)(2 * tap + 1) * plane_out];
-            rm[i] = msk[(long)tap * plane_out];
-          }
+          const int tap = min((ptid >> 7) + 2 * i, taps - 1);
+          rdy[i] = off[(long)(2 * tap) * plane_out];
+          rdx[i] = off[(long)(2 * tap + 1) * plane_out];
+          rm[i] = msk[(long)tap * plane_out];
         }
 #pragma unroll
         for (int i = 0; i < TPT; ++i) {
           const int tap = (ptid >> 7) + 2 * i;
           if (tap < taps) {
-            int32_t pix = 0;
-            uint32_t tw[4] = {0u, 0u, 0u, 0u};
-            if (tb_valid) {
-              const int ti = tap / g.kw, tj = tap - ti * g.kw;
-              const TapSample sm =
-                  make_tap_sample(tb_ho * g.sh - g.ph + ti * g.dh, tb_wo * g.sw - g.pw + tj * g.dw,
-                                  to_f32(rdy[i]), to_f32(rdx[i]), to_f32(rm[i]), g.H, g.W);
-              // +1: coordinates in the zero-bordered copy (y0, x0 >= -1 when inside,
-              // 0 with zero weights otherwise); slab 0 of image tb_n.
-              pix = tb_n * a.slabs_total * a.plane_px + (sm.y0 + 1) * g.Wp + (sm.x0 + 1);
-              TR::table_weights(sm, tw);
+            const int ti = tap / g.kw, tj = tap - ti * g.kw;
+            const TapSample sm =
+                make_tap_sample(tb_ho * g.sh - g.ph + ti * g.dh, tb_wo * g.sw - g.pw + tj * g.dw,
+                                to_f32(rdy[i]), to_f32(rdx[i]), to_f32(rm[i]), g.H, g.W);
+            // +1: coordinates in the zero-bordered copy (y0, x0 >= -1 when inside,
+            // 0 with zero weights otherwise); slab 0 of image tb_n.
+            int32_t pix = tb_n * a.slabs_total * a.plane_px + (sm.y0 + 1) * g.Wp + (sm.x0 + 1);
+            uint32_t tw[4];
+            TR::table_weights(sm, tw);
+            if (!tb_valid) {
+              pix = 0;
+              tw[0] = tw[1] = tw[2] = tw[3] = 0u;
             }
             tpix[tap * PT + tb_pl] = pix;
             tws[tap * PT + tb_pl] = make_uint4(tw[0], tw[1], tw[2], tw[3]);
@@ -420,13 +418,14 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
         }
       };
 
-      // -- gather state: kGatherAhead register sets, set m % kGatherAhead holds step m
-      uint4 gv[kGatherAhead][2][4];
+      // -- gather state: kGatherAhead register sets, set m % kGatherAhead holds step m;
+      //    [pixel][corner][half of the lane's 32 bytes]
+      uint4 gv[kGatherAhead][2][4][2];
       uint4 gw[kGatherAhead][2];
 
       // Gather of the cursor's step (rebuilding the table first when the step
       // opens a new deformable group), then move the cursor on.
-      auto issue_gather = [&](uint4 (&v)[2][4], uint4 (&w)[2]) {
+      auto issue_gather = [&](uint4 (&v)[2][4][2], uint4 (&w)[2]) {
         if (MULTI_DG && cur.new_dg) {
           // Every producer issued the previous group's last step before the
           // barrier that ended the previous K step, with its weights in registers.
@@ -438,66 +437,67 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
           const int e = cur.tap * PT + pxl + 64 * h;
-          const uint32_t o = ((uint32_t)(tpix[e] + sbase) << 6) + (uint32_t)q * 16u;
+          const uint32_t o = ((uint32_t)(tpix[e] + sbase) << 7) + (uint32_t)q * 16u;
           w[h] = tws[e];
           const unsigned char *top = xt + o;
           const unsigned char *bot = top + a.row_bytes;
-          v[h][0] = *(const uint4 *)(top);
-          v[h][1] = *(const uint4 *)(top + 64);
-          v[h][2] = *(const uint4 *)(bot);
-          v[h][3] = *(const uint4 *)(bot + 64);
+          v[h][0][0] = *(const uint4 *)(top);
+          v[h][0][1] = *(const uint4 *)(top + 64);
+          v[h][1][0] = *(const uint4 *)(top + 128);
+          v[h][1][1] = *(const uint4 *)(top + 192);
+          v[h][2][0] = *(const uint4 *)(bot);
+          v[h][2][1] = *(const uint4 *)(bot + 64);
+          v[h][3][0] = *(const uint4 *)(bot + 128);
+          v[h][3][1] = *(const uint4 *)(bot + 192);
         }
         cur.advance(nk, taps, spd);
       };
 
-      // weight tile of step ks -> ring slot ks % kWeightSlots, straight into LDS:
-      // lane i of copy c writes chunk c*64+i of the slot and reads the source
-      // chunk that the swizzle assigns to it.
-      const unsigned char *wp_tile = (const unsigned char *)a.wp +
-                                     ((size_t)(grp * a.n_ctiles + ctile) * nk) * (size_t)(CT * 64);
-      uint32_t wlane[WDMA];  // byte offset of this lane's source chunk inside a tile
-#pragma unroll
-      for (int c = 0; c < WDMA; ++c) {
-        const int d = ((wave - 4) * WDMA + c) * 64 + lane;
-        const int row = d >> 2;
-        wlane[c] = (uint32_t)(row * 64 + (((d & 3) ^ ((row >> 2) & 3)) * 16));
-      }
-      auto issue_weights = [&](int ks) {
-        const int kk = min(ks, nk - 1);  // past the end: repeat the last tile (never read)
-        const unsigned char *src = wp_tile + (size_t)kk * (CT * 64);
-        const int slot = ks & (kWeightSlots - 1);
-#pragma unroll
-        for (int c = 0; c < WDMA; ++c) {
-          const int blk = (wave - 4) * WDMA + c;  // 1 KiB block of the tile
-          copy16_global_to_lds(src + wlane[c], (uint32_t)(uintptr_t)(lptr_t)(&Ws[slot][blk * 64]));
+      // Blend the set (step s) into sample tile `buf` and refill it with the
+      // gather of the cursor's step, 16 bytes x 4 corners at a time: the loads go
+      // out between the blends, so the memory pipeline works while the VALU does.
+      auto commit_and_refill = [&](int buf, uint4 (&v)[2][4][2], uint4 (&w)[2]) {
+        if (MULTI_DG && cur.new_dg) {
+          cur.new_dg = false;
+          build_table((ch0 + cur.slab * KC) / g.ch_per_dg);
+          MDCN_BARRIER_LDS();  // R
         }
-      };
-
-      auto commit = [&](int buf, const uint4 (&v)[2][4], const uint4 (&w)[2]) {
+        const int sbase = (slab0 + cur.slab) * a.plane_px;
+        uint32_t o[2];
+        uint4 wn[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const int e = cur.tap * PT + pxl + 64 * h;
+          o[h] = ((uint32_t)(tpix[e] + sbase) << 7) + (uint32_t)q * 16u;
+          wn[h] = tws[e];
+        }
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
           const int row = pxl + 64 * h;
-          Xs[buf][row * 4 + (q ^ ((row >> 2) & 3))] = TR::blend(v[h], w[h]);
+#pragma unroll
+          for (int half = 0; half < 2; ++half) {
+            Xs[buf][tile_chunk(row, q + 4 * half)] =
+                TR::blend(v[h][0][half], v[h][1][half], v[h][2][half], v[h][3][half], w[h]);
+            const unsigned char *top = xt + o[h] + half * 64;
+            const unsigned char *bot = top + a.row_bytes;
+            v[h][0][half] = *(const uint4 *)(top);
+            v[h][1][half] = *(const uint4 *)(top + 128);
+            v[h][2][half] = *(const uint4 *)(bot);
+            v[h][3][half] = *(const uint4 *)(bot + 128);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+          w[h] = wn[h];
         }
+        cur.advance(nk, taps, spd);
       };
 
       build_table(ch0 / g.ch_per_dg);
       MDCN_BARRIER_LDS();  // B0: table visible
 
-      // Issue order is that of the steady state extended to "virtual" steps
-      // v = -1-kGatherAhead .. -1: step v issues gather(v+1+kGatherAhead) and then
-      // weights(v+1+kWeightAhead).  Every step from -1-kWeightAhead on issues
-      // exactly OPS vector-memory operations, so "at most kWeightAhead*OPS
-      // outstanding" always means the weight tile of the next step has landed.
 #pragma unroll
-      for (int v = -1 - kGatherAhead; v < -1; ++v) {
-        issue_gather(gv[v + 1 + kGatherAhead], gw[v + 1 + kGatherAhead]);
-        if (v + 1 + kWeightAhead >= 0) issue_weights(v + 1 + kWeightAhead);
-      }
-      commit(0, gv[0], gw[0]);
-      issue_gather(gv[0], gw[0]);
-      issue_weights(kWeightAhead);
-      MDCN_BARRIER(kWeightAhead * OPS);  // B1: X[0], W[0] visible
+      for (int j = 0; j < kGatherAhead; ++j) issue_gather(gv[j], gw[j]);
+      commit_and_refill(0, gv[0], gw[0]);
+      MDCN_BARRIER_LDS();  // B1: X[0] (and the consumers' W[0]) visible
 
       // The step loop runs in whole rounds of kGatherAhead steps (register sets are
       // addressed statically and the body stays branch-free, so the compiler's
@@ -507,15 +507,13 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
 #pragma unroll
         for (int j = 0; j < kGatherAhead; ++j) {
           const int ks = ks0 + j;
-          const int set = (j + 1) % kGatherAhead;  // holds step ks + 1
-          commit((ks + 1) & 1, gv[set], gw[set]);
-          issue_gather(gv[set], gw[set]);          // step ks + 1 + kGatherAhead
-          issue_weights(ks + 1 + kWeightAhead);
-          MDCN_BARRIER(kWeightAhead * OPS);  // end of step ks: X[ks+1], W[ks+1] visible
+          const int set = (j + 1) % kGatherAhead;  // holds step ks + 1, refilled with ks + 1 + kGatherAhead
+          commit_and_refill((ks + 1) & 1, gv[set], gw[set]);
+          MDCN_BARRIER_LDS();  // end of step ks: X[ks+1] visible
         }
       }
-      MDCN_BARRIER(0);      // E0: copies issued past the end have landed; consumers take tws
-      MDCN_BARRIER_LDS();   // E1: epilogue done, the table may be rebuilt
+      MDCN_BARRIER_LDS();   // E0: the tiles become the consumers' staging area
+      MDCN_BARRIER_LDS();   // E1: epilogue done, tiles and table may be rewritten
     } else {
       // =================== CONSUMER ===================
       const int wave_p = wave & 1;   // which 64 pixels
@@ -538,39 +536,68 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
         }
         cur.advance(nk, taps, spd);
       };
+      // Weight tile of step ks -> next ring slot, straight into LDS: lane i of
+      // copy c writes chunk c*64+i of the slot and reads the source chunk that
+      // the swizzle assigns to it.  The consumers issue these copies (they have
+      // the idle time); they are this wave's only vector-memory operations in
+      // the K loop, WDMA per step, so "at most kWeightAhead*WDMA outstanding"
+      // means the next step's tile has landed.
+      const unsigned char *wp_tile = (const unsigned char *)a.wp +
+                                     ((size_t)(grp * a.n_ctiles + ctile) * nk) * (size_t)(CT * kRowB);
+      uint32_t wlane[WDMA];  // byte offset of this lane's source chunk inside a tile
+#pragma unroll
+      for (int c = 0; c < WDMA; ++c) {
+        const int d = (wave * WDMA + c) * 64 + lane;
+        const int row = d >> 3;
+        wlane[c] = (uint32_t)(row * kRowB + (((d & 7) ^ swz(row)) * 16));
+      }
+      int islot = 0;  // ring slot of the next weight tile to issue
+      auto issue_weights = [&](int ks) {
+        const int kk = min(ks, nk - 1);  // past the end: repeat the last tile (never read)
+        const unsigned char *src = wp_tile + (size_t)kk * (CT * kRowB);
+#pragma unroll
+        for (int c = 0; c < WDMA; ++c) {
+          const int blk = wave * WDMA + c;  // 1 KiB block of the tile
+          copy16_global_to_lds(src + wlane[c], (uint32_t)(uintptr_t)(lptr_t)(&Ws[islot][blk * 64]));
+        }
+        islot = (islot == kWeightSlots - 1) ? 0 : islot + 1;
+      };
+
+      // (the previous tile's output stores are older than these copies, so the
+      // vmcnt waits below also cover them)
+#pragma unroll
+      for (int j = 0; j <= kWeightAhead; ++j) issue_weights(j);
       MDCN_BARRIER_LDS();  // B0
 #pragma unroll
       for (int v = 0; v <= kGatherAhead; ++v) mirror_issue();
-      MDCN_BARRIER_LDS();  // B1
+      MDCN_BARRIER(kWeightAhead * WDMA);  // B1: W[0] landed
 
+      int wslot = 0;
       for (int ks = 0; ks < nk_pad; ++ks) {
         const uint4 *X = Xs[ks & 1];
-        const uint4 *W = Ws[ks & (kWeightSlots - 1)];
+        const uint4 *W = Ws[wslot];
+        wslot = (wslot == kWeightSlots - 1) ? 0 : wslot + 1;
+        issue_weights(ks + 1 + kWeightAhead);
         if (ks < nk) {
 #pragma unroll
-        for (int ksub = 0; ksub < 2; ++ksub) {
-          const int ch = ksub * 2 + fhalf;
-          uint4 xf[NB], wf[MB];
+          for (int ksub = 0; ksub < 4; ++ksub) {
+            const int ch = ksub * 2 + fhalf;
+            uint4 xf[NB], wf[MB];
 #pragma unroll
-          for (int nb = 0; nb < NB; ++nb) {
-            const int row = wave_p * 64 + nb * 32 + frow;
-            xf[nb] = X[row * 4 + (ch ^ ((row >> 2) & 3))];
+            for (int nb = 0; nb < NB; ++nb) xf[nb] = X[tile_chunk(wave_p * 64 + nb * 32 + frow, ch)];
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+              wf[mb] = W[tile_chunk(wave_c * (CT / 2) + mb * 32 + frow, ch)];
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+              for (int mb = 0; mb < MB; ++mb) TR::mma(acc[nb][mb], xf[nb], wf[mb]);
           }
-#pragma unroll
-          for (int mb = 0; mb < MB; ++mb) {
-            const int row = wave_c * (CT / 2) + mb * 32 + frow;
-            wf[mb] = W[row * 4 + (ch ^ ((row >> 2) & 3))];
-          }
-#pragma unroll
-          for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-            for (int mb = 0; mb < MB; ++mb) TR::mma(acc[nb][mb], xf[nb], wf[mb]);
-        }
         }
         mirror_issue();
-        MDCN_BARRIER_LDS();  // end of step ks
+        MDCN_BARRIER(kWeightAhead * WDMA);  // end of step ks: W[ks+1] landed
       }
-      MDCN_BARRIER_LDS();  // E0
+      MDCN_BARRIER(0);  // E0: copies issued past the end have landed; tiles become staging
 
       // ---- epilogue: bias, round once, transpose through LDS, NCHW store ----
       // Accumulator block (A = samples, B = weights): register r of lane l holds
@@ -578,7 +605,8 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
       constexpr int RB = stage_row_bytes<E>();
       constexpr int CHUNK_PX = 16 / ES;           // pixels per 16-byte chunk
       constexpr int CHUNKS = 64 / CHUNK_PX;       // chunks per staged row
-      unsigned char *stage = (unsigned char *)tws + (size_t)wave * 32 * RB;
+      unsigned char *stage = (wave < 2 ? (unsigned char *)&Xs[0][0] : (unsigned char *)&Ws[0][0]) +
+                             (size_t)(wave & 1) * 32 * RB;
       E *out = (E *)a.out;
       const int pw0 = p0 + wave_p * 64;           // first pixel of this wave
       const bool vec_ok = a.out_vec_ok != 0;      // 16-byte chunks never straddle images, aligned

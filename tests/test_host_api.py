@@ -68,21 +68,24 @@ def test_eligibility_and_workspace():
     ws = lib.mdcn_workspace_bytes(ctypes.byref(p))
     assert ws >= 16 * 102 * 154 * 256 * 2 + 256 * 256 * 9 * 2
     assert ws < 1.02 * (16 * 102 * 154 * 256 * 2 + 256 * 256 * 9 * 2) + 4096
-    # fp32 needs Cin/groups and Cin/deform_groups to be multiples of 16, 16-bit of 32
-    p = capi.make_params(capi.MDCN_F32, 1, 16, 8, 8, 4, 3, 3)
+    # a K step is 128 bytes of channels: Cin/groups and Cin/deform_groups must be
+    # multiples of 32 (fp32) resp. 64 (fp16, bf16)
+    p = capi.make_params(capi.MDCN_F32, 1, 32, 8, 8, 4, 3, 3)
     assert lib.mdcn_fused_eligible(ctypes.byref(p)) == 1
-    p = capi.make_params(capi.MDCN_F16, 1, 16, 8, 8, 4, 3, 3)
+    p = capi.make_params(capi.MDCN_F16, 1, 32, 8, 8, 4, 3, 3)
     assert lib.mdcn_fused_eligible(ctypes.byref(p)) == 0
-    p = capi.make_params(capi.MDCN_F32, 1, 64, 8, 8, 4, 3, 3, deform_groups=8)
+    p = capi.make_params(capi.MDCN_F32, 1, 64, 8, 8, 4, 3, 3, deform_groups=4)
     assert lib.mdcn_fused_eligible(ctypes.byref(p)) == 0
     assert lib.mdcn_workspace_bytes(ctypes.byref(p)) == 0
+    p = capi.make_params(capi.MDCN_F32, 1, 64, 8, 8, 4, 6, 6)  # 36 taps exceed the table
+    assert lib.mdcn_fused_eligible(ctypes.byref(p)) == 0
     p.path = capi.PATH_DIRECT
     assert lib.mdcn_workspace_bytes(ctypes.byref(p)) == 0
 
 
 def test_forward_rejects_bad_calls_before_touching_the_device():
     lib = capi.load()
-    p = capi.make_params(capi.MDCN_F32, 1, 16, 8, 8, 4, 3, 3, (1, 1), (1, 1))
+    p = capi.make_params(capi.MDCN_F32, 1, 32, 8, 8, 4, 3, 3, (1, 1), (1, 1))
     assert lib.mdcn_forward(ctypes.byref(p), None) == -1  # null tensors
     buf = ctypes.create_string_buffer(64)
     addr = ctypes.addressof(buf)
