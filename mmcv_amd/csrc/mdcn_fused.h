@@ -528,6 +528,15 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
 
       const int frow = lane & 31;
       const int fhalf = lane >> 5;
+      // bias of this lane's output channels, fetched now so that the epilogue
+      // never waits on a load (a wait there would also wait for its own stores)
+      float bv[MB];
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        const int mycol = ctile * CT + wave_c * (CT / 2) + mb * 32 + frow;
+        bv[mb] = 0.0f;
+        if (a.bias && mycol < g.cout_g) bv[mb] = to_f32(((const E *)a.bias)[grp * g.cout_g + mycol]);
+      }
       // mirror of the producers' issue sequence, for the table-rebuild barriers
       auto mirror_issue = [&]() {
         if (MULTI_DG && cur.new_dg) {
@@ -613,17 +622,14 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
         const int col0 = ctile * CT + wave_c * (CT / 2) + mb * 32;  // channel within the group
-        const int mycol = col0 + frow;
-        float bv = 0.0f;
-        if (a.bias && mycol < g.cout_g) bv = to_f32(((const E *)a.bias)[grp * g.cout_g + mycol]);
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
 #pragma unroll
           for (int r4 = 0; r4 < 4; ++r4) {
             const int px = nb * 32 + r4 * 8 + fhalf * 4;
-            TR::store4(stage + frow * RB + px * ES, acc[nb][mb][r4 * 4 + 0] + bv,
-                       acc[nb][mb][r4 * 4 + 1] + bv, acc[nb][mb][r4 * 4 + 2] + bv,
-                       acc[nb][mb][r4 * 4 + 3] + bv);
+            TR::store4(stage + frow * RB + px * ES, acc[nb][mb][r4 * 4 + 0] + bv[mb],
+                       acc[nb][mb][r4 * 4 + 1] + bv[mb], acc[nb][mb][r4 * 4 + 2] + bv[mb],
+                       acc[nb][mb][r4 * 4 + 3] + bv[mb]);
           }
         }
         // the same wave wrote and now reads: only its own LDS operations matter
