@@ -5,64 +5,89 @@
 
 namespace mdcn {
 
-// NCHW input -> zero-bordered slab-major copy xt[N][Cin/KC][H+2][W+2][KC]
-// (KC channels = 64 bytes per pixel and slab).  The one-pixel zero border makes
+// NCHW input -> zero-bordered slab-major copy xt[N][Cin/KC][H+2][W+2][KC], KC =
+// 128 bytes of channels per pixel and slab.  The one-pixel zero border makes
 // every bilinear corner of an in-range position a plain load: a corner outside
 // the image reads a stored zero, which is exactly the per-corner rule of the
 // reference sampler (mmcv/ops/csrc/pytorch/cpu/modulated_deform_conv.cpp:17-27).
 //
-// One block moves a 64-channel x 64-column tile of one padded row through LDS:
-// reads run along W (contiguous in NCHW), writes along the KC channels of a
-// pixel and on to the next pixel (contiguous in xt).
-template <typename E, int KC>
-__global__ __launch_bounds__(256) void relayout_kernel(
-    Geom g, const E *__restrict__ in, E *__restrict__ xt, int n_xtiles,
-    int n_ctiles) {
-  __shared__ E tile[64][65];
+// One block moves one slab of 128 consecutive pixels of one padded row through
+// LDS.  Reads run along W in 32-bit words (two 16-bit pixels or one fp32 pixel,
+// a wave takes 256 contiguous bytes of one channel row); writes are 16 bytes per
+// lane, a wave covering 1 KiB of contiguous output.  The block's pixels are
+// padded columns 1+128*xc .. 128+128*xc, i.e. source columns 128*xc .. , so the
+// word reads are aligned; column 0 of the border is written by block xc == 0.
+template <typename E>
+__global__ __launch_bounds__(256) void relayout_kernel(Geom g, const E *__restrict__ in,
+                                                       E *__restrict__ xt, int n_xchunks,
+                                                       int words_ok) {
+  constexpr int KC = 128 / (int)sizeof(E);
+  constexpr int EPW = 4 / (int)sizeof(E);   // elements per 32-bit word
+  constexpr int ROWW = 33;                  // LDS words per pixel: 128 bytes + 4 of padding
+  __shared__ uint32_t tile[128 * ROWW];
+
   int b = blockIdx.x;
-  const int xtile = b % n_xtiles;
-  b /= n_xtiles;
-  const int ctile = b % n_ctiles;
-  b /= n_ctiles;
+  const int xc = b % n_xchunks;
+  b /= n_xchunks;
+  const int slabs_total = g.Cin / KC;
+  const int slab = b % slabs_total;
+  b /= slabs_total;
   const int yp = b % g.Hp;
   const int n = b / g.Hp;
-  const int slabs_total = g.Cin / KC;
 
   const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
   const bool row_inside = (yp >= 1) && (yp <= g.H);
-  {
-    const int xl = tid & 63;
-    const int xp = xtile * 64 + xl;
-    const bool col_inside = (xp >= 1) && (xp <= g.W);
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int cl = (tid >> 6) + 4 * i;
-      const int c = ctile * 64 + cl;
-      E v = from_f32<E>(0.0f);
-      if (row_inside && col_inside && c < g.Cin)
-        v = in[(((long)n * g.Cin + c) * g.H + (yp - 1)) * g.W + (xp - 1)];
-      tile[cl][xl] = v;
-    }
-  }
-  __syncthreads();
-  {
-    // lanes run over the KC channels of a slab, then over pixels
-    const int kc = tid % KC;
-    constexpr int PX_PER_PASS = 256 / KC;
-#pragma unroll
-    for (int sl = 0; sl < 64 / KC; ++sl) {
-      const int cl = sl * KC + kc;
-      const int c = ctile * 64 + cl;
-      const int slab = c / KC;
-#pragma unroll
-      for (int i = 0; i < 64 / PX_PER_PASS; ++i) {
-        const int xl = tid / KC + PX_PER_PASS * i;
-        const int xp = xtile * 64 + xl;
-        if (xp < g.Wp && c < g.Cin)
-          xt[((((long)n * slabs_total + slab) * g.Hp + yp) * g.Wp + xp) * KC + kc] = tile[cl][xl];
+
+  if (row_inside) {
+    // 64 row segments (KC channels x 128/(64*EPW) parts), 16 per wave
+#pragma unroll 4
+    for (int it = 0; it < 16; ++it) {
+      const int seg = wave + 4 * it;
+      const int c = seg % KC;
+      const int part = seg / KC;                      // fp32: two halves of 64 pixels
+      const int lp = (part * 64 + lane) * EPW;        // first local pixel of the word
+      const int x = xc * 128 + lp;
+      const E *src = in + (((long)n * g.Cin + slab * KC + c) * g.H + (yp - 1)) * g.W + x;
+      if (EPW == 2) {
+        uint32_t word = 0;
+        if (words_ok) {
+          if (x < g.W) word = *(const uint32_t *)src;  // W even: x + 1 < W too
+        } else {
+          uint32_t lo = 0, hi = 0;
+          if (x < g.W) lo = *(const uint16_t *)src;
+          if (x + 1 < g.W) hi = *((const uint16_t *)src + 1);
+          word = lo | (hi << 16);
+        }
+        uint16_t *t16 = (uint16_t *)tile;
+        t16[lp * (ROWW * 2) + c] = (uint16_t)(word & 0xffffu);
+        t16[(lp + 1) * (ROWW * 2) + c] = (uint16_t)(word >> 16);
+      } else {
+        uint32_t word = 0;
+        if (x < g.W) word = *(const uint32_t *)src;
+        tile[lp * ROWW + c] = word;
       }
     }
   }
+  __syncthreads();
+  unsigned char *dst_row =
+      (unsigned char *)xt + ((((long)n * slabs_total + slab) * g.Hp + yp) * g.Wp) * 128;
+#pragma unroll
+  for (int it = 0; it < 4; ++it) {
+    const int u = tid + 256 * it;
+    const int lp = u >> 3, q = u & 7;
+    const int xp = xc * 128 + 1 + lp;
+    if (xp < g.Wp) {
+      uint4 v = make_uint4(0u, 0u, 0u, 0u);
+      if (row_inside) {
+        const uint32_t *t = tile + lp * ROWW + q * 4;
+        v = make_uint4(t[0], t[1], t[2], t[3]);
+      }
+      *(uint4 *)(dst_row + (long)xp * 128 + q * 16) = v;
+    }
+  }
+  if (xc == 0 && tid < 8) *(uint4 *)(dst_row + tid * 16) = make_uint4(0u, 0u, 0u, 0u);
 }
 
 // weight[Cout][Cin/G][kh][kw] -> wp[G][n_ctiles][nk][CT][KC]: for every
