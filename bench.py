@@ -87,6 +87,9 @@ def main():
     ap.add_argument('--warmup', type=int, default=10)
     ap.add_argument('--workload', default='cfg4', choices=sorted(WORKLOADS))
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
+    ap.add_argument('--copy-probe', action='store_true',
+                    help='run a plain elementwise copy of known size instead (calibrates the '
+                         'FETCH_SIZE / WRITE_SIZE counters) and exit')
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
         log('bench.py: this path is built and measured on ONE GPU; '
@@ -95,6 +98,16 @@ def main():
         sys.exit(2)
 
     import torch
+    if a.copy_probe:
+        # 256 MiB read + 256 MiB written per launch by one elementwise kernel
+        src = torch.ones(128 * 1024 * 1024, dtype=torch.bfloat16, device='cuda')
+        dst = torch.empty_like(src)
+        for _ in range(a.steps):
+            torch.add(src, 1, out=dst)
+        torch.cuda.synchronize()
+        print(json.dumps({'copy_probe_bytes_read': src.numel() * 2,
+                          'copy_probe_bytes_written': dst.numel() * 2, 'launches': a.steps}))
+        return
     from common import make_case, cast_case
     from mmcv_amd.ops.modulated_deform_conv import ext_module
 
@@ -184,7 +197,9 @@ def main():
             'peak': peak,
             'unit': 'TFLOP/s',
             'frac': round(achieved / peak, 4),
-            'traffic': None,
+            # HBM bytes per launch of the fused kernel on cfg4/bf16 from rocprofv3 FETCH_SIZE and
+            # WRITE_SIZE, scaled by a copy kernel (profiles/fused_kernel_bf16_cfg4.md)
+            'traffic': 397.8e6 if a.workload == 'cfg4' else None,
         },
     }
     if not a.no_cpu:
