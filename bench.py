@@ -80,12 +80,85 @@ def cpu_baseline(case, flops_per_sample, budget_s=20.0):
     }
 
 
+# cfg 5: DCNv2 ResNet-50 stages c3-c5 at an 800x1344 image scale, batch 16, bf16:
+# (stage, channels, layers, input HxW of the first layer, output HxW)
+CFG5_STAGES = [('c3', 128, 4, (200, 336), (100, 168)),
+               ('c4', 256, 6, (100, 168), (50, 84)),
+               ('c5', 512, 3, (50, 84), (25, 42))]
+
+
+def cfg5_layers():
+    """The 13 deformable 3x3 convs: (name, C, (Hin, Win), stride)."""
+    layers = []
+    for name, c, n, hw_in, hw_out in CFG5_STAGES:
+        for i in range(n):
+            layers.append((f'{name}.{i}', c, hw_in if i == 0 else hw_out, 2 if i == 0 else 1))
+    return layers
+
+
+def run_cfg5(a):
+    """Per-layer and summed ms of the 13 layers.  Offsets and mask come from a
+    default-initialised 3x3 conv on the layer input (not the Pack's zero
+    initialisation, which would make every offset 0), then chunk/cat/sigmoid as
+    in ModulatedDeformConv2dPack.forward; that producer is timed separately."""
+    import torch
+    from mmcv_amd.ops import ModulatedDeformConv2dPack
+    from mmcv_amd.ops.modulated_deform_conv import ext_module
+    torch.manual_seed(20245)
+    N = 16
+    rows, tot_dcn, tot_prod, tot_flops, tot_pack = [], 0.0, 0.0, 0.0, 0.0
+    ev = lambda: torch.cuda.Event(enable_timing=True)
+    for name, C, (H, W), stride in cfg5_layers():
+        layer = ModulatedDeformConv2dPack(C, C, 3, stride=stride, padding=1, deform_groups=1)
+        torch.nn.Conv2d.reset_parameters(layer.conv_offset)
+        layer = layer.cuda().bfloat16()
+        x = torch.randn(N, C, H, W, device='cuda').bfloat16()
+        with torch.no_grad():
+            def producer():
+                raw = layer.conv_offset(x)
+                o1, o2, m = torch.chunk(raw, 3, dim=1)
+                return torch.cat((o1, o2), dim=1), torch.sigmoid(m)
+            off, msk = producer()
+            Ho, Wo = off.shape[2:]
+            out = torch.empty(N, C, Ho, Wo, dtype=torch.bfloat16, device='cuda')
+            empty = x.new_empty(0)
+            kw = dict(kernel_h=3, kernel_w=3, stride_h=stride, stride_w=stride, pad_h=1, pad_w=1,
+                      dilation_h=1, dilation_w=1, group=1, deformable_group=1, with_bias=True)
+            dcn = lambda: ext_module.modulated_deform_conv_forward(
+                x, layer.weight, layer.bias, empty, off, msk, out, empty, **kw)
+            pack = lambda: layer(x)   # one extension call: conv_offset + split + sigmoid + DCN
+            t = []
+            for fn in (producer, dcn, pack):
+                for _ in range(a.warmup):
+                    fn()
+                torch.cuda.synchronize()
+                e0, e1 = ev(), ev()
+                e0.record()
+                for _ in range(a.steps):
+                    fn()
+                e1.record()
+                torch.cuda.synchronize()
+                t.append(e0.elapsed_time(e1) / a.steps)
+        flops = 2.0 * N * Ho * Wo * C * C * 9
+        rows.append({'layer': name, 'C': C, 'in': [H, W], 'stride': stride,
+                     'producer_ms': round(t[0], 4), 'dcn_ms': round(t[1], 4),
+                     'dcn_TFLOPs': round(flops / t[1] / 1e9, 1), 'pack_fused_ms': round(t[2], 4)})
+        log(rows[-1])
+        tot_prod += t[0]
+        tot_dcn += t[1]
+        tot_pack += t[2]
+        tot_flops += flops
+        del x, off, msk, out, layer
+        torch.cuda.empty_cache()
+    return rows, tot_dcn, tot_prod, tot_flops, tot_pack
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=50)
     ap.add_argument('--warmup', type=int, default=10)
-    ap.add_argument('--workload', default='cfg4', choices=sorted(WORKLOADS))
+    ap.add_argument('--workload', default='cfg4', choices=sorted(WORKLOADS) + ['cfg5'])
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     ap.add_argument('--copy-probe', action='store_true',
                     help='run a plain elementwise copy of known size instead (calibrates the '
@@ -107,6 +180,22 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({'copy_probe_bytes_read': src.numel() * 2,
                           'copy_probe_bytes_written': dst.numel() * 2, 'launches': a.steps}))
+        return
+    if a.workload == 'cfg5':
+        assert torch.cuda.is_available(), 'bench.py needs a GPU'
+        rows, tot_dcn, tot_prod, tot_flops, tot_pack = run_cfg5(a)
+        print(json.dumps({
+            'metric': 'DCNv2 fwd summed ms over 13 layers (ResNet-50 c3-c5, N=16, 800x1344 scale, bf16)',
+            'value': round(tot_dcn, 4), 'unit': 'ms', 'n_gpus': 1, 'steps': a.steps,
+            'warmup': a.warmup, 'ms_per_step': round(tot_dcn, 4), 'higher_is_better': False,
+            'scaling': 'weak', 'vs_baseline': None, 'dtype': 'bf16', 'data': 'synthetic',
+            'config': {'workload': 'cfg5: 13 DCNv2 3x3 layers, c3 4x128ch@100x168, c4 6x256ch@50x84, '
+                                   'c5 3x512ch@25x42, first layer of each stage stride 2'},
+            'dcn_TFLOPs': round(tot_flops / tot_dcn / 1e9, 1),
+            'pct_mfma_peak': round(100.0 * tot_flops / tot_dcn / 1e9 / PEAK_TFLOPS['bf16'], 2),
+            'offset_mask_producer_ms': round(tot_prod, 4),
+            'summed_ms_with_producer': round(tot_dcn + tot_prod, 4),
+            'summed_ms_pack_fused': round(tot_pack, 4), 'layers': rows}), flush=True)
         return
     from common import make_case, cast_case
     from mmcv_amd.ops.modulated_deform_conv import ext_module

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define MDCN_ABI_VERSION 1
+#define MDCN_ABI_VERSION 2
 
 /* Element type of every tensor of a call (the Python wrapper unifies them to
  * offset's dtype, mmcv/ops/modulated_deform_conv.py:136-139). */
@@ -110,6 +110,48 @@ int mdcn_forward(const mdcn_params *p, void *hip_stream);
  *   ms[0] input re-layout, ms[1] weight repack, ms[2] main kernel, ms[3] total.
  * Stages a path does not run report 0.  For measurement only. */
 int mdcn_forward_timed(const mdcn_params *p, void *hip_stream, float ms[4]);
+
+/*
+ * The deformable convolution together with the step in front of it in
+ * ModulatedDeformConv2dPack.forward (mmcv/ops/modulated_deform_conv.py:327-335):
+ *
+ *   raw    = conv_offset(x)                 plain conv, Cin -> 3*dgroups*kh*kw channels,
+ *                                           kernel/stride/padding/dilation of the DCN (:297-305)
+ *   o1, o2, m = chunk(raw, 3, dim=1);  offset = cat(o1, o2);  mask = sigmoid(m)
+ *   y      = modulated_deform_conv2d(x, offset, mask, weight, bias, ...)
+ *
+ * `conv` describes the deformable convolution as for mdcn_forward(); its
+ * `offset` and `mask` fields are not read.  The offsets are channels
+ * [0, 2*dgroups*kh*kw) of raw as they lie and the mask is the sigmoid of the
+ * remaining channels, taken while the kernel reads them, so chunk, cat and
+ * sigmoid cost no pass over memory.  Two modes:
+ *   offset_weight != NULL: conv_offset runs here as well, on the re-laid-out
+ *       input copy the main kernel uses.  offset_weight is
+ *       (3*dgroups*kh*kw, Cin, kh, kw), offset_bias (3*dgroups*kh*kw) or NULL.
+ *       `raw`, when not NULL, receives the conv_offset output, dense
+ *       (N, 3*dgroups*kh*kw, Ho, Wo); NULL keeps it in the workspace only.
+ *   offset_weight == NULL: `raw` is an input, the dense conv_offset output
+ *       computed by the caller.
+ * raw is rounded to `dtype` before it is used and so is the sigmoid, as in the
+ * reference's sequence of tensor operations.
+ */
+typedef struct mdcn_pack_params {
+  mdcn_params conv;
+  const void *offset_weight;
+  const void *offset_bias;
+  void *raw;
+} mdcn_pack_params;
+
+/* Bytes of device scratch mdcn_pack_forward() needs (conv.workspace must hold
+ * that many); 0 for an invalid *p. */
+size_t mdcn_pack_workspace_bytes(const mdcn_pack_params *p);
+
+/* Enqueue the pack-level forward on `hip_stream`.  Returns an mdcn_status. */
+int mdcn_pack_forward(const mdcn_pack_params *p, void *hip_stream);
+
+/* mdcn_pack_forward() with per-stage times: ms[0] input re-layout, ms[1] weight
+ * repacks, ms[2] main kernel, ms[3] total, ms[4] conv_offset.  For measurement only. */
+int mdcn_pack_forward_timed(const mdcn_pack_params *p, void *hip_stream, float ms[5]);
 
 #ifdef __cplusplus
 }

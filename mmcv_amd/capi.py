@@ -15,7 +15,8 @@ MDCN_OK = 0
 
 EXPORTS = ('mdcn_abi_version', 'mdcn_status_string', 'mdcn_output_size',
            'mdcn_fused_eligible', 'mdcn_workspace_bytes', 'mdcn_forward',
-           'mdcn_forward_timed')
+           'mdcn_forward_timed', 'mdcn_pack_workspace_bytes', 'mdcn_pack_forward',
+           'mdcn_pack_forward_timed')
 
 
 class MdcnParams(ctypes.Structure):
@@ -26,6 +27,11 @@ class MdcnParams(ctypes.Structure):
                 [(n, ctypes.c_int32) for n in
                  ('dtype', 'path', 'N', 'Cin', 'H', 'W', 'Cout', 'kh', 'kw',
                   'sh', 'sw', 'ph', 'pw', 'dh', 'dw', 'groups', 'dgroups')])
+
+
+class MdcnPackParams(ctypes.Structure):
+    _fields_ = [('conv', MdcnParams), ('offset_weight', ctypes.c_void_p),
+                ('offset_bias', ctypes.c_void_p), ('raw', ctypes.c_void_p)]
 
 
 _lib = None
@@ -53,6 +59,14 @@ def load():
         lib.mdcn_forward_timed.restype = ctypes.c_int
         lib.mdcn_forward_timed.argtypes = [P, ctypes.c_void_p,
                                            ctypes.POINTER(ctypes.c_float)]
+        PP = ctypes.POINTER(MdcnPackParams)
+        lib.mdcn_pack_workspace_bytes.restype = ctypes.c_size_t
+        lib.mdcn_pack_workspace_bytes.argtypes = [PP]
+        lib.mdcn_pack_forward.restype = ctypes.c_int
+        lib.mdcn_pack_forward.argtypes = [PP, ctypes.c_void_p]
+        lib.mdcn_pack_forward_timed.restype = ctypes.c_int
+        lib.mdcn_pack_forward_timed.argtypes = [PP, ctypes.c_void_p,
+                                                ctypes.POINTER(ctypes.c_float)]
         _lib = lib
     return _lib
 

@@ -169,6 +169,107 @@ std::vector<double> modulated_deform_conv_forward_timed(
   return {ms[0], ms[1], ms[2], ms[3]};
 }
 
+// ModulatedDeformConv2dPack.forward in one call
+// (mmcv/ops/modulated_deform_conv.py:327-335): conv_offset, the channel split,
+// the sigmoid and the deformable convolution.  `offset_weight` with zero
+// elements means that `raw` already holds the conv_offset output (computed by
+// the caller); otherwise conv_offset runs here and `raw`, when it has elements,
+// receives its output.  Returns per-stage milliseconds when `timed`.
+std::vector<double> modulated_deform_conv_pack_forward(
+    Tensor input, Tensor offset_weight, Tensor offset_bias, Tensor raw,
+    Tensor weight, Tensor bias, Tensor output, int kernel_h, int kernel_w,
+    int stride_h, int stride_w, int pad_h, int pad_w, int dilation_h,
+    int dilation_w, int group, int deformable_group, bool with_bias, bool timed) {
+  const char *op = "modulated_deform_conv_pack_forward";
+  TORCH_CHECK(input.dim() == 4 && weight.dim() == 4, op, " expects 4-D input and weight");
+  const at::Device dev = input.device();
+  TORCH_CHECK(dev.is_cuda(), op, ": implementation for device ", device_str(dev), " not found.");
+  c10::DeviceGuard guard(dev);
+  const int64_t batch = input.size(0), channels = input.size(1);
+  const int64_t channels_out = weight.size(0);
+  TORCH_CHECK(weight.size(2) == kernel_h && weight.size(3) == kernel_w,
+              "Input shape and kernel shape won't match: (", kernel_h, " x ", kernel_w,
+              " vs ", weight.size(2), " x ", weight.size(3), ").");
+  TORCH_CHECK(channels == weight.size(1) * group,
+              "Input shape and kernel channels won't match: (", channels, " vs ",
+              weight.size(1) * group, ").");
+  const bool own_conv = offset_weight.numel() > 0;
+  const auto st = input.scalar_type();
+  const Tensor *all[] = {&weight, &bias, &output, &offset_weight, &offset_bias, &raw};
+  const char *names[] = {"weight", "bias", "output", "offset_weight", "offset_bias", "raw"};
+  for (int i = 0; i < 6; ++i) {
+    if (all[i]->numel() == 0) continue;
+    TORCH_CHECK(all[i]->device() == dev, op, ": at param ", names[i], ", inconsistent device: ",
+                device_str(all[i]->device()), " vs ", device_str(dev));
+    TORCH_CHECK(all[i]->scalar_type() == st, op, ": expected ", names[i], " to have dtype ",
+                c10::toString(st), " but got ", c10::toString(all[i]->scalar_type()));
+  }
+
+  mdcn_pack_params pp{};
+  mdcn_params &p = pp.conv;
+  p.dtype = mdcn_dtype_of(input);
+  p.path = g_path;
+  p.N = (int)batch; p.Cin = (int)channels; p.H = (int)input.size(2); p.W = (int)input.size(3);
+  p.Cout = (int)channels_out; p.kh = kernel_h; p.kw = kernel_w;
+  p.sh = stride_h; p.sw = stride_w; p.ph = pad_h; p.pw = pad_w;
+  p.dh = dilation_h; p.dw = dilation_w;
+  p.groups = group; p.dgroups = deformable_group;
+  int32_t Ho = 0, Wo = 0;
+  int rc = mdcn_output_size(&p, &Ho, &Wo);
+  TORCH_CHECK(rc == MDCN_OK, op, ": ", mdcn_status_string(rc));
+  const int64_t co = (int64_t)3 * deformable_group * kernel_h * kernel_w;
+  TORCH_CHECK(output.numel() == batch * channels_out * Ho * Wo && output.is_contiguous(), op,
+              ": output must be a dense (", batch, ", ", channels_out, ", ", Ho, ", ", Wo,
+              ") tensor, got ", output.sizes());
+  if (own_conv) {
+    TORCH_CHECK(offset_weight.dim() == 4 && offset_weight.size(0) == co &&
+                    offset_weight.size(1) == channels && offset_weight.size(2) == kernel_h &&
+                    offset_weight.size(3) == kernel_w,
+                op, ": offset_weight must be (", co, ", ", channels, ", ", kernel_h, ", ",
+                kernel_w, "), got ", offset_weight.sizes());
+    TORCH_CHECK(offset_bias.numel() == 0 || offset_bias.numel() == co, op,
+                ": offset_bias must have ", co, " elements, got ", offset_bias.numel());
+  } else {
+    TORCH_CHECK(raw.numel() > 0, op, ": needs offset_weight or raw");
+  }
+  if (raw.numel() > 0)
+    TORCH_CHECK(raw.dim() == 4 && raw.size(0) == batch && raw.size(1) == co && raw.size(2) == Ho &&
+                    raw.size(3) == Wo && (own_conv ? raw.is_contiguous() : true),
+                op, ": raw must be a dense (", batch, ", ", co, ", ", Ho, ", ", Wo,
+                ") tensor, got ", raw.sizes());
+  if (with_bias)
+    TORCH_CHECK(bias.numel() == channels_out, op, ": bias must have ", channels_out,
+                " elements, got ", bias.numel());
+
+  std::vector<Tensor> keep;
+  auto dense = [&](const Tensor &t) {
+    keep.push_back(t.contiguous());
+    return keep.back().data_ptr();
+  };
+  p.input = dense(input);
+  p.weight = dense(weight);
+  p.bias = with_bias ? dense(bias) : nullptr;
+  p.output = output.data_ptr();
+  if (own_conv) {
+    pp.offset_weight = dense(offset_weight);
+    pp.offset_bias = offset_bias.numel() ? dense(offset_bias) : nullptr;
+    pp.raw = raw.numel() ? raw.data_ptr() : nullptr;
+  } else {
+    pp.raw = dense(raw);
+  }
+  const size_t ws = mdcn_pack_workspace_bytes(&pp);
+  if (ws > 0) {
+    keep.push_back(at::empty({(int64_t)ws}, input.options().dtype(at::kByte)));
+    p.workspace = keep.back().data_ptr();
+    p.workspace_bytes = ws;
+  }
+  void *stream = (void *)c10::hip::getCurrentHIPStream().stream();
+  float ms[5] = {0, 0, 0, 0, 0};
+  rc = timed ? mdcn_pack_forward_timed(&pp, stream, ms) : mdcn_pack_forward(&pp, stream);
+  TORCH_CHECK(rc == MDCN_OK, op, ": ", mdcn_status_string(rc));
+  return {ms[0], ms[1], ms[2], ms[3], ms[4]};
+}
+
 void modulated_deform_conv_backward(
     Tensor input, Tensor weight, Tensor bias, Tensor ones, Tensor offset,
     Tensor mask, Tensor columns, Tensor grad_input, Tensor grad_weight,
@@ -192,6 +293,13 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("pad_h"), py::arg("pad_w"), py::arg("dilation_h"),
         py::arg("dilation_w"), py::arg("group"), py::arg("deformable_group"),
         py::arg("with_bias"));
+  m.def("modulated_deform_conv_pack_forward", &modulated_deform_conv_pack_forward,
+        "conv_offset + chunk/cat/sigmoid + modulated deform conv forward", py::arg("input"),
+        py::arg("offset_weight"), py::arg("offset_bias"), py::arg("raw"), py::arg("weight"),
+        py::arg("bias"), py::arg("output"), py::arg("kernel_h"), py::arg("kernel_w"),
+        py::arg("stride_h"), py::arg("stride_w"), py::arg("pad_h"), py::arg("pad_w"),
+        py::arg("dilation_h"), py::arg("dilation_w"), py::arg("group"),
+        py::arg("deformable_group"), py::arg("with_bias"), py::arg("timed") = false);
   m.def("modulated_deform_conv_backward", &modulated_deform_conv_backward,
         "modulated deform conv backward", py::arg("input"), py::arg("weight"),
         py::arg("bias"), py::arg("ones"), py::arg("offset"), py::arg("mask"),

@@ -10,6 +10,7 @@
 #include "mdcn_common.h"
 #include "mdcn_direct.h"
 #include "mdcn_fused.h"
+#include "mdcn_oconv.h"
 #include "mdcn_prepass.h"
 
 namespace {
@@ -25,7 +26,7 @@ inline size_t align_up(size_t v) { return (v + kAlign - 1) / kAlign * kAlign; }
 
 inline size_t elem_size(int dtype) { return dtype == MDCN_F32 ? 4 : 2; }
 
-int check_params(const mdcn_params *p, Geom *g, bool need_ptrs) {
+int check_params(const mdcn_params *p, Geom *g, bool need_ptrs, bool need_offsets = true) {
   if (!p) return MDCN_ERR_NULL;
   if (p->dtype != MDCN_F32 && p->dtype != MDCN_F16 && p->dtype != MDCN_BF16)
     return MDCN_ERR_DTYPE;
@@ -40,8 +41,8 @@ int check_params(const mdcn_params *p, Geom *g, bool need_ptrs) {
   if ((long)p->H + 2L * p->ph < (long)p->dh * (p->kh - 1) + 1 ||
       (long)p->W + 2L * p->pw < (long)p->dw * (p->kw - 1) + 1 || Ho <= 0 || Wo <= 0)
     return MDCN_ERR_SHAPE;
-  if (need_ptrs && (!p->input || !p->offset || !p->mask || !p->weight || !p->output))
-    return MDCN_ERR_NULL;
+  if (need_ptrs && (!p->input || !p->weight || !p->output)) return MDCN_ERR_NULL;
+  if (need_ptrs && need_offsets && (!p->offset || !p->mask)) return MDCN_ERR_NULL;
   g->N = p->N; g->Cin = p->Cin; g->H = p->H; g->W = p->W;
   g->Cout = p->Cout; g->kh = p->kh; g->kw = p->kw;
   g->sh = p->sh; g->sw = p->sw; g->ph = p->ph; g->pw = p->pw;
@@ -98,6 +99,16 @@ struct Plan {
   int n_chunk;       // images per launch of the fused path
   size_t xt_bytes;   // channels-last copy of one chunk
   size_t wp_bytes;   // packed weights
+  // pack-level call only
+  int CO, CO_pad;    // conv_offset channels: 3 * DG * taps, rounded up to 32
+  size_t owp_bytes;  // packed conv_offset weights (fused path, conv_offset run here)
+  size_t raw_bytes;  // conv_offset output kept in the workspace
+};
+
+// What a pack-level call adds to the plain one.
+struct PackExtra {
+  const void *offset_weight, *offset_bias;
+  void *raw;
 };
 
 int make_plan(const mdcn_params *p, const Geom &g, Plan *pl) {
@@ -105,7 +116,9 @@ int make_plan(const mdcn_params *p, const Geom &g, Plan *pl) {
   if (p->path == MDCN_PATH_FUSED && !ok) return MDCN_ERR_PATH;
   pl->fused = ok && p->path != MDCN_PATH_DIRECT;
   pl->CT = pl->KC = pl->n_ctiles = pl->slabs = pl->n_chunk = 0;
-  pl->xt_bytes = pl->wp_bytes = 0;
+  pl->xt_bytes = pl->wp_bytes = pl->owp_bytes = pl->raw_bytes = 0;
+  pl->CO = 3 * g.DG * g.taps;
+  pl->CO_pad = (pl->CO + 31) / 32 * 32;
   if (!pl->fused) return MDCN_OK;
   const size_t es = elem_size(p->dtype);
   pl->KC = slab_channels(p->dtype);
@@ -117,6 +130,39 @@ int make_plan(const mdcn_params *p, const Geom &g, Plan *pl) {
   pl->xt_bytes = align_up((size_t)img * pl->n_chunk);
   pl->wp_bytes = align_up((size_t)g.G * pl->n_ctiles * pl->slabs * g.taps * pl->CT * pl->KC * es);
   return MDCN_OK;
+}
+
+// Workspace of a pack-level call: [xt][wp][owp][raw] on the fused path, [raw] on
+// the direct one (nothing when the caller's own raw buffer serves).
+int make_pack_plan(const mdcn_pack_params *pp, const Geom &g, Plan *pl) {
+  const mdcn_params *p = &pp->conv;
+  const int rc = make_plan(p, g, pl);
+  if (rc != MDCN_OK) return rc;
+  const size_t es = elem_size(p->dtype);
+  const size_t plane = (size_t)g.Ho * g.Wo;
+  if (pp->offset_weight) {
+    if (pl->fused) {
+      if (pl->CO_pad > 128) {  // accumulator blocks of the conv_offset kernel
+        if (p->path == MDCN_PATH_FUSED) return MDCN_ERR_PATH;
+        pl->fused = false;
+        pl->xt_bytes = pl->wp_bytes = 0;
+      } else {
+        pl->owp_bytes = align_up((size_t)(g.Cin / pl->KC) * g.taps * 4 * (pl->CO_pad / 32) * 64 * 16);
+        pl->raw_bytes = align_up((size_t)pl->n_chunk * plane * pl->CO_pad * es);
+      }
+    }
+    if (!pl->fused && !pp->raw) pl->raw_bytes = align_up((size_t)g.N * pl->CO * plane * es);
+  }
+  return MDCN_OK;
+}
+
+template <typename E, int COF>
+hipError_t launch_oconv(const OconvArgs &oa, hipStream_t st) {
+  constexpr int PXF = COF == 1 ? 4 : (COF == 2 ? 2 : 1);
+  const long px_per_block = 4L * 32 * PXF;
+  const long blocks = (oa.total_px + px_per_block - 1) / px_per_block;
+  hipLaunchKernelGGL((oconv_kernel<E, COF, PXF>), dim3((unsigned)blocks), dim3(256), 0, st, oa);
+  return hipGetLastError();
 }
 
 template <typename E, int CT, int TMAX, bool MULTI_DG>
@@ -155,7 +201,7 @@ hipError_t launch_fused(const FusedArgs &fa, int CT, hipStream_t st) {
 
 template <typename E>
 int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t st,
-              float *ms) {
+              float *ms, const PackExtra *px) {
   hipEvent_t ev[2] = {nullptr, nullptr};
   auto tic = [&]() { if (ms) (void)hipEventRecord(ev[0], st); };
   auto toc = [&](int slot) {
@@ -168,6 +214,7 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
   };
   if (ms) {
     ms[0] = ms[1] = ms[2] = ms[3] = 0.f;
+    if (px) ms[4] = 0.f;
     if (hipEventCreate(&ev[0]) != hipSuccess || hipEventCreate(&ev[1]) != hipSuccess)
       return MDCN_ERR_LAUNCH;
   }
@@ -175,13 +222,40 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
   const size_t es = sizeof(E);
   const long plane_out = (long)g.Ho * g.Wo;
 
+  // the conv_offset output of a pack-level call as dense (N, CO, Ho, Wo)
+  auto nchw_raw_view = [&](const E *raw) {
+    OffMaskView v;
+    v.off = raw;
+    v.msk = raw + (long)2 * g.DG * g.taps * plane_out;
+    v.off_n = v.msk_n = (long)pl.CO * plane_out;
+    v.off_ch = v.msk_ch = plane_out;
+    v.off_px = v.msk_px = 1;
+    v.logit = 1;
+    return v;
+  };
+
   if (!pl.fused) {
+    OffMaskView om = dense_view(p->offset, p->mask, g);
+    if (px) {
+      E *raw = (E *)px->raw;
+      if (px->offset_weight) {
+        if (!raw) raw = (E *)p->workspace;
+        const long total = (long)g.N * pl.CO * plane_out;
+        const int grid = (int)std::min<long>((total + 255) / 256, 1L << 20);
+        tic();
+        hipLaunchKernelGGL(oconv_direct_kernel<E>, dim3(grid), dim3(256), 0, st, g,
+                           (const E *)p->input, (const E *)px->offset_weight,
+                           (const E *)px->offset_bias, raw, pl.CO, total);
+        if (hipGetLastError() != hipSuccess) rc = MDCN_ERR_LAUNCH;
+        toc(4);
+      }
+      om = nchw_raw_view(raw);
+    }
     const long total = (long)g.N * g.Cout * plane_out;
     const int grid = (int)std::min<long>((total + 255) / 256, 1L << 20);
     tic();
     hipLaunchKernelGGL(direct_kernel<E>, dim3(grid), dim3(256), 0, st, g,
-                       (const E *)p->input, (const E *)p->offset,
-                       (const E *)p->mask, (const E *)p->weight,
+                       (const E *)p->input, om, (const E *)p->weight,
                        (const E *)p->bias, (E *)p->output, total);
     if (hipGetLastError() != hipSuccess) rc = MDCN_ERR_LAUNCH;
     toc(2);
@@ -189,6 +263,10 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
     unsigned char *ws = (unsigned char *)p->workspace;
     E *xt = (E *)ws;
     E *wp = (E *)(ws + pl.xt_bytes);
+    E *owp = (E *)(ws + pl.xt_bytes + pl.wp_bytes);
+    E *raw_pm = (E *)(ws + pl.xt_bytes + pl.wp_bytes + pl.owp_bytes);
+    const bool own_oconv = px && px->offset_weight;
+    const int cof = pl.CO_pad / 32;
 
     // weights: once per call
     {
@@ -199,6 +277,13 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
                          (const E *)p->weight, wp, pl.CT, pl.KC, pl.n_ctiles,
                          pl.slabs, total);
       if (hipGetLastError() != hipSuccess) rc = MDCN_ERR_LAUNCH;
+      if (own_oconv) {
+        const long ototal = (long)(g.Cin / pl.KC) * g.taps * 4 * cof * 64 * (16 / (long)es);
+        const int ogrid = (int)std::min<long>((ototal + 255) / 256, 1L << 16);
+        hipLaunchKernelGGL(pack_offset_weight_kernel<E>, dim3(ogrid), dim3(256), 0, st, g,
+                           (const E *)px->offset_weight, owp, pl.CO, cof, ototal);
+        if (hipGetLastError() != hipSuccess) rc = MDCN_ERR_LAUNCH;
+      }
       toc(1);
     }
     for (int n0 = 0; n0 < g.N && rc == MDCN_OK; n0 += pl.n_chunk) {
@@ -221,8 +306,46 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
       fa.g = gc;
       fa.xt = xt;
       fa.wp = wp;
-      fa.offset = (const E *)p->offset + (size_t)n0 * g.DG * 2 * g.taps * plane_out;
-      fa.mask = (const E *)p->mask + (size_t)n0 * g.DG * g.taps * plane_out;
+      if (own_oconv) {
+        OconvArgs oa;
+        oa.g = gc;
+        oa.xt = xt;
+        oa.owp = owp;
+        oa.obias = px->offset_bias;
+        oa.raw = raw_pm;
+        oa.total_px = (long)gc.N * plane_out;
+        oa.CO = pl.CO;
+        oa.CO_pad = pl.CO_pad;
+        oa.slabs_total = g.Cin / pl.KC;
+        oa.plane_px = g.Hp * g.Wp;
+        tic();
+        hipError_t e = cof == 1 ? launch_oconv<E, 1>(oa, st)
+                     : cof == 2 ? launch_oconv<E, 2>(oa, st)
+                     : cof == 3 ? launch_oconv<E, 3>(oa, st)
+                                : launch_oconv<E, 4>(oa, st);
+        if (e != hipSuccess) rc = MDCN_ERR_LAUNCH;
+        if (px->raw) {
+          const long total = (long)gc.N * pl.CO * plane_out;
+          const int grid = (int)std::min<long>((total + 255) / 256, 1L << 20);
+          hipLaunchKernelGGL(raw_to_nchw_kernel<E>, dim3(grid), dim3(256), 0, st, raw_pm,
+                             (E *)px->raw + (size_t)n0 * pl.CO * plane_out, pl.CO, pl.CO_pad,
+                             plane_out, total);
+          if (hipGetLastError() != hipSuccess) rc = MDCN_ERR_LAUNCH;
+        }
+        toc(4);
+        // pixel-major: the values of one pixel are CO_pad consecutive elements
+        fa.om.off = raw_pm;
+        fa.om.msk = raw_pm + 2 * g.DG * g.taps;
+        fa.om.off_n = fa.om.msk_n = plane_out * pl.CO_pad;
+        fa.om.off_ch = fa.om.msk_ch = 1;
+        fa.om.off_px = fa.om.msk_px = pl.CO_pad;
+        fa.om.logit = 1;
+      } else if (px) {
+        fa.om = nchw_raw_view((const E *)px->raw + (size_t)n0 * pl.CO * plane_out);
+      } else {
+        fa.om = dense_view((const E *)p->offset + (size_t)n0 * g.DG * 2 * g.taps * plane_out,
+                           (const E *)p->mask + (size_t)n0 * g.DG * g.taps * plane_out, g);
+      }
       fa.bias = p->bias;
       fa.out = (E *)p->output + (size_t)n0 * g.Cout * plane_out;
       fa.total_px = (long)gc.N * plane_out;
@@ -239,31 +362,39 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
     }
   }
   if (ms) {
-    ms[3] = ms[0] + ms[1] + ms[2];
+    ms[3] = ms[0] + ms[1] + ms[2] + (px ? ms[4] : 0.f);
     (void)hipEventDestroy(ev[0]);
     (void)hipEventDestroy(ev[1]);
   }
   return rc;
 }
 
-int run(const mdcn_params *p, void *stream, float *ms) {
+int run(const mdcn_params *p, void *stream, float *ms, const mdcn_pack_params *pp = nullptr) {
   Geom g;
-  int rc = check_params(p, &g, true);
+  int rc = check_params(p, &g, true, pp == nullptr);
   if (rc != MDCN_OK) return rc;
   Plan pl;
-  rc = make_plan(p, g, &pl);
-  if (rc != MDCN_OK) return rc;
-  if (pl.fused) {
-    const size_t need = pl.xt_bytes + pl.wp_bytes;
-    if (!p->workspace || p->workspace_bytes < need ||
-        ((uintptr_t)p->workspace % kAlign) != 0)
-      return MDCN_ERR_WORKSPACE;
+  PackExtra px_store, *px = nullptr;
+  if (pp) {
+    if (!pp->offset_weight && !pp->raw) return MDCN_ERR_NULL;
+    rc = make_pack_plan(pp, g, &pl);
+    px_store.offset_weight = pp->offset_weight;
+    px_store.offset_bias = pp->offset_bias;
+    px_store.raw = pp->raw;
+    px = &px_store;
+  } else {
+    rc = make_plan(p, g, &pl);
   }
+  if (rc != MDCN_OK) return rc;
+  const size_t need = pl.xt_bytes + pl.wp_bytes + pl.owp_bytes + pl.raw_bytes;
+  if (need > 0 && (!p->workspace || p->workspace_bytes < need ||
+                   ((uintptr_t)p->workspace % kAlign) != 0))
+    return MDCN_ERR_WORKSPACE;
   hipStream_t st = (hipStream_t)stream;
   switch (p->dtype) {
-    case MDCN_F32: return run_typed<float>(p, g, pl, st, ms);
-    case MDCN_F16: return run_typed<f16_t>(p, g, pl, st, ms);
-    default: return run_typed<bf16_t>(p, g, pl, st, ms);
+    case MDCN_F32: return run_typed<float>(p, g, pl, st, ms, px);
+    case MDCN_F16: return run_typed<f16_t>(p, g, pl, st, ms, px);
+    default: return run_typed<bf16_t>(p, g, pl, st, ms, px);
   }
 }
 
@@ -317,6 +448,24 @@ int mdcn_forward(const mdcn_params *p, void *hip_stream) {
 int mdcn_forward_timed(const mdcn_params *p, void *hip_stream, float ms[4]) {
   if (!ms) return MDCN_ERR_NULL;
   return run(p, hip_stream, ms);
+}
+
+size_t mdcn_pack_workspace_bytes(const mdcn_pack_params *pp) {
+  Geom g;
+  if (!pp || check_params(&pp->conv, &g, false) != MDCN_OK) return 0;
+  Plan pl;
+  if (make_pack_plan(pp, g, &pl) != MDCN_OK) return 0;
+  return pl.xt_bytes + pl.wp_bytes + pl.owp_bytes + pl.raw_bytes;
+}
+
+int mdcn_pack_forward(const mdcn_pack_params *pp, void *hip_stream) {
+  if (!pp) return MDCN_ERR_NULL;
+  return run(&pp->conv, hip_stream, nullptr, pp);
+}
+
+int mdcn_pack_forward_timed(const mdcn_pack_params *pp, void *hip_stream, float ms[5]) {
+  if (!pp || !ms) return MDCN_ERR_NULL;
+  return run(&pp->conv, hip_stream, ms, pp);
 }
 
 }  // extern "C"

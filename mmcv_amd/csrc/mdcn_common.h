@@ -68,4 +68,39 @@ __device__ __forceinline__ TapSample make_tap_sample(int base_y, int base_x,
   return s;
 }
 
+// Where the offsets and the mask of one output pixel live, in elements: image n,
+// pixel rem = ho * Wo + wo, channel c sits at base + n * _n + rem * _px + c * _ch.
+// The reference op takes two dense NCHW tensors (_px = 1, _ch = Ho * Wo); the
+// pack-level entry points read both out of the one conv_offset output, whose
+// first 2/3 of the channels are the offsets (chunk + cat of
+// mmcv/ops/modulated_deform_conv.py:329-330 is the identity on them) and whose
+// last third holds the mask before the sigmoid (`logit`, :331).
+struct OffMaskView {
+  const void *off, *msk;
+  long off_n, msk_n;
+  long off_ch, msk_ch;
+  int off_px, msk_px;
+  int logit;
+};
+
+__host__ __device__ inline OffMaskView dense_view(const void *off, const void *msk, const Geom &g) {
+  OffMaskView v;
+  const long plane = (long)g.Ho * g.Wo;
+  v.off = off; v.msk = msk;
+  v.off_n = (long)g.DG * 2 * g.taps * plane; v.msk_n = (long)g.DG * g.taps * plane;
+  v.off_ch = plane; v.msk_ch = plane;
+  v.off_px = 1; v.msk_px = 1;
+  v.logit = 0;
+  return v;
+}
+
+// Mask value from the stored element; a logit goes through the sigmoid and is
+// rounded to the element type once, as torch.sigmoid on an E tensor does.
+template <typename E>
+__device__ __forceinline__ float mask_value(E raw, int logit) {
+  float m = to_f32(raw);
+  if (logit) m = to_f32(from_f32<E>(1.0f / (1.0f + expf(-m))));
+  return m;
+}
+
 }  // namespace mdcn

@@ -10,8 +10,7 @@ namespace mdcn {
 
 template <typename E>
 __global__ __launch_bounds__(256) void direct_kernel(
-    Geom g, const E *__restrict__ input, const E *__restrict__ offset,
-    const E *__restrict__ mask, const E *__restrict__ weight,
+    Geom g, const E *__restrict__ input, OffMaskView om, const E *__restrict__ weight,
     const E *__restrict__ bias, E *__restrict__ output, long total) {
   const long plane_out = (long)g.Ho * g.Wo;
   const long plane_in = (long)g.H * g.W;
@@ -29,15 +28,17 @@ __global__ __launch_bounds__(256) void direct_kernel(
       const int c = grp * g.cin_g + cl;
       const int dgi = c / g.ch_per_dg;
       const E *im = input + ((long)n * g.Cin + c) * plane_in;
-      const E *off = offset + ((long)n * g.DG + dgi) * 2 * g.taps * plane_out;
-      const E *msk = mask + ((long)n * g.DG + dgi) * g.taps * plane_out;
+      const E *off = (const E *)om.off + (long)n * om.off_n + pix * om.off_px +
+                     (long)(dgi * 2 * g.taps) * om.off_ch;
+      const E *msk = (const E *)om.msk + (long)n * om.msk_n + pix * om.msk_px +
+                     (long)(dgi * g.taps) * om.msk_ch;
       const E *wrow = weight + ((long)co * g.cin_g + cl) * g.taps;
       for (int i = 0; i < g.kh; ++i) {
         for (int j = 0; j < g.kw; ++j) {
           const int tap = i * g.kw + j;
-          const float dy = to_f32(off[(long)(2 * tap) * plane_out + pix]);
-          const float dx = to_f32(off[(long)(2 * tap + 1) * plane_out + pix]);
-          const float m = to_f32(msk[(long)tap * plane_out + pix]);
+          const float dy = to_f32(off[(long)(2 * tap) * om.off_ch]);
+          const float dx = to_f32(off[(long)(2 * tap + 1) * om.off_ch]);
+          const float m = mask_value<E>(msk[(long)tap * om.msk_ch], om.logit);
           const TapSample s =
               make_tap_sample(ho * g.sh - g.ph + i * g.dh,
                               wo * g.sw - g.pw + j * g.dw, dy, dx, m, g.H, g.W);

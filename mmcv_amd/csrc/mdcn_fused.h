@@ -53,8 +53,7 @@ struct FusedArgs {
   Geom g;
   const void *xt;      // zero-bordered slab-major input copy
   const void *wp;      // packed weights
-  const void *offset;
-  const void *mask;
+  OffMaskView om;      // offsets and mask of the images of this launch
   const void *bias;    // may be null
   void *out;
   long total_px;       // N * Ho * Wo
@@ -384,16 +383,18 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
       }
       auto build_table = [&](int dgi) {
         // (an invalid pixel reads the entries of pixel 0 of image 0 and stores zeros)
-        const E *off = (const E *)a.offset + ((long)tb_n * g.DG + dgi) * 2 * taps * plane_out + tb_rem;
-        const E *msk = (const E *)a.mask + ((long)tb_n * g.DG + dgi) * taps * plane_out + tb_rem;
+        const E *off = (const E *)a.om.off + (long)tb_n * a.om.off_n + (long)tb_rem * a.om.off_px +
+                       (long)(dgi * 2 * taps) * a.om.off_ch;
+        const E *msk = (const E *)a.om.msk + (long)tb_n * a.om.msk_n + (long)tb_rem * a.om.msk_px +
+                       (long)(dgi * taps) * a.om.msk_ch;
         // all loads first (unconditional, clamped), then the arithmetic
         E rdy[TPT], rdx[TPT], rm[TPT];
 #pragma unroll
         for (int i = 0; i < TPT; ++i) {
           const int tap = min((ptid >> 7) + 2 * i, taps - 1);
-          rdy[i] = off[(long)(2 * tap) * plane_out];
-          rdx[i] = off[(long)(2 * tap + 1) * plane_out];
-          rm[i] = msk[(long)tap * plane_out];
+          rdy[i] = off[(long)(2 * tap) * a.om.off_ch];
+          rdx[i] = off[(long)(2 * tap + 1) * a.om.off_ch];
+          rm[i] = msk[(long)tap * a.om.msk_ch];
         }
 #pragma unroll
         for (int i = 0; i < TPT; ++i) {
@@ -402,7 +403,7 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
             const int ti = tap / g.kw, tj = tap - ti * g.kw;
             const TapSample sm =
                 make_tap_sample(tb_ho * g.sh - g.ph + ti * g.dh, tb_wo * g.sw - g.pw + tj * g.dw,
-                                to_f32(rdy[i]), to_f32(rdx[i]), to_f32(rm[i]), g.H, g.W);
+                                to_f32(rdy[i]), to_f32(rdx[i]), mask_value<E>(rm[i], a.om.logit), g.H, g.W);
             // +1: coordinates in the zero-bordered copy (y0, x0 >= -1 when inside,
             // 0 with zero weights otherwise); slab 0 of image tb_n.
             int32_t pix = tb_n * a.slabs_total * a.plane_px + (sm.y0 + 1) * g.Wp + (sm.x0 + 1);
@@ -512,6 +513,12 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
           MDCN_BARRIER_LDS();  // end of step ks: X[ks+1] visible
         }
       }
+      // The gathers issued past the last step are never read.  Retire them with a
+      // wait the compiler can see: it tracks these loads' destination registers,
+      // carries that state round the tile loop into the consumer branch (it cannot
+      // know that a wave keeps its role) and would otherwise guard the consumers'
+      // registers with vmcnt waits that also wait for their in-flight weight copies.
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), other counters untouched
       MDCN_BARRIER_LDS();   // E0: the tiles become the consumers' staging area
       MDCN_BARRIER_LDS();   // E1: epilogue done, tiles and table may be rewritten
     } else {

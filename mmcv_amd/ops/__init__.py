@@ -1,11 +1,13 @@
 from .modulated_deform_conv import (ModulatedDeformConv2d,
                                     ModulatedDeformConv2dFunction,
                                     ModulatedDeformConv2dPack,
-                                    modulated_deform_conv2d)
+                                    modulated_deform_conv2d,
+                                    modulated_deform_conv2d_pack)
 from .registry import MODELS, build_conv_layer
 
 __all__ = [
     'ModulatedDeformConv2d', 'ModulatedDeformConv2dPack',
-    'ModulatedDeformConv2dFunction', 'modulated_deform_conv2d', 'MODELS',
+    'ModulatedDeformConv2dFunction', 'modulated_deform_conv2d',
+    'modulated_deform_conv2d_pack', 'MODELS',
     'build_conv_layer'
 ]

@@ -220,6 +220,43 @@ class ModulatedDeformConv2d(nn.Module):
                                        self.deform_groups)
 
 
+def modulated_deform_conv2d_pack(x, conv_offset, weight, bias, stride, padding,
+                                 dilation, groups, deform_groups, own_conv=True,
+                                 return_raw=False, timed=False):
+    """Forward of ``ModulatedDeformConv2dPack``
+    (mmcv/ops/modulated_deform_conv.py:327-335) as one extension call: the
+    offsets are the first two thirds of ``conv_offset``'s output channels as they
+    lie, the mask is the sigmoid of the last third, both read by the kernel
+    itself.  ``own_conv=False`` leaves ``conv_offset`` to torch.  No autograd."""
+    stride, padding, dilation = _pair(stride), _pair(padding), _pair(dilation)
+    cw, cb = conv_offset.weight, conv_offset.bias
+    x = x.type_as(cw)
+    weight = weight.type_as(x)
+    with_bias = bias is not None
+    bias = bias.type_as(x) if with_bias else x.new_empty(0)
+    output = x.new_empty(_conv_output_size(x, weight, stride, padding, dilation))
+    empty = x.new_empty(0)
+    if own_conv:
+        raw = x.new_empty((x.size(0), cw.size(0)) + tuple(output.shape[2:])) if return_raw else empty
+        ow, ob = cw, (cb if cb is not None else empty)
+    else:
+        with torch.no_grad():
+            raw = conv_offset(x)
+        ow = ob = empty
+    ms = ext_module.modulated_deform_conv_pack_forward(
+        x, ow.detach(), ob.detach(), raw, weight.detach(), bias.detach(), output,
+        kernel_h=weight.size(2), kernel_w=weight.size(3),
+        stride_h=stride[0], stride_w=stride[1], pad_h=padding[0], pad_w=padding[1],
+        dilation_h=dilation[0], dilation_w=dilation[1], group=groups,
+        deformable_group=deform_groups, with_bias=with_bias, timed=timed)
+    out = (output,)
+    if return_raw:
+        out += (raw,)
+    if timed:
+        out += (ms,)
+    return out[0] if len(out) == 1 else out
+
+
 @MODELS.register_module('DCNv2')
 class ModulatedDeformConv2dPack(ModulatedDeformConv2d):
     """DCNv2 that predicts its own offsets and mask with a zero-initialised
@@ -258,7 +295,22 @@ class ModulatedDeformConv2dPack(ModulatedDeformConv2d):
             self.conv_offset.weight.data.zero_()
             self.conv_offset.bias.data.zero_()
 
+    #: How much of ``forward`` runs inside the HIP library for device tensors
+    #: that need no gradient: ``'full'`` = conv_offset, channel split, sigmoid
+    #: and the deformable convolution in one extension call; ``'split'`` =
+    #: conv_offset by torch, the rest fused; ``'none'`` = the reference's
+    #: sequence of tensor operations.
+    fuse = 'full'
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:  # type: ignore
+        needs_grad = torch.is_grad_enabled() and (
+            x.requires_grad or any(p.requires_grad for p in self.parameters()))
+        if self.fuse != 'none' and x.is_cuda and x.dim() == 4 and not needs_grad \
+                and not torch.is_autocast_enabled():
+            return modulated_deform_conv2d_pack(
+                x, self.conv_offset, self.weight, self.bias, self.stride,
+                self.padding, self.dilation, self.groups, self.deform_groups,
+                own_conv=self.fuse == 'full')
         # first two thirds of conv_offset's channels are the offsets, the last
         # third the mask logits (:328-331)
         raw = self.conv_offset(x)

@@ -103,3 +103,104 @@ def capi_forward(case, path=capi.PATH_AUTO, timed=False):
     assert rc == 0, capi.status_string(rc)
     torch.cuda.synchronize()
     return out
+
+
+def make_pack_case(seed, N, Cin, Cout, H, W, k=3, stride=1, padding=1, dilation=1,
+                   groups=1, deform_groups=1, offset_std=0.05):
+    """Seeded fp32 CPU tensors of a Pack layer: input, conv_offset weight and
+    bias (random, so that offsets and mask are not trivial: the layer's own
+    zero initialisation would make it a plain convolution), weight, bias."""
+    kh, kw = pair(k)
+    g = torch.Generator().manual_seed(seed)
+    co = 3 * deform_groups * kh * kw
+    x = torch.randn(N, Cin, H, W, generator=g)
+    ow = torch.randn(co, Cin, kh, kw, generator=g) * offset_std
+    ob = torch.randn(co, generator=g) * 0.5
+    fan_in = Cin // groups * kh * kw
+    w = torch.randn(Cout, Cin // groups, kh, kw, generator=g) * math.sqrt(2.0 / fan_in)
+    b = torch.randn(Cout, generator=g) * 0.01
+    return dict(input=x, offset_weight=ow, offset_bias=ob, weight=w, bias=b,
+                stride=pair(stride), padding=pair(padding), dilation=pair(dilation),
+                groups=groups, deform_groups=deform_groups)
+
+
+def cast_pack_case(case, dtype, device=None):
+    out = dict(case)
+    for k in ('input', 'offset_weight', 'offset_bias', 'weight', 'bias'):
+        if out[k] is not None:
+            out[k] = out[k].to(dtype)
+            if device is not None:
+                out[k] = out[k].to(device)
+    return out
+
+
+def oracle_conv_offset(case):
+    """conv_offset on the CPU oracle: a deformable convolution with zero offsets
+    and unit mask is the plain convolution."""
+    x, ow = case['input'], case['offset_weight']
+    kh, kw = ow.shape[2:]
+    Ho, Wo = out_hw(x.shape[2], x.shape[3], kh, kw, case['stride'], case['padding'], case['dilation'])
+    N = x.shape[0]
+    zero = dict(input=x, offset=torch.zeros(N, 2 * kh * kw, Ho, Wo), mask=torch.ones(N, kh * kw, Ho, Wo),
+                weight=ow, bias=case['offset_bias'], stride=case['stride'], padding=case['padding'],
+                dilation=case['dilation'], groups=1, deform_groups=1)
+    return oracle_forward(zero)
+
+
+def split_raw(raw, deform_groups, taps):
+    """chunk / cat / sigmoid of ModulatedDeformConv2dPack.forward on a torch
+    tensor of any dtype (each step rounds to that dtype, as in the reference)."""
+    o1, o2, m = torch.chunk(raw, 3, dim=1)
+    return torch.cat((o1, o2), dim=1).contiguous(), torch.sigmoid(m).contiguous()
+
+
+def capi_pack_forward(case, own_conv=True, raw=None, want_raw=False, path=capi.PATH_AUTO, timed=False):
+    """mdcn_pack_forward through ctypes on device tensors; returns (output, raw
+    or None[, ms])."""
+    lib = capi.load()
+    x, w, b = case['input'], case['weight'], case['bias']
+    N, Cin, H, W = x.shape
+    Cout, _, kh, kw = w.shape
+    pp = capi.MdcnPackParams()
+    pp.conv = capi.make_params(DT[x.dtype], N, Cin, H, W, Cout, kh, kw, case['stride'],
+                               case['padding'], case['dilation'], case['groups'],
+                               case['deform_groups'], path)
+    p = pp.conv
+    rc, Ho, Wo = capi.output_size(p)
+    assert rc == 0, capi.status_string(rc)
+    co = 3 * case['deform_groups'] * kh * kw
+    out = torch.empty(N, Cout, Ho, Wo, dtype=x.dtype, device=x.device)
+    keep = [t.contiguous() for t in (x, w)]
+    p.input, p.weight = (t.data_ptr() for t in keep)
+    if b is not None:
+        keep.append(b.contiguous())
+        p.bias = keep[-1].data_ptr()
+    p.output = out.data_ptr()
+    raw_out = None
+    if own_conv:
+        keep.append(case['offset_weight'].contiguous())
+        pp.offset_weight = keep[-1].data_ptr()
+        if case['offset_bias'] is not None:
+            keep.append(case['offset_bias'].contiguous())
+            pp.offset_bias = keep[-1].data_ptr()
+        if want_raw:
+            raw_out = torch.empty(N, co, Ho, Wo, dtype=x.dtype, device=x.device)
+            pp.raw = raw_out.data_ptr()
+    else:
+        keep.append(raw.contiguous())
+        pp.raw = keep[-1].data_ptr()
+    ws_bytes = lib.mdcn_pack_workspace_bytes(ctypes.byref(pp))
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=x.device)
+    p.workspace = ws.data_ptr() if ws_bytes else None
+    p.workspace_bytes = ws_bytes
+    stream = torch.cuda.current_stream().cuda_stream
+    if timed:
+        ms = (ctypes.c_float * 5)()
+        rc = lib.mdcn_pack_forward_timed(ctypes.byref(pp), ctypes.c_void_p(stream), ms)
+        assert rc == 0, capi.status_string(rc)
+        torch.cuda.synchronize()
+        return out, raw_out, list(ms)
+    rc = lib.mdcn_pack_forward(ctypes.byref(pp), ctypes.c_void_p(stream))
+    assert rc == 0, capi.status_string(rc)
+    torch.cuda.synchronize()
+    return out, raw_out

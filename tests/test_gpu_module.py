@@ -211,3 +211,38 @@ def test_fused_matches_direct_on_cfg3_shape():
     a = capi_forward(dev, path=capi.PATH_FUSED)
     b = capi_forward(dev, path=capi.PATH_DIRECT)
     assert float((a - b).abs().max() / b.abs().max()) <= 1e-4
+
+
+CFG5_SHAPES = [  # (C, Hin, Win, stride): the six distinct layer shapes of the ResNet-50 c3-c5 config
+    (128, 200, 336, 2), (128, 100, 168, 1), (256, 100, 168, 2), (256, 50, 84, 1),
+    (512, 50, 84, 2), (512, 25, 42, 1)]
+
+
+@pytest.mark.parametrize('shape', CFG5_SHAPES, ids=lambda s: 'x'.join(map(str, s)))
+def test_cfg5_layer_shapes(shape):
+    """bf16, batch 16, offsets/mask from a default-initialised 3x3 conv on the
+    input (chunk / cat / sigmoid as in the Pack); first and last sample against
+    the fp32 oracle on the same bf16 tensors."""
+    C, H, W, stride = shape
+    N = 16
+    torch.manual_seed(5000 + C + stride)
+    conv = torch.nn.Conv2d(C, 27, 3, stride=stride, padding=1).cuda().bfloat16()
+    x = torch.randn(N, C, H, W, device='cuda').bfloat16()
+    g = torch.Generator().manual_seed(C)
+    w = (torch.randn(C, C, 3, 3, generator=g) * (2.0 / (C * 9)) ** 0.5).bfloat16().cuda()
+    b = (torch.randn(C, generator=g) * 0.01).bfloat16().cuda()
+    with torch.no_grad():
+        raw = conv(x)
+        o1, o2, m = torch.chunk(raw, 3, dim=1)
+        off, msk = torch.cat((o1, o2), dim=1).contiguous(), torch.sigmoid(m).contiguous()
+    case = dict(input=x, offset=off, mask=msk, weight=w, bias=b, stride=(stride, stride),
+                padding=(1, 1), dilation=(1, 1), groups=1, deform_groups=1)
+    y = capi_forward(case, path=capi.PATH_FUSED)
+    assert torch.isfinite(y).all()
+    for n in (0, N - 1):
+        sub = dict(case)
+        for k in ('input', 'offset', 'mask'):
+            sub[k] = case[k][n:n + 1]
+        err = rel_err(y[n:n + 1].float().cpu().numpy(), oracle_forward(sub))
+        print(f'  cfg5 {shape} sample {n}: err {err:.3e}', flush=True)
+        assert err <= TOL[torch.bfloat16], (shape, n, err)
