@@ -156,12 +156,38 @@ int make_pack_plan(const mdcn_pack_params *pp, const Geom &g, Plan *pl) {
   return MDCN_OK;
 }
 
+// conv_offset of one batch chunk: the tiled kernel when its input patch and one
+// slab of weights fit an LDS budget, else the gather variant.
 template <typename E, int COF>
-hipError_t launch_oconv(const OconvArgs &oa, hipStream_t st) {
+hipError_t launch_oconv(OconvArgs oa, hipStream_t st) {
+  const Geom &g = oa.g;
+  const int PW = 31 * g.sw + (g.kw - 1) * g.dw + 1;
+  const long wbytes = (long)g.taps * 4 * COF * 1024;
+  auto lds_bytes = [&](int th) {
+    return (long)((th - 1) * g.sh + (g.kh - 1) * g.dh + 1) * PW * kRowB + wbytes;
+  };
+  oa.tiles_x = (g.Wo + 31) / 32;
+  oa.PW = PW;
+  auto tiled = [&](int th, auto kernel) {
+    oa.TH = th;
+    oa.tiles_y = (g.Ho + th - 1) / th;
+    oa.PH = (th - 1) * g.sh + (g.kh - 1) * g.dh + 1;
+    const long tiles = (long)g.N * oa.tiles_y * oa.tiles_x;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)tiles), dim3(256), 0, st, oa);
+    return hipGetLastError();
+  };
+  // 8 rows per workgroup when that still fills the chip, else 4
+  if constexpr (COF <= 2) {
+    const long tiles8 = (long)g.N * ((g.Ho + 7) / 8) * oa.tiles_x;
+    if (lds_bytes(8) <= kOconvLdsSmall && tiles8 >= 2L * num_cus())
+      return tiled(8, oconv_tiled_kernel<E, COF, 2, kOconvLdsSmall>);
+  }
+  if (lds_bytes(4) <= kOconvLdsSmall) return tiled(4, oconv_tiled_kernel<E, COF, 1, kOconvLdsSmall>);
+  if (lds_bytes(4) <= kOconvLdsLarge) return tiled(4, oconv_tiled_kernel<E, COF, 1, kOconvLdsLarge>);
   constexpr int PXF = COF == 1 ? 4 : (COF == 2 ? 2 : 1);
   const long px_per_block = 4L * 32 * PXF;
   const long blocks = (oa.total_px + px_per_block - 1) / px_per_block;
-  hipLaunchKernelGGL((oconv_kernel<E, COF, PXF>), dim3((unsigned)blocks), dim3(256), 0, st, oa);
+  hipLaunchKernelGGL((oconv_gather_kernel<E, COF, PXF>), dim3((unsigned)blocks), dim3(256), 0, st, oa);
   return hipGetLastError();
 }
 

@@ -23,7 +23,14 @@ struct OconvArgs {
   int CO_pad;         // CO rounded up to 32
   int slabs_total;    // Cin / KC
   int plane_px;       // Hp * Wp
+  // tiled kernel: a workgroup computes TH x 32 output pixels of one image from a
+  // PH x PW patch of the input copy
+  int TH, tiles_x, tiles_y, PH, PW;
 };
+
+// LDS budgets of the tiled kernel (bytes): two workgroups per CU, or one.
+constexpr int kOconvLdsSmall = 80 * 1024;
+constexpr int kOconvLdsLarge = 156 * 1024;
 
 // conv_offset weight (CO, Cin, kh, kw) -> MFMA B fragments: for every
 // (slab, tap, ksub, 32-channel block) the 64 lanes' 16-byte operands back to
@@ -57,14 +64,16 @@ __global__ __launch_bounds__(256) void pack_offset_weight_kernel(Geom g, const E
   }
 }
 
-// Implicit GEMM raw[pixel][co] = sum_{c, tap} x[pixel + tap][c] * ow[co][c][tap] + ob[co].
-// No LDS: the A operand of the MFMA (32 pixels x 16 bytes of channels) is loaded
-// from the input copy as it lies, the B operand from the packed weights; each
-// wave owns PXF blocks of 32 consecutive pixels and all COF blocks of 32 output
-// channels.  A tap outside the one-pixel zero border (padding > 1) contributes a
-// zero fragment.
+// Implicit GEMM raw[pixel][co] = sum_{c, tap} x[pixel + tap][c] * ow[co][c][tap] + ob[co],
+// variant without LDS for geometries whose input patch does not fit the tiled
+// kernel below (large dilated kernels with stride): the A operand of the MFMA
+// (32 pixels x 16 bytes of channels) is loaded from the input copy as it lies,
+// the B operand from the packed weights; each wave owns PXF blocks of 32
+// consecutive pixels and all COF blocks of 32 output channels.  A tap outside the
+// one-pixel zero border (padding > 1) contributes a zero fragment.  Every lane of
+// an A load reads another cache line, which makes this the slow variant.
 template <typename E, int COF, int PXF>
-__global__ __launch_bounds__(256) void oconv_kernel(OconvArgs a) {
+__global__ __launch_bounds__(256) void oconv_gather_kernel(OconvArgs a) {
   using TR = ElemTraits<E>;
   const Geom &g = a.g;
   const int lane = threadIdx.x & 63;
@@ -147,6 +156,142 @@ __global__ __launch_bounds__(256) void oconv_kernel(OconvArgs a) {
       for (int r = 0; r < 16; ++r) {
         const long p = p_wave + pf * 32 + (r >> 2) * 8 + fhalf * 4 + (r & 3);
         if (p < a.total_px) raw[p * a.CO_pad + co] = from_f32<E>(acc[pf][cf][r] + b);
+      }
+    }
+  }
+}
+
+// Tiled variant, the usual one.  A workgroup of 4 waves computes TH = 4 * PXF
+// output rows x 32 output columns of one image.  Per channel slab it copies the
+// input patch those outputs need (PH x PW pixels, 128 bytes each, contiguous
+// runs of PW pixels in the copy) to LDS with coalesced 16-byte loads, zero
+// filling what lies outside the bordered copy, and every (tap, 16-byte channel
+// chunk) then takes its A operand from LDS: lane (pixel column r, half h) of wave
+// w reads chunk 2 * ksub + h of patch pixel ((w * PXF + pf) * sh + i * dh,
+// r * sw + j * dw).  Chunk c of patch pixel q sits at c ^ (q & 7), which spreads
+// the 32 rows of a fragment read over all banks when sw is odd.  The slab's
+// packed weights (taps * 4 * COF KiB) follow the patch in LDS, so that no global
+// load sits between the MFMAs.  With the small budget two workgroups share a CU
+// and the copy of one overlaps the MFMAs of the other.
+template <typename E, int COF, int PXF, int LDS_BYTES>
+__global__ __launch_bounds__(256, LDS_BYTES <= kOconvLdsSmall ? 2 : 1) void oconv_tiled_kernel(
+    OconvArgs a) {
+  using TR = ElemTraits<E>;
+  __shared__ uint4 patch[LDS_BYTES / 16];
+  const Geom &g = a.g;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int frow = lane & 31;
+  const int fhalf = lane >> 5;
+
+  int b = blockIdx.x;
+  const int tx = b % a.tiles_x;
+  b /= a.tiles_x;
+  const int ty = b % a.tiles_y;
+  const int n = b / a.tiles_y;
+  const int ho0 = ty * a.TH, wo0 = tx * 32;
+  const int py0 = ho0 * g.sh - g.ph + 1;  // patch origin in the bordered copy (may lie outside)
+  const int px0 = wo0 * g.sw - g.pw + 1;
+  const int patch_px = a.PH * a.PW;
+
+  f32x16 acc[PXF][COF];
+#pragma unroll
+  for (int pf = 0; pf < PXF; ++pf)
+#pragma unroll
+    for (int cf = 0; cf < COF; ++cf)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[pf][cf][r] = 0.0f;
+
+  // patch pixel of this lane's output pixel for tap (0, 0)
+  int q0[PXF];
+#pragma unroll
+  for (int pf = 0; pf < PXF; ++pf) q0[pf] = ((wave * PXF + pf) * g.sh) * a.PW + frow * g.sw;
+
+  uint4 *wlds = patch + patch_px * 8;
+  const int wchunks = g.taps * 4 * COF * 64;  // 16-byte chunks of one slab's weights
+  for (int slab = 0; slab < a.slabs_total; ++slab) {
+    const uint4 *src = (const uint4 *)a.xt + ((long)n * a.slabs_total + slab) * a.plane_px * 8;
+    const uint4 *wsrc = (const uint4 *)a.owp + (long)slab * wchunks;
+    __syncthreads();  // the previous slab's fragment reads are done
+    // copies in batches of kBatch independent loads per thread, so that their
+    // latencies overlap instead of adding up
+    constexpr int kBatch = 8;
+    for (int base = tid; base < wchunks; base += 256 * kBatch) {
+      uint4 v[kBatch];
+#pragma unroll
+      for (int j = 0; j < kBatch; ++j) {
+        const int idx = base + 256 * j;
+        v[j] = wsrc[idx < wchunks ? idx : 0];
+      }
+#pragma unroll
+      for (int j = 0; j < kBatch; ++j) {
+        const int idx = base + 256 * j;
+        if (idx < wchunks) wlds[idx] = v[j];
+      }
+    }
+    for (int base = tid; base < patch_px * 8; base += 256 * kBatch) {
+      uint4 v[kBatch];
+      int dst[kBatch];
+#pragma unroll
+      for (int j = 0; j < kBatch; ++j) {
+        const int idx = base + 256 * j;
+        const int q = idx >> 3, c = idx & 7;
+        const int r = q / a.PW;
+        const int y = py0 + r, x = px0 + (q - r * a.PW);
+        const bool ok = idx < patch_px * 8 && y >= 0 && y < g.Hp && x >= 0 && x < g.Wp;
+        v[j] = src[ok ? ((long)y * g.Wp + x) * 8 + c : 0];
+        if (!ok) v[j] = make_uint4(0u, 0u, 0u, 0u);
+        dst[j] = idx < patch_px * 8 ? q * 8 + (c ^ (q & 7)) : -1;
+      }
+#pragma unroll
+      for (int j = 0; j < kBatch; ++j)
+        if (dst[j] >= 0) patch[dst[j]] = v[j];
+    }
+    __syncthreads();
+    for (int ti = 0; ti < g.kh; ++ti) {
+      for (int tj = 0; tj < g.kw; ++tj) {
+        const int tap = ti * g.kw + tj;
+        const int dq = ti * g.dh * a.PW + tj * g.dw;
+        const uint4 *wfrag = wlds + tap * 4 * COF * 64 + lane;
+#pragma unroll
+        for (int ksub = 0; ksub < 4; ++ksub) {
+          uint4 af[PXF], bf[COF];
+#pragma unroll
+          for (int cf = 0; cf < COF; ++cf) bf[cf] = wfrag[(ksub * COF + cf) * 64];
+#pragma unroll
+          for (int pf = 0; pf < PXF; ++pf) {
+            const int q = q0[pf] + dq;
+            af[pf] = patch[q * 8 + ((ksub * 2 + fhalf) ^ (q & 7))];
+          }
+#pragma unroll
+          for (int pf = 0; pf < PXF; ++pf)
+#pragma unroll
+            for (int cf = 0; cf < COF; ++cf) TR::mma(acc[pf][cf], af[pf], bf[cf]);
+        }
+      }
+    }
+  }
+
+  // Accumulator block (A = pixels, B = channels): register r of lane l holds
+  //   pixel column = (r/4)*8 + (l/32)*4 + r%4,  channel = l%32.
+  E *raw = (E *)a.raw;
+  const long plane_out = (long)g.Ho * g.Wo;
+#pragma unroll
+  for (int cf = 0; cf < COF; ++cf) {
+    const int co = cf * 32 + frow;
+    float bias = 0.0f;
+    if (a.obias && co < a.CO) bias = to_f32(((const E *)a.obias)[co]);
+#pragma unroll
+    for (int pf = 0; pf < PXF; ++pf) {
+      const int ho = ho0 + wave * PXF + pf;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int wo = wo0 + (r >> 2) * 8 + fhalf * 4 + (r & 3);
+        if (ho < g.Ho && wo < g.Wo) {
+          const long p = (long)n * plane_out + (long)ho * g.Wo + wo;
+          raw[p * a.CO_pad + co] = from_f32<E>(acc[pf][cf][r] + bias);
+        }
       }
     }
   }

@@ -21,6 +21,8 @@ CASES = [
     ('c64_5x5', dict(N=1, Cin=64, Cout=48, H=12, W=12, k=5, padding=2)),
     ('c64_1x3', dict(N=1, Cin=64, Cout=64, H=7, W=21, k=(1, 3), padding=(0, 1))),
     ('c64_odd_tail', dict(N=3, Cin=64, Cout=64, H=11, W=13)),
+    ('c64_wide_rows', dict(N=2, Cin=64, Cout=64, H=37, W=70)),
+    ('c64_5x5_d3_s2_big_patch', dict(N=1, Cin=64, Cout=32, H=30, W=41, k=5, padding=6, dilation=3, stride=2)),
     ('c16_direct', dict(N=2, Cin=16, Cout=24, H=9, W=10)),
     ('c20_direct_dg2_s2', dict(N=1, Cin=20, Cout=10, H=12, W=9, stride=2, deform_groups=2)),
 ]
