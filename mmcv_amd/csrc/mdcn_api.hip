@@ -317,14 +317,14 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
       gc.N = std::min(pl.n_chunk, g.N - n0);
       const E *in = (const E *)p->input + (size_t)n0 * g.Cin * g.H * g.W;
       {
-        // columns 1 .. W+1 of the padded row in chunks of 128 (column 0 rides along)
-        const int n_xchunks = (gc.W + 1 + 127) / 128;
-        const long blocks = (long)gc.N * gc.Hp * (gc.Cin / pl.KC) * n_xchunks;
-        // 16-bit pixels are read two at a time when every row starts word aligned
-        const int words_ok = (gc.W % 2 == 0) && (((uintptr_t)in % 4) == 0);
+        // runs of 128 pixels of the image plane
+        const int n_pchunks = (gc.H * gc.W + 127) / 128;
+        const long blocks = (long)gc.N * (gc.Cin / pl.KC) * n_pchunks;
+        // 16-bit pixels are read two at a time when every channel plane starts word aligned
+        const int words_ok = ((gc.H * gc.W) % 2 == 0) && (((uintptr_t)in % 4) == 0);
         tic();
         hipLaunchKernelGGL(relayout_kernel<E>, dim3((unsigned)blocks), dim3(256), 0, st, gc, in,
-                           xt, n_xchunks, words_ok);
+                           xt, n_pchunks, words_ok);
         if (hipGetLastError() != hipSuccess) rc = MDCN_ERR_LAUNCH;
         toc(0);
       }

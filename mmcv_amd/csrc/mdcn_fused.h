@@ -47,7 +47,10 @@ constexpr int kRowChunks = kRowB / 16;
 constexpr int kGatherAhead = 2;    // K steps a gather is in flight
 constexpr int kWeightAhead = 1;    // K steps a weight-tile copy is in flight
 constexpr int kWeightSlots = kWeightAhead + 2;
-constexpr int kThreads = 512;
+constexpr int kProducerWaves = 4;                        // waves 4 .. 4 + kProducerWaves - 1
+constexpr int kThreads = 256 + 64 * kProducerWaves;
+constexpr int kPxPerLane = 8 / kProducerWaves;           // pixels of the tile a producer lane serves
+constexpr int kTapGroups = kProducerWaves / 2;           // producer lanes per pixel in the table build
 
 struct FusedArgs {
   Geom g;
@@ -319,7 +322,7 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
   constexpr int MB = CT / 64;        // 32-channel accumulator blocks per consumer wave
   constexpr int NB = 2;              // 32-pixel blocks per consumer wave
   constexpr int WDMA = CT / 32;      // 1 KiB direct-to-LDS copies per consumer wave and K step
-  constexpr int TPT = (TMAX + 1) / 2;  // table entries per producer lane
+  constexpr int TPT = (TMAX + kTapGroups - 1) / kTapGroups;  // table entries per producer lane
   static_assert(kWeightAhead * WDMA < 64, "vmcnt holds 6 bits");
 
   __shared__ uint4 Xs[2][PT * kRowChunks];                // sample tiles
@@ -391,14 +394,14 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
         E rdy[TPT], rdx[TPT], rm[TPT];
 #pragma unroll
         for (int i = 0; i < TPT; ++i) {
-          const int tap = min((ptid >> 7) + 2 * i, taps - 1);
+          const int tap = min((ptid >> 7) + kTapGroups * i, taps - 1);
           rdy[i] = off[(long)(2 * tap) * a.om.off_ch];
           rdx[i] = off[(long)(2 * tap + 1) * a.om.off_ch];
           rm[i] = msk[(long)tap * a.om.msk_ch];
         }
 #pragma unroll
         for (int i = 0; i < TPT; ++i) {
-          const int tap = (ptid >> 7) + 2 * i;
+          const int tap = (ptid >> 7) + kTapGroups * i;
           if (tap < taps) {
             const int ti = tap / g.kw, tj = tap - ti * g.kw;
             const TapSample sm =
@@ -421,12 +424,12 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
 
       // -- gather state: kGatherAhead register sets, set m % kGatherAhead holds step m;
       //    [pixel][corner][half of the lane's 32 bytes]
-      uint4 gv[kGatherAhead][2][4][2];
-      uint4 gw[kGatherAhead][2];
+      uint4 gv[kGatherAhead][kPxPerLane][4][2];
+      uint4 gw[kGatherAhead][kPxPerLane];
 
       // Gather of the cursor's step (rebuilding the table first when the step
       // opens a new deformable group), then move the cursor on.
-      auto issue_gather = [&](uint4 (&v)[2][4][2], uint4 (&w)[2]) {
+      auto issue_gather = [&](uint4 (&v)[kPxPerLane][4][2], uint4 (&w)[kPxPerLane]) {
         if (MULTI_DG && cur.new_dg) {
           // Every producer issued the previous group's last step before the
           // barrier that ended the previous K step, with its weights in registers.
@@ -436,8 +439,8 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
         }
         const int sbase = (slab0 + cur.slab) * a.plane_px;
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          const int e = cur.tap * PT + pxl + 64 * h;
+        for (int h = 0; h < kPxPerLane; ++h) {
+          const int e = cur.tap * PT + pxl + (PT / kPxPerLane) * h;
           const uint32_t o = ((uint32_t)(tpix[e] + sbase) << 7) + (uint32_t)q * 16u;
           w[h] = tws[e];
           const unsigned char *top = xt + o;
@@ -457,24 +460,24 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
       // Blend the set (step s) into sample tile `buf` and refill it with the
       // gather of the cursor's step, 16 bytes x 4 corners at a time: the loads go
       // out between the blends, so the memory pipeline works while the VALU does.
-      auto commit_and_refill = [&](int buf, uint4 (&v)[2][4][2], uint4 (&w)[2]) {
+      auto commit_and_refill = [&](int buf, uint4 (&v)[kPxPerLane][4][2], uint4 (&w)[kPxPerLane]) {
         if (MULTI_DG && cur.new_dg) {
           cur.new_dg = false;
           build_table((ch0 + cur.slab * KC) / g.ch_per_dg);
           MDCN_BARRIER_LDS();  // R
         }
         const int sbase = (slab0 + cur.slab) * a.plane_px;
-        uint32_t o[2];
-        uint4 wn[2];
+        uint32_t o[kPxPerLane];
+        uint4 wn[kPxPerLane];
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          const int e = cur.tap * PT + pxl + 64 * h;
+        for (int h = 0; h < kPxPerLane; ++h) {
+          const int e = cur.tap * PT + pxl + (PT / kPxPerLane) * h;
           o[h] = ((uint32_t)(tpix[e] + sbase) << 7) + (uint32_t)q * 16u;
           wn[h] = tws[e];
         }
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          const int row = pxl + 64 * h;
+        for (int h = 0; h < kPxPerLane; ++h) {
+          const int row = pxl + (PT / kPxPerLane) * h;
 #pragma unroll
           for (int half = 0; half < 2; ++half) {
             Xs[buf][tile_chunk(row, q + 4 * half)] =

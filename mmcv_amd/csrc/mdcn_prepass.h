@@ -11,15 +11,17 @@ namespace mdcn {
 // the image reads a stored zero, which is exactly the per-corner rule of the
 // reference sampler (mmcv/ops/csrc/pytorch/cpu/modulated_deform_conv.cpp:17-27).
 //
-// One block moves one slab of 128 consecutive pixels of one padded row through
-// LDS.  Reads run along W in 32-bit words (two 16-bit pixels or one fp32 pixel,
-// a wave takes 256 contiguous bytes of one channel row); writes are 16 bytes per
-// lane, a wave covering 1 KiB of contiguous output.  The block's pixels are
-// padded columns 1+128*xc .. 128+128*xc, i.e. source columns 128*xc .. , so the
-// word reads are aligned; column 0 of the border is written by block xc == 0.
+// One block moves one slab of 128 consecutive pixels of the image plane (rows
+// run on into each other, so every block but the last of a plane is full
+// whatever W is) through LDS.  Reads run along the plane in 32-bit words (two
+// 16-bit pixels or one fp32 pixel; a wave takes 256 contiguous bytes of one
+// channel), writes are 16 bytes per lane, 128 per pixel.  The pixel that ends an
+// image row also zeroes the two border pixels that follow it in the copy (right
+// border of its row, left border of the next); the first block of a plane
+// zeroes the top border row and the pixel after it, the last one the bottom row.
 template <typename E>
 __global__ __launch_bounds__(256) void relayout_kernel(Geom g, const E *__restrict__ in,
-                                                       E *__restrict__ xt, int n_xchunks,
+                                                       E *__restrict__ xt, int n_pchunks,
                                                        int words_ok) {
   constexpr int KC = 128 / (int)sizeof(E);
   constexpr int EPW = 4 / (int)sizeof(E);   // elements per 32-bit word
@@ -27,37 +29,37 @@ __global__ __launch_bounds__(256) void relayout_kernel(Geom g, const E *__restri
   __shared__ uint32_t tile[128 * ROWW];
 
   int b = blockIdx.x;
-  const int xc = b % n_xchunks;
-  b /= n_xchunks;
+  const int pc = b % n_pchunks;
+  b /= n_pchunks;
   const int slabs_total = g.Cin / KC;
   const int slab = b % slabs_total;
-  b /= slabs_total;
-  const int yp = b % g.Hp;
-  const int n = b / g.Hp;
+  const int n = b / slabs_total;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const bool row_inside = (yp >= 1) && (yp <= g.H);
+  const int plane = g.H * g.W;
+  const int p0 = pc * 128;
 
-  if (row_inside) {
-    // 64 row segments (KC channels x 128/(64*EPW) parts), 16 per wave
+  {
+    const E *src_slab = in + ((long)n * g.Cin + slab * KC) * plane;
+    // 64 segments (KC channels x 128/(64*EPW) parts of the pixel run), 16 per wave
 #pragma unroll 4
     for (int it = 0; it < 16; ++it) {
       const int seg = wave + 4 * it;
       const int c = seg % KC;
       const int part = seg / KC;                      // fp32: two halves of 64 pixels
       const int lp = (part * 64 + lane) * EPW;        // first local pixel of the word
-      const int x = xc * 128 + lp;
-      const E *src = in + (((long)n * g.Cin + slab * KC + c) * g.H + (yp - 1)) * g.W + x;
+      const int p = p0 + lp;
+      const E *src = src_slab + (long)c * plane + p;
       if (EPW == 2) {
         uint32_t word = 0;
         if (words_ok) {
-          if (x < g.W) word = *(const uint32_t *)src;  // W even: x + 1 < W too
+          if (p < plane) word = *(const uint32_t *)src;  // plane even: p + 1 < plane too
         } else {
           uint32_t lo = 0, hi = 0;
-          if (x < g.W) lo = *(const uint16_t *)src;
-          if (x + 1 < g.W) hi = *((const uint16_t *)src + 1);
+          if (p < plane) lo = *(const uint16_t *)src;
+          if (p + 1 < plane) hi = *((const uint16_t *)src + 1);
           word = lo | (hi << 16);
         }
         uint16_t *t16 = (uint16_t *)tile;
@@ -65,29 +67,37 @@ __global__ __launch_bounds__(256) void relayout_kernel(Geom g, const E *__restri
         t16[(lp + 1) * (ROWW * 2) + c] = (uint16_t)(word >> 16);
       } else {
         uint32_t word = 0;
-        if (x < g.W) word = *(const uint32_t *)src;
+        if (p < plane) word = *(const uint32_t *)src;
         tile[lp * ROWW + c] = word;
       }
     }
   }
   __syncthreads();
-  unsigned char *dst_row =
-      (unsigned char *)xt + ((((long)n * slabs_total + slab) * g.Hp + yp) * g.Wp) * 128;
+  unsigned char *dst_slab =
+      (unsigned char *)xt + (((long)n * slabs_total + slab) * g.Hp * g.Wp) * 128;
+  const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
 #pragma unroll
   for (int it = 0; it < 4; ++it) {
     const int u = tid + 256 * it;
     const int lp = u >> 3, q = u & 7;
-    const int xp = xc * 128 + 1 + lp;
-    if (xp < g.Wp) {
-      uint4 v = make_uint4(0u, 0u, 0u, 0u);
-      if (row_inside) {
-        const uint32_t *t = tile + lp * ROWW + q * 4;
-        v = make_uint4(t[0], t[1], t[2], t[3]);
+    const int p = p0 + lp;
+    if (p < plane) {
+      const int y = p / g.W;
+      const int x = p - y * g.W;
+      const uint32_t *t = tile + lp * ROWW + q * 4;
+      unsigned char *d = dst_slab + ((long)(y + 1) * g.Wp + (x + 1)) * 128 + q * 16;
+      *(uint4 *)d = make_uint4(t[0], t[1], t[2], t[3]);
+      if (x == g.W - 1) {
+        *(uint4 *)(d + 128) = zero;
+        *(uint4 *)(d + 256) = zero;
       }
-      *(uint4 *)(dst_row + (long)xp * 128 + q * 16) = v;
     }
   }
-  if (xc == 0 && tid < 8) *(uint4 *)(dst_row + tid * 16) = make_uint4(0u, 0u, 0u, 0u);
+  if (pc == 0)  // top border row and the left border pixel of the first image row
+    for (int i = tid; i < (g.Wp + 1) * 8; i += 256) *(uint4 *)(dst_slab + (long)i * 16) = zero;
+  if (pc == n_pchunks - 1)  // bottom border row
+    for (int i = tid; i < g.Wp * 8; i += 256)
+      *(uint4 *)(dst_slab + ((long)(g.Hp - 1) * g.Wp) * 128 + (long)i * 16) = zero;
 }
 
 // weight[Cout][Cin/G][kh][kw] -> wp[G][n_ctiles][nk][CT][KC]: for every
