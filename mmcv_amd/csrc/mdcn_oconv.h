@@ -210,44 +210,48 @@ __global__ __launch_bounds__(256, LDS_BYTES <= kOconvLdsSmall ? 2 : 1) void ocon
 
   uint4 *wlds = patch + patch_px * 8;
   const int wchunks = g.taps * 4 * COF * 64;  // 16-byte chunks of one slab's weights
-  for (int slab = 0; slab < a.slabs_total; ++slab) {
+  const int total_chunks = patch_px * 8 + wchunks;
+
+  // A slab's LDS contents arrive by direct-to-LDS copies, 1 KiB per wave and
+  // instruction: lane l of copy j fills chunk i = 256 * j + 64 * wave + l of the
+  // LDS array and reads the source chunk that belongs there (the swizzle is
+  // applied on the source side).  Per chunk, once per workgroup and the same for
+  // every slab: soff >= 0 is an offset into the slab's plane of the copy, soff < 0
+  // weight chunk -1 - soff.  A patch pixel outside the copy reads the copy's
+  // corner pixel (0, 0), a stored zero.  All copies of a slab are in flight
+  // together; nothing the compiler sees waits between them.
+  constexpr int NB = (LDS_BYTES / 16 + 255) / 256;
+  int soff[NB];
+#pragma unroll
+  for (int j = 0; j < NB; ++j) {
+    const int idx = tid + 256 * j;
+    const int q = idx >> 3;
+    const int c = (idx & 7) ^ (q & 7);
+    const int r = q / a.PW;
+    const int y = py0 + r, x = px0 + (q - r * a.PW);
+    const bool in_copy = y >= 0 && y < g.Hp && x >= 0 && x < g.Wp;
+    if (idx < patch_px * 8) soff[j] = in_copy ? (y * g.Wp + x) * 8 + c : c;
+    else if (idx < total_chunks) soff[j] = -1 - (idx - patch_px * 8);
+    else soff[j] = 0;
+  }
+  const uint32_t lds_wave = (uint32_t)(uintptr_t)(lptr_t)(&patch[0]) +
+                            (uint32_t)__builtin_amdgcn_readfirstlane(wave) * 1024u;
+  auto fetch = [&](int slab) {
     const uint4 *src = (const uint4 *)a.xt + ((long)n * a.slabs_total + slab) * a.plane_px * 8;
     const uint4 *wsrc = (const uint4 *)a.owp + (long)slab * wchunks;
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+      if (256 * j < total_chunks) {
+        const uint4 *ptr = soff[j] >= 0 ? src + soff[j] : wsrc + (-1 - soff[j]);
+        copy16_global_to_lds(ptr, lds_wave + (uint32_t)j * 4096u);
+      }
+    }
+  };
+
+  for (int slab = 0; slab < a.slabs_total; ++slab) {
     __syncthreads();  // the previous slab's fragment reads are done
-    // copies in batches of kBatch independent loads per thread, so that their
-    // latencies overlap instead of adding up
-    constexpr int kBatch = 8;
-    for (int base = tid; base < wchunks; base += 256 * kBatch) {
-      uint4 v[kBatch];
-#pragma unroll
-      for (int j = 0; j < kBatch; ++j) {
-        const int idx = base + 256 * j;
-        v[j] = wsrc[idx < wchunks ? idx : 0];
-      }
-#pragma unroll
-      for (int j = 0; j < kBatch; ++j) {
-        const int idx = base + 256 * j;
-        if (idx < wchunks) wlds[idx] = v[j];
-      }
-    }
-    for (int base = tid; base < patch_px * 8; base += 256 * kBatch) {
-      uint4 v[kBatch];
-      int dst[kBatch];
-#pragma unroll
-      for (int j = 0; j < kBatch; ++j) {
-        const int idx = base + 256 * j;
-        const int q = idx >> 3, c = idx & 7;
-        const int r = q / a.PW;
-        const int y = py0 + r, x = px0 + (q - r * a.PW);
-        const bool ok = idx < patch_px * 8 && y >= 0 && y < g.Hp && x >= 0 && x < g.Wp;
-        v[j] = src[ok ? ((long)y * g.Wp + x) * 8 + c : 0];
-        if (!ok) v[j] = make_uint4(0u, 0u, 0u, 0u);
-        dst[j] = idx < patch_px * 8 ? q * 8 + (c ^ (q & 7)) : -1;
-      }
-#pragma unroll
-      for (int j = 0; j < kBatch; ++j)
-        if (dst[j] >= 0) patch[dst[j]] = v[j];
-    }
+    fetch(slab);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     for (int ti = 0; ti < g.kh; ++ti) {
       for (int tj = 0; tj < g.kw; ++tj) {
