@@ -55,7 +55,7 @@ enum mdcn_status {
  * device that is current when the call is made:
  *   input  (N, Cin, H, W)                      NCHW
  *   offset (N, dgroups*2*kh*kw, Ho, Wo)        channel 2t = dy, 2t+1 = dx of tap t = i*kw + j
- *   mask   (N, dgroups*kh*kw, Ho, Wo)
+ *   mask   (N, dgroups*kh*kw, Ho, Wo)           or NULL: unmodulated (DCNv1), see below
  *   weight (Cout, Cin/groups, kh, kw)
  *   bias   (Cout) or NULL                      NULL <=> with_bias == false
  *   output (N, Cout, Ho, Wo)                   written in full, need not be initialised
@@ -63,6 +63,12 @@ enum mdcn_status {
  * (mmcv/ops/csrc/pytorch/modulated_deform_conv.cpp:87-90).  Sampling positions and
  * bilinear weights are always computed in fp32; products are accumulated in
  * fp32 and rounded once to `dtype` after the bias add.
+ *
+ * mask == NULL (with bias == NULL) is the deformable convolution without
+ * modulation, `deform_conv_forward` of the reference
+ * (mmcv/ops/csrc/pytorch/deform_conv.cpp:140-260, sampler
+ * cpu/deform_conv.cpp:5-38): the same sampling rule with factor 1.  The
+ * reference's im2col_step only sizes its scratch buffers and has no counterpart.
  */
 typedef struct mdcn_params {
   const void *input;
@@ -140,6 +146,8 @@ typedef struct mdcn_pack_params {
   const void *offset_weight;
   const void *offset_bias;
   void *raw;
+  int32_t unmodulated;  /* 1: DeformConv2dPack.forward (mmcv/ops/deform_conv.py:405-409): conv_offset has
+                           2*dgroups*kh*kw channels, all of them offsets, and there is no mask */
 } mdcn_pack_params;
 
 /* Bytes of device scratch mdcn_pack_forward() needs (conv.workspace must hold

@@ -31,7 +31,8 @@ class MdcnParams(ctypes.Structure):
 
 class MdcnPackParams(ctypes.Structure):
     _fields_ = [('conv', MdcnParams), ('offset_weight', ctypes.c_void_p),
-                ('offset_bias', ctypes.c_void_p), ('raw', ctypes.c_void_p)]
+                ('offset_bias', ctypes.c_void_p), ('raw', ctypes.c_void_p),
+                ('unmodulated', ctypes.c_int32)]
 
 
 _lib = None

@@ -179,7 +179,8 @@ std::vector<double> modulated_deform_conv_pack_forward(
     Tensor input, Tensor offset_weight, Tensor offset_bias, Tensor raw,
     Tensor weight, Tensor bias, Tensor output, int kernel_h, int kernel_w,
     int stride_h, int stride_w, int pad_h, int pad_w, int dilation_h,
-    int dilation_w, int group, int deformable_group, bool with_bias, bool timed) {
+    int dilation_w, int group, int deformable_group, bool with_bias, bool timed,
+    bool unmodulated) {
   const char *op = "modulated_deform_conv_pack_forward";
   TORCH_CHECK(input.dim() == 4 && weight.dim() == 4, op, " expects 4-D input and weight");
   const at::Device dev = input.device();
@@ -217,7 +218,8 @@ std::vector<double> modulated_deform_conv_pack_forward(
   int32_t Ho = 0, Wo = 0;
   int rc = mdcn_output_size(&p, &Ho, &Wo);
   TORCH_CHECK(rc == MDCN_OK, op, ": ", mdcn_status_string(rc));
-  const int64_t co = (int64_t)3 * deformable_group * kernel_h * kernel_w;
+  const int64_t co = (int64_t)(unmodulated ? 2 : 3) * deformable_group * kernel_h * kernel_w;
+  pp.unmodulated = unmodulated ? 1 : 0;
   TORCH_CHECK(output.numel() == batch * channels_out * Ho * Wo && output.is_contiguous(), op,
               ": output must be a dense (", batch, ", ", channels_out, ", ", Ho, ", ", Wo,
               ") tensor, got ", output.sizes());
@@ -270,6 +272,105 @@ std::vector<double> modulated_deform_conv_pack_forward(
   return {ms[0], ms[1], ms[2], ms[3], ms[4]};
 }
 
+// Deformable convolution without modulation
+// (mmcv/ops/csrc/pytorch/deform_conv.cpp:140-260; pybind.cpp:38-62,525-547 for the
+// argument names).  `columns`, `ones` and `im2col_step` size the reference's
+// scratch buffers and are not needed here; the step must still divide the batch,
+// as its caller asserts (mmcv/ops/deform_conv.py:115-117).
+void deform_conv_forward(Tensor input, Tensor weight, Tensor offset, Tensor output,
+                         Tensor columns, Tensor ones, int kW, int kH, int dW, int dH,
+                         int padW, int padH, int dilationW, int dilationH, int group,
+                         int deformable_group, int im2col_step) {
+  (void)columns;
+  (void)ones;
+  const char *op = "deform_conv_forward";
+  TORCH_CHECK(weight.dim() == 4, "4D weight tensor (nOutputPlane,nInputPlane,kH,kW) expected, but got: ",
+              weight.dim());
+  TORCH_CHECK(kW > 0 && kH > 0, "kernel size should be greater than zero, but got kH: ", kH, " kW: ", kW);
+  TORCH_CHECK(weight.size(2) == kH && weight.size(3) == kW,
+              "kernel size should be consistent with weight, but got kH: ", kH, " kW: ", kW,
+              " weight.size(2): ", weight.size(2), ", weight.size(3): ", weight.size(3));
+  TORCH_CHECK(dW > 0 && dH > 0, "stride should be greater than zero, but got dH: ", dH, " dW: ", dW);
+  TORCH_CHECK(dilationW > 0 && dilationH > 0, "dilation should be greater than 0, but got dilationH: ",
+              dilationH, " dilationW: ", dilationW);
+  TORCH_CHECK(input.dim() == 3 || input.dim() == 4, "3D or 4D input tensor expected but got: ", input.dim());
+  if (input.dim() == 3) {  // the reference forces a batch of one (:171-176)
+    input = input.unsqueeze(0);
+    offset = offset.unsqueeze(0);
+  }
+  TORCH_CHECK(offset.dim() == 4, op, " expects a 4-D offset");
+  const int64_t batch = input.size(0), planes = weight.size(1) * group;
+  TORCH_CHECK(planes % deformable_group == 0, "input channels must divide deformable group size");
+  TORCH_CHECK(input.size(1) == planes, "invalid number of input planes, expected: ", planes,
+              ", but got: ", input.size(1));
+  TORCH_CHECK(input.size(2) >= kH && input.size(3) >= kW, "input image is smaller than kernel");
+  TORCH_CHECK(im2col_step > 0 && batch % im2col_step == 0, op,
+              ": batch size must be divisible by im2col_step");
+  const at::Device dev = input.device();
+  TORCH_CHECK(dev.is_cuda(), "deformable_im2col_impl: implementation for device ", device_str(dev),
+              " not found.");
+  c10::DeviceGuard guard(dev);
+  const auto st = input.scalar_type();
+  const Tensor *all[] = {&weight, &offset, &output};
+  const char *names[] = {"weight", "offset", "output"};
+  for (int i = 0; i < 3; ++i) {
+    TORCH_CHECK(all[i]->device() == dev, op, ": at param ", names[i], ", inconsistent device: ",
+                device_str(all[i]->device()), " vs ", device_str(dev));
+    TORCH_CHECK(all[i]->scalar_type() == st, op, ": expected ", names[i], " to have dtype ",
+                c10::toString(st), " but got ", c10::toString(all[i]->scalar_type()));
+  }
+  mdcn_params p{};
+  p.dtype = mdcn_dtype_of(input);
+  p.path = g_path;
+  p.N = (int)batch; p.Cin = (int)planes; p.H = (int)input.size(2); p.W = (int)input.size(3);
+  p.Cout = (int)weight.size(0); p.kh = kH; p.kw = kW;
+  p.sh = dH; p.sw = dW; p.ph = padH; p.pw = padW; p.dh = dilationH; p.dw = dilationW;
+  p.groups = group; p.dgroups = deformable_group;
+  int32_t Ho = 0, Wo = 0;
+  int rc = mdcn_output_size(&p, &Ho, &Wo);
+  TORCH_CHECK(rc == MDCN_OK, "Given input size: (", planes, " x ", input.size(2), " x ", input.size(3),
+              "). Output size is too small");
+  TORCH_CHECK(offset.size(0) == batch, "invalid batch size of offset");
+  TORCH_CHECK(offset.size(2) == Ho && offset.size(3) == Wo,
+              "invalid spatial size of offset, expected height: ", Ho, " width: ", Wo,
+              ", but got height: ", offset.size(2), " width: ", offset.size(3));
+  TORCH_CHECK(offset.size(1) == (int64_t)deformable_group * 2 * kH * kW,
+              "invalid number of channels of offset");
+  TORCH_CHECK(output.numel() == batch * weight.size(0) * Ho * Wo && output.is_contiguous(), op,
+              ": output must be a dense (", batch, ", ", weight.size(0), ", ", Ho, ", ", Wo,
+              ") tensor, got ", output.sizes());
+  std::vector<Tensor> keep = {input.contiguous(), offset.contiguous(), weight.contiguous()};
+  p.input = keep[0].data_ptr();
+  p.offset = keep[1].data_ptr();
+  p.mask = nullptr;
+  p.weight = keep[2].data_ptr();
+  p.bias = nullptr;
+  p.output = output.data_ptr();
+  const size_t ws = mdcn_workspace_bytes(&p);
+  if (ws > 0) {
+    keep.push_back(at::empty({(int64_t)ws}, input.options().dtype(at::kByte)));
+    p.workspace = keep.back().data_ptr();
+    p.workspace_bytes = ws;
+  }
+  rc = mdcn_forward(&p, (void *)c10::hip::getCurrentHIPStream().stream());
+  TORCH_CHECK(rc == MDCN_OK, op, ": ", mdcn_status_string(rc));
+}
+
+void deform_conv_backward_input(Tensor input, Tensor offset, Tensor gradOutput, Tensor gradInput,
+                                Tensor gradOffset, Tensor weight, Tensor columns, int kW, int kH,
+                                int dW, int dH, int padW, int padH, int dilationW, int dilationH,
+                                int group, int deformable_group, int im2col_step) {
+  TORCH_CHECK(false, "deform_conv_backward_input: this build implements the forward pass only");
+}
+
+void deform_conv_backward_parameters(Tensor input, Tensor offset, Tensor gradOutput,
+                                     Tensor gradWeight, Tensor columns, Tensor ones, int kW, int kH,
+                                     int dW, int dH, int padW, int padH, int dilationW,
+                                     int dilationH, int group, int deformable_group, float scale,
+                                     int im2col_step) {
+  TORCH_CHECK(false, "deform_conv_backward_parameters: this build implements the forward pass only");
+}
+
 void modulated_deform_conv_backward(
     Tensor input, Tensor weight, Tensor bias, Tensor ones, Tensor offset,
     Tensor mask, Tensor columns, Tensor grad_input, Tensor grad_weight,
@@ -299,7 +400,24 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("bias"), py::arg("output"), py::arg("kernel_h"), py::arg("kernel_w"),
         py::arg("stride_h"), py::arg("stride_w"), py::arg("pad_h"), py::arg("pad_w"),
         py::arg("dilation_h"), py::arg("dilation_w"), py::arg("group"),
-        py::arg("deformable_group"), py::arg("with_bias"), py::arg("timed") = false);
+        py::arg("deformable_group"), py::arg("with_bias"), py::arg("timed") = false,
+        py::arg("unmodulated") = false);
+  m.def("deform_conv_forward", &deform_conv_forward, "deform_conv_forward", py::arg("input"),
+        py::arg("weight"), py::arg("offset"), py::arg("output"), py::arg("columns"), py::arg("ones"),
+        py::arg("kW"), py::arg("kH"), py::arg("dW"), py::arg("dH"), py::arg("padW"), py::arg("padH"),
+        py::arg("dilationW"), py::arg("dilationH"), py::arg("group"), py::arg("deformable_group"),
+        py::arg("im2col_step"));
+  m.def("deform_conv_backward_input", &deform_conv_backward_input, "deform_conv_backward_input",
+        py::arg("input"), py::arg("offset"), py::arg("gradOutput"), py::arg("gradInput"),
+        py::arg("gradOffset"), py::arg("weight"), py::arg("columns"), py::arg("kW"), py::arg("kH"),
+        py::arg("dW"), py::arg("dH"), py::arg("padW"), py::arg("padH"), py::arg("dilationW"),
+        py::arg("dilationH"), py::arg("group"), py::arg("deformable_group"), py::arg("im2col_step"));
+  m.def("deform_conv_backward_parameters", &deform_conv_backward_parameters,
+        "deform_conv_backward_parameters", py::arg("input"), py::arg("offset"), py::arg("gradOutput"),
+        py::arg("gradWeight"), py::arg("columns"), py::arg("ones"), py::arg("kW"), py::arg("kH"),
+        py::arg("dW"), py::arg("dH"), py::arg("padW"), py::arg("padH"), py::arg("dilationW"),
+        py::arg("dilationH"), py::arg("group"), py::arg("deformable_group"), py::arg("scale"),
+        py::arg("im2col_step"));
   m.def("modulated_deform_conv_backward", &modulated_deform_conv_backward,
         "modulated deform conv backward", py::arg("input"), py::arg("weight"),
         py::arg("bias"), py::arg("ones"), py::arg("offset"), py::arg("mask"),

@@ -42,7 +42,7 @@ int check_params(const mdcn_params *p, Geom *g, bool need_ptrs, bool need_offset
       (long)p->W + 2L * p->pw < (long)p->dw * (p->kw - 1) + 1 || Ho <= 0 || Wo <= 0)
     return MDCN_ERR_SHAPE;
   if (need_ptrs && (!p->input || !p->weight || !p->output)) return MDCN_ERR_NULL;
-  if (need_ptrs && need_offsets && (!p->offset || !p->mask)) return MDCN_ERR_NULL;
+  if (need_ptrs && need_offsets && !p->offset) return MDCN_ERR_NULL;  // mask NULL: unmodulated
   g->N = p->N; g->Cin = p->Cin; g->H = p->H; g->W = p->W;
   g->Cout = p->Cout; g->kh = p->kh; g->kw = p->kw;
   g->sh = p->sh; g->sw = p->sw; g->ph = p->ph; g->pw = p->pw;
@@ -100,7 +100,8 @@ struct Plan {
   size_t xt_bytes;   // channels-last copy of one chunk
   size_t wp_bytes;   // packed weights
   // pack-level call only
-  int CO, CO_pad;    // conv_offset channels: 3 * DG * taps, rounded up to 32
+  int CO, CO_pad;    // conv_offset channels: 3 (2 when unmodulated) * DG * taps, rounded up to 32
+  int mask_kind;     // kMaskLogit, or kMaskNone when unmodulated
   size_t owp_bytes;  // packed conv_offset weights (fused path, conv_offset run here)
   size_t raw_bytes;  // conv_offset output kept in the workspace
 };
@@ -119,6 +120,7 @@ int make_plan(const mdcn_params *p, const Geom &g, Plan *pl) {
   pl->xt_bytes = pl->wp_bytes = pl->owp_bytes = pl->raw_bytes = 0;
   pl->CO = 3 * g.DG * g.taps;
   pl->CO_pad = (pl->CO + 31) / 32 * 32;
+  pl->mask_kind = kMaskLogit;
   if (!pl->fused) return MDCN_OK;
   const size_t es = elem_size(p->dtype);
   pl->KC = slab_channels(p->dtype);
@@ -138,6 +140,11 @@ int make_pack_plan(const mdcn_pack_params *pp, const Geom &g, Plan *pl) {
   const mdcn_params *p = &pp->conv;
   const int rc = make_plan(p, g, pl);
   if (rc != MDCN_OK) return rc;
+  if (pp->unmodulated) {
+    pl->CO = 2 * g.DG * g.taps;
+    pl->CO_pad = (pl->CO + 31) / 32 * 32;
+    pl->mask_kind = kMaskNone;
+  }
   const size_t es = elem_size(p->dtype);
   const size_t plane = (size_t)g.Ho * g.Wo;
   if (pp->offset_weight) {
@@ -256,7 +263,8 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
     v.off_n = v.msk_n = (long)pl.CO * plane_out;
     v.off_ch = v.msk_ch = plane_out;
     v.off_px = v.msk_px = 1;
-    v.logit = 1;
+    v.logit = pl.mask_kind;
+    if (pl.mask_kind == kMaskNone) v.msk = raw;
     return v;
   };
 
@@ -365,12 +373,13 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
         fa.om.off_n = fa.om.msk_n = plane_out * pl.CO_pad;
         fa.om.off_ch = fa.om.msk_ch = 1;
         fa.om.off_px = fa.om.msk_px = pl.CO_pad;
-        fa.om.logit = 1;
+        fa.om.logit = pl.mask_kind;
+        if (pl.mask_kind == kMaskNone) fa.om.msk = raw_pm;
       } else if (px) {
         fa.om = nchw_raw_view((const E *)px->raw + (size_t)n0 * pl.CO * plane_out);
       } else {
         fa.om = dense_view((const E *)p->offset + (size_t)n0 * g.DG * 2 * g.taps * plane_out,
-                           (const E *)p->mask + (size_t)n0 * g.DG * g.taps * plane_out, g);
+                           p->mask ? (const E *)p->mask + (size_t)n0 * g.DG * g.taps * plane_out : nullptr, g);
       }
       fa.bias = p->bias;
       fa.out = (E *)p->output + (size_t)n0 * g.Cout * plane_out;

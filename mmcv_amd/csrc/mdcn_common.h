@@ -74,7 +74,10 @@ __device__ __forceinline__ TapSample make_tap_sample(int base_y, int base_x,
 // pack-level entry points read both out of the one conv_offset output, whose
 // first 2/3 of the channels are the offsets (chunk + cat of
 // mmcv/ops/modulated_deform_conv.py:329-330 is the identity on them) and whose
-// last third holds the mask before the sigmoid (`logit`, :331).
+// last third holds the mask before the sigmoid (`logit` = 1, :331).  `logit` = 2
+// stands for "no mask": the unmodulated deformable convolution (DCNv1,
+// mmcv/ops/csrc/pytorch/cpu/deform_conv.cpp:115-167, the same sampler without
+// the factor); msk then aliases off so that the kernels' loads stay valid.
 struct OffMaskView {
   const void *off, *msk;
   long off_n, msk_n;
@@ -82,6 +85,7 @@ struct OffMaskView {
   int off_px, msk_px;
   int logit;
 };
+constexpr int kMaskPlain = 0, kMaskLogit = 1, kMaskNone = 2;
 
 __host__ __device__ inline OffMaskView dense_view(const void *off, const void *msk, const Geom &g) {
   OffMaskView v;
@@ -90,7 +94,10 @@ __host__ __device__ inline OffMaskView dense_view(const void *off, const void *m
   v.off_n = (long)g.DG * 2 * g.taps * plane; v.msk_n = (long)g.DG * g.taps * plane;
   v.off_ch = plane; v.msk_ch = plane;
   v.off_px = 1; v.msk_px = 1;
-  v.logit = 0;
+  v.logit = kMaskPlain;
+  if (!msk) {  // unmodulated: read (and ignore) offsets instead
+    v.msk = off; v.msk_n = v.off_n; v.logit = kMaskNone;
+  }
   return v;
 }
 
@@ -99,7 +106,8 @@ __host__ __device__ inline OffMaskView dense_view(const void *off, const void *m
 template <typename E>
 __device__ __forceinline__ float mask_value(E raw, int logit) {
   float m = to_f32(raw);
-  if (logit) m = to_f32(from_f32<E>(1.0f / (1.0f + expf(-m))));
+  if (logit == kMaskLogit) m = to_f32(from_f32<E>(1.0f / (1.0f + expf(-m))));
+  if (logit == kMaskNone) m = 1.0f;
   return m;
 }
 

@@ -86,8 +86,11 @@ def capi_forward(case, path=capi.PATH_AUTO, timed=False):
     out = torch.empty(N, Cout, Ho, Wo, dtype=x.dtype, device=x.device)
     ws_bytes = lib.mdcn_workspace_bytes(ctypes.byref(p))
     ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=x.device)
-    keep = [t.contiguous() for t in (x, off, msk, w)]
-    p.input, p.offset, p.mask, p.weight = (t.data_ptr() for t in keep)
+    keep = [t.contiguous() for t in (x, off, w)]
+    p.input, p.offset, p.weight = (t.data_ptr() for t in keep)
+    if msk is not None:  # None: unmodulated (DCNv1)
+        keep.append(msk.contiguous())
+        p.mask = keep[-1].data_ptr()
     p.bias = b.contiguous().data_ptr() if b is not None else None
     p.output = out.data_ptr()
     p.workspace = ws.data_ptr() if ws_bytes else None
@@ -106,13 +109,13 @@ def capi_forward(case, path=capi.PATH_AUTO, timed=False):
 
 
 def make_pack_case(seed, N, Cin, Cout, H, W, k=3, stride=1, padding=1, dilation=1,
-                   groups=1, deform_groups=1, offset_std=0.05):
+                   groups=1, deform_groups=1, offset_std=0.05, unmodulated=False):
     """Seeded fp32 CPU tensors of a Pack layer: input, conv_offset weight and
     bias (random, so that offsets and mask are not trivial: the layer's own
     zero initialisation would make it a plain convolution), weight, bias."""
     kh, kw = pair(k)
     g = torch.Generator().manual_seed(seed)
-    co = 3 * deform_groups * kh * kw
+    co = (2 if unmodulated else 3) * deform_groups * kh * kw
     x = torch.randn(N, Cin, H, W, generator=g)
     ow = torch.randn(co, Cin, kh, kw, generator=g) * offset_std
     ob = torch.randn(co, generator=g) * 0.5
@@ -154,7 +157,8 @@ def split_raw(raw, deform_groups, taps):
     return torch.cat((o1, o2), dim=1).contiguous(), torch.sigmoid(m).contiguous()
 
 
-def capi_pack_forward(case, own_conv=True, raw=None, want_raw=False, path=capi.PATH_AUTO, timed=False):
+def capi_pack_forward(case, own_conv=True, raw=None, want_raw=False, path=capi.PATH_AUTO, timed=False,
+                      unmodulated=False):
     """mdcn_pack_forward through ctypes on device tensors; returns (output, raw
     or None[, ms])."""
     lib = capi.load()
@@ -168,7 +172,8 @@ def capi_pack_forward(case, own_conv=True, raw=None, want_raw=False, path=capi.P
     p = pp.conv
     rc, Ho, Wo = capi.output_size(p)
     assert rc == 0, capi.status_string(rc)
-    co = 3 * case['deform_groups'] * kh * kw
+    co = (2 if unmodulated else 3) * case['deform_groups'] * kh * kw
+    pp.unmodulated = 1 if unmodulated else 0
     out = torch.empty(N, Cout, Ho, Wo, dtype=x.dtype, device=x.device)
     keep = [t.contiguous() for t in (x, w)]
     p.input, p.weight = (t.data_ptr() for t in keep)

@@ -196,3 +196,33 @@ def test_onnx_symbolic_name():
     name, nargs, kw = ModulatedDeformConv2dFunction.symbolic(G(), 1, 2, 3, 4, None, 1, 1, 1, 1, 1)
     assert name == 'mmcv::MMCVModulatedDeformConv2d' and nargs == 4
     assert set(kw) == {'stride_i', 'padding_i', 'dilation_i', 'groups_i', 'deform_groups_i'}
+
+
+def test_dcnv1_python_layer():
+    import pytest
+    from mmcv_amd.ops import MODELS, DeformConv2d, DeformConv2dPack
+    import mmcv_amd._ext as ext
+    for n in ('deform_conv_forward', 'deform_conv_backward_input', 'deform_conv_backward_parameters'):
+        assert hasattr(ext, n)
+    assert MODELS.get('DCN') is DeformConv2dPack
+    layer = DeformConv2dPack(8, 6, 3, stride=2, padding=1, deformable_groups=2)
+    assert layer.deform_groups == 2 and layer.conv_offset.out_channels == 2 * 2 * 9
+    assert layer.conv_offset.stride == (2, 2) and not hasattr(layer, 'bias')
+    assert float(layer.conv_offset.weight.detach().abs().sum()) == 0.0
+    assert 'bias=False' in repr(layer)
+    with pytest.raises(AssertionError):
+        DeformConv2d(1, 1, 2, bias=True)
+    with pytest.raises(AssertionError):
+        DeformConv2d(3, 2, 3, groups=2)
+    with pytest.raises(AssertionError):
+        DeformConv2d(3, 4, 3, groups=3)
+    with pytest.raises(ValueError, match='Expected 4D tensor'):
+        layer(torch.zeros(8, 5, 5))
+    # version-1 checkpoints name the offset conv "<module>_offset"
+    sd = {'w': layer.weight.detach().clone(), 'o.weight': torch.ones(36, 8, 3, 3), 'o.bias': torch.ones(36)}
+    state = {'dcn.weight': sd['w'], 'dcn_offset.weight': sd['o.weight'], 'dcn_offset.bias': sd['o.bias']}
+    missing, unexpected, errors = [], [], []
+    layer._load_from_state_dict(state, 'dcn.', {}, True, missing, unexpected, errors)
+    assert not errors
+    assert 'dcn.conv_offset.weight' in state and 'dcn.conv_offset.bias' in state
+    assert 'dcn_offset.weight' not in state and 'dcn_offset.bias' not in state
