@@ -41,6 +41,9 @@ def _lib():
             getattr(_LIB, f'mdcn_oracle_{t}_im2col').argtypes = (
                 [ctypes.c_void_p] * 3 + [ctypes.c_int] * 14 + [ctypes.c_void_p])
             getattr(_LIB, f'mdcn_oracle_{t}_forward').restype = ctypes.c_int
+            getattr(_LIB, f'mdcn_oracle_{t}_backward').restype = ctypes.c_int
+            getattr(_LIB, f'mdcn_oracle_{t}_backward').argtypes = (
+                [ctypes.c_void_p] * 11 + [ctypes.c_int] * 16)
             getattr(_LIB, f'mdcn_oracle_{t}_forward').argtypes = (
                 [ctypes.c_void_p] * 7 + [ctypes.c_int] * 16)
     return _LIB
@@ -126,6 +129,63 @@ def forward(input, offset, mask, weight, bias=None, stride=1, padding=0,
         raise RuntimeError("Input shape and kernel channels won't match: "
                            f'({Cin} vs {wcin * groups}).')
     return out
+
+
+def backward(input, offset, mask, weight, grad_output, with_bias=True, stride=1,
+             padding=0, dilation=1, groups=1, deform_groups=1):
+    """Whole DCNv2 backward on numpy arrays (float32 or float64): returns
+    (grad_input, grad_offset, grad_mask, grad_weight, grad_bias or None)."""
+    input = np.ascontiguousarray(input)
+    t = _tag(input.dtype)
+    dt = input.dtype
+    offset = np.ascontiguousarray(offset, dtype=dt)
+    mask = np.ascontiguousarray(mask, dtype=dt)
+    weight = np.ascontiguousarray(weight, dtype=dt)
+    grad_output = np.ascontiguousarray(grad_output, dtype=dt)
+    N, Cin, H, W = input.shape
+    Cout, wcin, kh, kw = weight.shape
+    (sh, sw), (ph, pw), (dh, dw) = _pair(stride), _pair(padding), _pair(dilation)
+    Ho, Wo = output_hw(H, W, kh, kw, stride, padding, dilation)
+    assert grad_output.shape == (N, Cout, Ho, Wo), grad_output.shape
+    assert offset.shape == (N, deform_groups * 2 * kh * kw, Ho, Wo), offset.shape
+    assert mask.shape == (N, deform_groups * kh * kw, Ho, Wo), mask.shape
+    g_in = np.empty_like(input)
+    g_off = np.zeros_like(offset)
+    g_mask = np.zeros_like(mask)
+    g_w = np.empty_like(weight)
+    g_b = np.empty((Cout,), dtype=dt) if with_bias else None
+    columns = np.empty((Cin * kh * kw, Ho * Wo), dtype=dt)
+    rc = getattr(_lib(), f'mdcn_oracle_{t}_backward')(
+        _ptr(input), _ptr(weight), _ptr(offset), _ptr(mask), _ptr(grad_output),
+        _ptr(g_in), _ptr(g_w), _ptr(g_b) if with_bias else None, _ptr(g_off),
+        _ptr(g_mask), _ptr(columns), N, Cin, H, W, Cout, wcin, kh, kw, sh, sw,
+        ph, pw, dh, dw, groups, deform_groups)
+    if rc != 0:
+        raise RuntimeError("Input shape and kernel channels won't match: "
+                           f'({Cin} vs {wcin * groups}).')
+    return g_in, g_off, g_mask, g_w, g_b
+
+
+def reference_backward(input, offset, mask, weight, grad_output, with_bias=True,
+                       stride=1, padding=0, dilation=1, groups=1, deform_groups=1):
+    """mmcv's compiled CPU ``modulated_deform_conv_backward`` on torch CPU tensors,
+    called the way mmcv/ops/modulated_deform_conv.py:172-213 calls it."""
+    import torch
+    ext = load_reference_ext()
+    if ext is None or not hasattr(ext, 'modulated_deform_conv_backward'):
+        raise RuntimeError('oracle/_ref is not built (or predates the backward binding)')
+    (sh, sw), (ph, pw), (dh, dw) = _pair(stride), _pair(padding), _pair(dilation)
+    kh, kw = weight.shape[2:]
+    bias = input.new_zeros(weight.shape[0]) if with_bias else input.new_empty(0)
+    g_in, g_off, g_mask = torch.zeros_like(input), torch.zeros_like(offset), torch.zeros_like(mask)
+    g_w, g_b = torch.zeros_like(weight), torch.zeros_like(bias)
+    ext.modulated_deform_conv_backward(
+        input.contiguous(), weight.contiguous(), bias, input.new_empty(0),
+        offset.contiguous(), mask.contiguous(), input.new_empty(0), g_in, g_w, g_b,
+        g_off, g_mask, grad_output.contiguous(), kernel_h=kh, kernel_w=kw,
+        stride_h=sh, stride_w=sw, pad_h=ph, pad_w=pw, dilation_h=dh, dilation_w=dw,
+        group=groups, deformable_group=deform_groups, with_bias=with_bias)
+    return g_in, g_off, g_mask, g_w, (g_b if with_bias else None)
 
 
 def load_reference_ext():

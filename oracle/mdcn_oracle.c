@@ -28,12 +28,14 @@
 #define T float
 #define FN(name) MDCN_CAT(mdcn_oracle_f32_, name)
 #include "mdcn_oracle_impl.h"
+#include "mdcn_oracle_bwd_impl.h"
 #undef T
 #undef FN
 
 #define T double
 #define FN(name) MDCN_CAT(mdcn_oracle_f64_, name)
 #include "mdcn_oracle_impl.h"
+#include "mdcn_oracle_bwd_impl.h"
 #undef T
 #undef FN
 
