@@ -161,6 +161,39 @@ int mdcn_pack_forward(const mdcn_pack_params *p, void *hip_stream);
  * repacks, ms[2] main kernel, ms[3] total, ms[4] conv_offset.  For measurement only. */
 int mdcn_pack_forward_timed(const mdcn_pack_params *p, void *hip_stream, float ms[5]);
 
+/*
+ * Backward of mdcn_forward(): replaces the body of
+ * modulated_deform_conv_backward_fallthrough for device tensors
+ * (mmcv/ops/csrc/pytorch/modulated_deform_conv.cpp:140-251) and, with
+ * conv.mask == NULL, of deform_conv_backward_input / _parameters
+ * (mmcv/ops/csrc/pytorch/deform_conv.cpp:262-525).  `conv` holds the forward's
+ * input, offset, mask, weight and geometry (bias and output are not read);
+ * grad_output is (N, Cout, Ho, Wo).  Every gradient that is not NULL is written
+ * in full (not accumulated into): grad_input like input, grad_offset like
+ * offset, grad_mask like mask (must be NULL when conv.mask is), grad_weight like
+ * weight, grad_bias (Cout).  grad_input and grad_offset/grad_mask are produced
+ * together: pass all of them or none.  Sums are formed in fp32 and rounded once.
+ * The scatter into grad_input and the pixel reduction of grad_weight use
+ * floating-point atomics, so results vary in the last bits from run to run, as
+ * the reference's CUDA kernels' do.
+ */
+typedef struct mdcn_bwd_params {
+  mdcn_params conv;
+  const void *grad_output;
+  void *grad_input;
+  void *grad_offset;
+  void *grad_mask;
+  void *grad_weight;
+  void *grad_bias;
+} mdcn_bwd_params;
+
+/* Bytes of device scratch mdcn_backward() needs (fp32 staging of grad_input and
+ * grad_weight for 16-bit tensors); may be 0. */
+size_t mdcn_backward_workspace_bytes(const mdcn_bwd_params *p);
+
+/* Enqueue the backward on `hip_stream`.  Returns an mdcn_status. */
+int mdcn_backward(const mdcn_bwd_params *p, void *hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -16,7 +16,7 @@ MDCN_OK = 0
 EXPORTS = ('mdcn_abi_version', 'mdcn_status_string', 'mdcn_output_size',
            'mdcn_fused_eligible', 'mdcn_workspace_bytes', 'mdcn_forward',
            'mdcn_forward_timed', 'mdcn_pack_workspace_bytes', 'mdcn_pack_forward',
-           'mdcn_pack_forward_timed')
+           'mdcn_pack_forward_timed', 'mdcn_backward_workspace_bytes', 'mdcn_backward')
 
 
 class MdcnParams(ctypes.Structure):
@@ -33,6 +33,12 @@ class MdcnPackParams(ctypes.Structure):
     _fields_ = [('conv', MdcnParams), ('offset_weight', ctypes.c_void_p),
                 ('offset_bias', ctypes.c_void_p), ('raw', ctypes.c_void_p),
                 ('unmodulated', ctypes.c_int32)]
+
+
+class MdcnBwdParams(ctypes.Structure):
+    _fields_ = [('conv', MdcnParams)] + [(n, ctypes.c_void_p) for n in
+                                         ('grad_output', 'grad_input', 'grad_offset', 'grad_mask',
+                                          'grad_weight', 'grad_bias')]
 
 
 _lib = None
@@ -68,6 +74,11 @@ def load():
         lib.mdcn_pack_forward_timed.restype = ctypes.c_int
         lib.mdcn_pack_forward_timed.argtypes = [PP, ctypes.c_void_p,
                                                 ctypes.POINTER(ctypes.c_float)]
+        BP = ctypes.POINTER(MdcnBwdParams)
+        lib.mdcn_backward_workspace_bytes.restype = ctypes.c_size_t
+        lib.mdcn_backward_workspace_bytes.argtypes = [BP]
+        lib.mdcn_backward.restype = ctypes.c_int
+        lib.mdcn_backward.argtypes = [BP, ctypes.c_void_p]
         _lib = lib
     return _lib
 

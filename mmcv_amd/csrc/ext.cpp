@@ -356,21 +356,100 @@ void deform_conv_forward(Tensor input, Tensor weight, Tensor offset, Tensor outp
   TORCH_CHECK(rc == MDCN_OK, op, ": ", mdcn_status_string(rc));
 }
 
-void deform_conv_backward_input(Tensor input, Tensor offset, Tensor gradOutput, Tensor gradInput,
-                                Tensor gradOffset, Tensor weight, Tensor columns, int kW, int kH,
-                                int dW, int dH, int padW, int padH, int dilationW, int dilationH,
-                                int group, int deformable_group, int im2col_step) {
-  TORCH_CHECK(false, "deform_conv_backward_input: this build implements the forward pass only");
+// Shared by the three backward ops: checks, contiguity, workspace and the call.
+// Tensors with zero elements stand for "not wanted".
+void run_backward(const char *op, const Tensor &input, const Tensor &weight, const Tensor &offset,
+                  const Tensor &mask, const Tensor &grad_output, Tensor grad_input,
+                  Tensor grad_offset, Tensor grad_mask, Tensor grad_weight, Tensor grad_bias,
+                  int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w,
+                  int dilation_h, int dilation_w, int group, int deformable_group) {
+  TORCH_CHECK(input.dim() == 4 && weight.dim() == 4 && offset.dim() == 4 && grad_output.dim() == 4, op,
+              " expects 4-D input, weight, offset and grad_output");
+  const at::Device dev = input.device();
+  TORCH_CHECK(dev.is_cuda(), op, ": implementation for device ", device_str(dev), " not found.");
+  c10::DeviceGuard guard(dev);
+  TORCH_CHECK(weight.size(2) == kernel_h && weight.size(3) == kernel_w,
+              "Input shape and kernel shape won't match: (", kernel_h, " x ", kernel_w, " vs ",
+              weight.size(2), " x ", weight.size(3), ").");
+  TORCH_CHECK(input.size(1) == weight.size(1) * group, "Input shape and kernel channels won't match: (",
+              input.size(1), " vs ", weight.size(1) * group, ").");
+  const auto st = input.scalar_type();
+  const Tensor *all[] = {&weight, &offset, &mask, &grad_output, &grad_input, &grad_offset,
+                         &grad_mask, &grad_weight, &grad_bias};
+  const char *names[] = {"weight", "offset", "mask", "grad_output", "grad_input", "grad_offset",
+                         "grad_mask", "grad_weight", "grad_bias"};
+  for (int i = 0; i < 9; ++i) {
+    if (all[i]->numel() == 0) continue;
+    TORCH_CHECK(all[i]->device() == dev, op, ": at param ", names[i], ", inconsistent device: ",
+                device_str(all[i]->device()), " vs ", device_str(dev));
+    TORCH_CHECK(all[i]->scalar_type() == st, op, ": expected ", names[i], " to have dtype ",
+                c10::toString(st), " but got ", c10::toString(all[i]->scalar_type()));
+    if (i >= 4) TORCH_CHECK(all[i]->is_contiguous(), op, ": ", names[i], " must be contiguous");
+  }
+  mdcn_bwd_params bp{};
+  mdcn_params &p = bp.conv;
+  p.dtype = mdcn_dtype_of(input);
+  p.N = (int)input.size(0); p.Cin = (int)input.size(1); p.H = (int)input.size(2); p.W = (int)input.size(3);
+  p.Cout = (int)weight.size(0); p.kh = kernel_h; p.kw = kernel_w;
+  p.sh = stride_h; p.sw = stride_w; p.ph = pad_h; p.pw = pad_w; p.dh = dilation_h; p.dw = dilation_w;
+  p.groups = group; p.dgroups = deformable_group;
+  int32_t Ho = 0, Wo = 0;
+  int rc = mdcn_output_size(&p, &Ho, &Wo);
+  TORCH_CHECK(rc == MDCN_OK, op, ": ", mdcn_status_string(rc));
+  const int64_t taps = (int64_t)kernel_h * kernel_w;
+  TORCH_CHECK(grad_output.size(0) == p.N && grad_output.size(1) == p.Cout && grad_output.size(2) == Ho &&
+                  grad_output.size(3) == Wo,
+              op, ": grad_output must be (", p.N, ", ", p.Cout, ", ", Ho, ", ", Wo, "), got ",
+              grad_output.sizes());
+  TORCH_CHECK(offset.size(0) == p.N && offset.size(1) == deformable_group * 2 * taps &&
+                  offset.size(2) == Ho && offset.size(3) == Wo,
+              op, ": offset must be (", p.N, ", ", deformable_group * 2 * taps, ", ", Ho, ", ", Wo,
+              "), got ", offset.sizes());
+  const bool modulated = mask.numel() > 0;
+  if (modulated)
+    TORCH_CHECK(mask.size(0) == p.N && mask.size(1) == deformable_group * taps && mask.size(2) == Ho &&
+                    mask.size(3) == Wo,
+                op, ": mask must be (", p.N, ", ", deformable_group * taps, ", ", Ho, ", ", Wo, "), got ",
+                mask.sizes());
+  auto same = [&](const Tensor &grad, const Tensor &like, const char *name) {
+    TORCH_CHECK(grad.numel() == 0 || grad.numel() == like.numel(), op, ": ", name, " has ", grad.numel(),
+                " elements, expected ", like.numel());
+  };
+  same(grad_input, input, "grad_input");
+  same(grad_offset, offset, "grad_offset");
+  same(grad_mask, mask, "grad_mask");
+  same(grad_weight, weight, "grad_weight");
+  TORCH_CHECK(grad_bias.numel() == 0 || grad_bias.numel() == p.Cout, op, ": grad_bias must have ", p.Cout,
+              " elements");
+  std::vector<Tensor> keep = {input.contiguous(), offset.contiguous(), weight.contiguous(),
+                              grad_output.contiguous()};
+  p.input = keep[0].data_ptr();
+  p.offset = keep[1].data_ptr();
+  p.weight = keep[2].data_ptr();
+  bp.grad_output = keep[3].data_ptr();
+  if (modulated) {
+    keep.push_back(mask.contiguous());
+    p.mask = keep.back().data_ptr();
+  }
+  auto ptr = [](Tensor &t) { return t.numel() ? t.data_ptr() : nullptr; };
+  bp.grad_input = ptr(grad_input);
+  bp.grad_offset = ptr(grad_offset);
+  bp.grad_mask = ptr(grad_mask);
+  bp.grad_weight = ptr(grad_weight);
+  bp.grad_bias = ptr(grad_bias);
+  const size_t ws = mdcn_backward_workspace_bytes(&bp);
+  if (ws > 0) {
+    keep.push_back(at::empty({(int64_t)ws}, input.options().dtype(at::kByte)));
+    p.workspace = keep.back().data_ptr();
+    p.workspace_bytes = ws;
+  }
+  rc = mdcn_backward(&bp, (void *)c10::hip::getCurrentHIPStream().stream());
+  TORCH_CHECK(rc == MDCN_OK, op, ": ", mdcn_status_string(rc));
 }
 
-void deform_conv_backward_parameters(Tensor input, Tensor offset, Tensor gradOutput,
-                                     Tensor gradWeight, Tensor columns, Tensor ones, int kW, int kH,
-                                     int dW, int dH, int padW, int padH, int dilationW,
-                                     int dilationH, int group, int deformable_group, float scale,
-                                     int im2col_step) {
-  TORCH_CHECK(false, "deform_conv_backward_parameters: this build implements the forward pass only");
-}
-
+// mmcv/ops/csrc/pytorch/modulated_deform_conv.cpp:140-251.  The reference adds
+// into the gradient tensors its caller hands over freshly zeroed
+// (mmcv/ops/modulated_deform_conv.py:177-181); here they are overwritten.
 void modulated_deform_conv_backward(
     Tensor input, Tensor weight, Tensor bias, Tensor ones, Tensor offset,
     Tensor mask, Tensor columns, Tensor grad_input, Tensor grad_weight,
@@ -378,9 +457,47 @@ void modulated_deform_conv_backward(
     int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h,
     int pad_w, int dilation_h, int dilation_w, int group, int deformable_group,
     const bool with_bias) {
-  TORCH_CHECK(false,
-              "modulated_deform_conv_backward: this build implements the forward "
-              "pass only");
+  (void)bias;
+  (void)ones;
+  (void)columns;
+  run_backward("modulated_deform_conv_backward", input, weight, offset, mask, grad_output, grad_input,
+               grad_offset, grad_mask, grad_weight, with_bias ? grad_bias : Tensor(at::empty({0}, input.options())),
+               kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w, dilation_h, dilation_w, group,
+               deformable_group);
+}
+
+// mmcv/ops/csrc/pytorch/deform_conv.cpp:262-384: gradients of the unmodulated
+// convolution with respect to input and offset.
+void deform_conv_backward_input(Tensor input, Tensor offset, Tensor gradOutput, Tensor gradInput,
+                                Tensor gradOffset, Tensor weight, Tensor columns, int kW, int kH,
+                                int dW, int dH, int padW, int padH, int dilationW, int dilationH,
+                                int group, int deformable_group, int im2col_step) {
+  (void)columns;
+  TORCH_CHECK(im2col_step > 0 && input.size(0) % im2col_step == 0,
+              "deform_conv_backward_input: batch size must be divisible by im2col_step");
+  const Tensor none = at::empty({0}, input.options());
+  run_backward("deform_conv_backward_input", input, weight, offset, none, gradOutput, gradInput,
+               gradOffset, none, none, none, kH, kW, dH, dW, padH, padW, dilationH, dilationW, group,
+               deformable_group);
+}
+
+// mmcv/ops/csrc/pytorch/deform_conv.cpp:386-525: gradWeight += scale * (gradient
+// with respect to the weight).
+void deform_conv_backward_parameters(Tensor input, Tensor offset, Tensor gradOutput,
+                                     Tensor gradWeight, Tensor columns, Tensor ones, int kW, int kH,
+                                     int dW, int dH, int padW, int padH, int dilationW,
+                                     int dilationH, int group, int deformable_group, float scale,
+                                     int im2col_step) {
+  (void)columns;
+  (void)ones;
+  TORCH_CHECK(im2col_step > 0 && input.size(0) % im2col_step == 0,
+              "deform_conv_backward_parameters: batch size must be divisible by im2col_step");
+  const Tensor none = at::empty({0}, input.options());
+  Tensor gw = at::empty_like(gradWeight, gradWeight.options(), at::MemoryFormat::Contiguous);
+  run_backward("deform_conv_backward_parameters", input, gradWeight, offset, none, gradOutput, none,
+               none, none, gw, none, kH, kW, dH, dW, padH, padW, dilationH, dilationW, group,
+               deformable_group);
+  gradWeight.add_(gw, scale);
 }
 
 }  // namespace

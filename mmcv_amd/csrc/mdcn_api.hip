@@ -9,6 +9,7 @@
 
 #include "mdcn_common.h"
 #include "mdcn_direct.h"
+#include "mdcn_backward.h"
 #include "mdcn_fused.h"
 #include "mdcn_oconv.h"
 #include "mdcn_prepass.h"
@@ -433,6 +434,92 @@ int run(const mdcn_params *p, void *stream, float *ms, const mdcn_pack_params *p
   }
 }
 
+struct BwdPlan {
+  size_t gin_bytes, gw_bytes;  // fp32 staging (0 for fp32 tensors)
+};
+
+void make_bwd_plan(const mdcn_bwd_params *bp, const Geom &g, BwdPlan *pl) {
+  const bool staged = bp->conv.dtype != MDCN_F32;
+  pl->gin_bytes = (staged && bp->grad_input) ? align_up((size_t)g.N * g.Cin * g.H * g.W * 4) : 0;
+  pl->gw_bytes = (staged && bp->grad_weight) ? align_up((size_t)g.Cout * g.cin_g * g.taps * 4) : 0;
+}
+
+template <typename E>
+int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &pl, hipStream_t st) {
+  const mdcn_params *p = &bp->conv;
+  const long plane_out = (long)g.Ho * g.Wo;
+  const OffMaskView om = dense_view(p->offset, p->mask, g);
+  unsigned char *ws = (unsigned char *)p->workspace;
+  auto blocks_for = [](long n) { return (int)std::min<long>((n + 255) / 256, 1L << 20); };
+  int rc = MDCN_OK;
+  auto check = [&]() { if (hipGetLastError() != hipSuccess) rc = MDCN_ERR_LAUNCH; };
+
+  if (bp->grad_input) {
+    const long n_in = (long)g.N * g.Cin * g.H * g.W;
+    float *gin32 = pl.gin_bytes ? (float *)ws : (float *)bp->grad_input;
+    hipLaunchKernelGGL(fill_zero_kernel<float>, dim3(blocks_for(n_in)), dim3(256), 0, st, gin32, n_in);
+    check();
+    const long total = (long)g.N * g.DG * g.taps * plane_out;
+    hipLaunchKernelGGL(bwd_data_kernel<E>, dim3(blocks_for(total)), dim3(256), 0, st, g,
+                       (const E *)p->input, om, (const E *)p->weight, (const E *)bp->grad_output,
+                       gin32, (E *)bp->grad_offset, (E *)bp->grad_mask, total);
+    check();
+    if (pl.gin_bytes) {
+      hipLaunchKernelGGL(round_kernel<E>, dim3(blocks_for(n_in)), dim3(256), 0, st, gin32,
+                         (E *)bp->grad_input, n_in);
+      check();
+    }
+  }
+  if (bp->grad_weight) {
+    const long n_w = (long)g.Cout * g.cin_g * g.taps;
+    float *gw32 = pl.gw_bytes ? (float *)(ws + pl.gin_bytes) : (float *)bp->grad_weight;
+    hipLaunchKernelGGL(fill_zero_kernel<float>, dim3(blocks_for(n_w)), dim3(256), 0, st, gw32, n_w);
+    check();
+    BwdWeightArgs wa;
+    wa.g = g;
+    wa.input = p->input;
+    wa.om = om;
+    wa.gout = bp->grad_output;
+    wa.gw32 = gw32;
+    wa.k_tiles = (g.cin_g * g.taps + 63) / 64;
+    wa.co_tiles = (g.cout_g + 255) / 256;
+    wa.px_chunks = (int)((plane_out + 63) / 64);
+    const long tiles = (long)wa.k_tiles * wa.co_tiles * g.G;
+    const long work = (long)g.N * wa.px_chunks;
+    wa.splits = (int)std::max<long>(1, std::min<long>(work, (4L * num_cus() + tiles - 1) / tiles));
+    wa.g_vec_ok = (plane_out % (16 / (long)sizeof(E)) == 0) && (((uintptr_t)bp->grad_output % 16) == 0);
+    hipLaunchKernelGGL(bwd_weight_kernel<E>, dim3((unsigned)tiles, (unsigned)wa.splits), dim3(256), 0,
+                       st, wa);
+    check();
+    if (pl.gw_bytes) {
+      hipLaunchKernelGGL(round_kernel<E>, dim3(blocks_for(n_w)), dim3(256), 0, st, gw32,
+                         (E *)bp->grad_weight, n_w);
+      check();
+    }
+  }
+  if (bp->grad_bias) {
+    hipLaunchKernelGGL(bwd_bias_kernel<E>, dim3(g.Cout), dim3(256), 0, st, g,
+                       (const E *)bp->grad_output, (E *)bp->grad_bias);
+    check();
+  }
+  return rc;
+}
+
+int check_bwd(const mdcn_bwd_params *bp, Geom *g, bool need_ptrs) {
+  if (!bp) return MDCN_ERR_NULL;
+  const mdcn_params *p = &bp->conv;
+  int rc = check_params(p, g, false);
+  if (rc != MDCN_OK) return rc;
+  if (!need_ptrs) return MDCN_OK;
+  if (!p->input || !p->offset || !p->weight || !bp->grad_output) return MDCN_ERR_NULL;
+  // grad_input and the offset/mask gradients come out of one kernel
+  const bool data = bp->grad_input != nullptr;
+  if (data != (bp->grad_offset != nullptr)) return MDCN_ERR_NULL;
+  if (p->mask ? (data != (bp->grad_mask != nullptr)) : (bp->grad_mask != nullptr)) return MDCN_ERR_NULL;
+  if ((uint64_t)g->N * g->DG * g->taps * g->Ho * g->Wo > 0x7fffffffffffull) return MDCN_ERR_TOO_LARGE;
+  return MDCN_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -496,6 +583,32 @@ size_t mdcn_pack_workspace_bytes(const mdcn_pack_params *pp) {
 int mdcn_pack_forward(const mdcn_pack_params *pp, void *hip_stream) {
   if (!pp) return MDCN_ERR_NULL;
   return run(&pp->conv, hip_stream, nullptr, pp);
+}
+
+size_t mdcn_backward_workspace_bytes(const mdcn_bwd_params *bp) {
+  Geom g;
+  if (check_bwd(bp, &g, false) != MDCN_OK) return 0;
+  BwdPlan pl;
+  make_bwd_plan(bp, g, &pl);
+  return pl.gin_bytes + pl.gw_bytes;
+}
+
+int mdcn_backward(const mdcn_bwd_params *bp, void *hip_stream) {
+  Geom g;
+  const int rc = check_bwd(bp, &g, true);
+  if (rc != MDCN_OK) return rc;
+  BwdPlan pl;
+  make_bwd_plan(bp, g, &pl);
+  const size_t need = pl.gin_bytes + pl.gw_bytes;
+  const mdcn_params *p = &bp->conv;
+  if (need > 0 && (!p->workspace || p->workspace_bytes < need || ((uintptr_t)p->workspace % kAlign) != 0))
+    return MDCN_ERR_WORKSPACE;
+  hipStream_t st = (hipStream_t)hip_stream;
+  switch (p->dtype) {
+    case MDCN_F32: return run_backward_typed<float>(bp, g, pl, st);
+    case MDCN_F16: return run_backward_typed<f16_t>(bp, g, pl, st);
+    default: return run_backward_typed<bf16_t>(bp, g, pl, st);
+  }
 }
 
 int mdcn_pack_forward_timed(const mdcn_pack_params *pp, void *hip_stream, float ms[5]) {

@@ -1,0 +1,309 @@
+// Backward of the (modulated) deformable convolution: gradients with respect to
+// input, offset, mask, weight and bias
+// (mmcv/ops/csrc/pytorch/modulated_deform_conv.cpp:140-251 and the kernels
+// cpu/modulated_deform_conv.cpp:34-107,170-320).  The reference materialises the
+// column gradient W^T * grad_output per sample and runs three element-wise
+// kernels and two library GEMMs over it; here nothing of column size reaches
+// memory:
+//   bwd_data_kernel    one thread per (image, deformable group, tap, output
+//                      pixel): builds the column gradients of its channels on
+//                      the fly and turns them into grad_offset, grad_mask (plain
+//                      stores, every element has one owner) and grad_input
+//                      (fp32 atomics, four corners per channel),
+//   bwd_weight_kernel  grad_weight = grad_output * columns^T as an MFMA GEMM
+//                      whose reduction runs over pixels; the columns tile is
+//                      sampled into LDS and never stored,
+//   bwd_bias_kernel    row sums of grad_output.
+// Accumulation is fp32 throughout; 16-bit tensors receive their gradients through
+// fp32 staging buffers in the workspace (round_kernel).
+#pragma once
+
+#include "mdcn_common.h"
+#include "mdcn_fused.h"
+
+namespace mdcn {
+
+template <typename T>
+__global__ __launch_bounds__(256) void fill_zero_kernel(T *p, long n) {
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
+    p[i] = (T)0;
+}
+
+template <typename E>
+__global__ __launch_bounds__(256) void round_kernel(const float *__restrict__ src, E *__restrict__ dst,
+                                                    long n) {
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
+    dst[i] = from_f32<E>(src[i]);
+}
+
+// grad_bias[co] = sum over images and pixels of grad_output[:, co] (one block per channel).
+template <typename E>
+__global__ __launch_bounds__(256) void bwd_bias_kernel(Geom g, const E *__restrict__ gout,
+                                                       E *__restrict__ gbias) {
+  __shared__ float part[256];
+  const int co = blockIdx.x;
+  const long plane = (long)g.Ho * g.Wo;
+  float s = 0.0f;
+  for (int n = 0; n < g.N; ++n) {
+    const E *row = gout + ((long)n * g.Cout + co) * plane;
+    for (long p = threadIdx.x; p < plane; p += 256) s += to_f32(row[p]);
+  }
+  part[threadIdx.x] = s;
+  __syncthreads();
+  for (int w = 128; w > 0; w >>= 1) {
+    if ((int)threadIdx.x < w) part[threadIdx.x] += part[threadIdx.x + w];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) gbias[co] = from_f32<E>(part[0]);
+}
+
+// Channels whose column gradient a thread of bwd_data_kernel holds at a time.
+constexpr int kBwdChunk = 16;
+
+// One thread per (n, dg, tap, pixel).  For its channels, kBwdChunk at a time:
+//   d[c] = sum_co weight[co, c, tap] * grad_output[n, co, pixel]    (the column gradient)
+//   grad_mask   += d[c] * bilinear(x[c], pos)
+//   grad_offset += d[c] * mask * d(bilinear)/d(pos)                  (y, then x)
+//   grad_input[c, corner] += d[c] * mask * corner weight             (atomics)
+// with the forward's sampling rule: nothing for a position outside (-1,H)x(-1,W),
+// no contribution from a corner outside the image
+// (cpu/modulated_deform_conv.cpp:34-107,170-320).
+template <typename E>
+__global__ __launch_bounds__(256) void bwd_data_kernel(Geom g, const E *__restrict__ input,
+                                                       OffMaskView om, const E *__restrict__ weight,
+                                                       const E *__restrict__ gout,
+                                                       float *__restrict__ gin32, E *__restrict__ goff,
+                                                       E *__restrict__ gmask, long total) {
+  const long plane_out = (long)g.Ho * g.Wo;
+  const long plane_in = (long)g.H * g.W;
+  for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (long)gridDim.x * blockDim.x) {
+    const long pix = idx % plane_out;
+    long r = idx / plane_out;
+    const int tap = (int)(r % g.taps);
+    r /= g.taps;
+    const int dgi = (int)(r % g.DG);
+    const int n = (int)(r / g.DG);
+    const int ho = (int)(pix / g.Wo), wo = (int)(pix - (long)ho * g.Wo);
+    const int ti = tap / g.kw, tj = tap - ti * g.kw;
+
+    const E *off = (const E *)om.off + (long)n * om.off_n + pix * om.off_px +
+                   (long)(dgi * 2 * g.taps) * om.off_ch;
+    const E *msk = (const E *)om.msk + (long)n * om.msk_n + pix * om.msk_px +
+                   (long)(dgi * g.taps) * om.msk_ch;
+    const float dy = to_f32(off[(long)(2 * tap) * om.off_ch]);
+    const float dx = to_f32(off[(long)(2 * tap + 1) * om.off_ch]);
+    const float m = mask_value<E>(msk[(long)tap * om.msk_ch], om.logit);
+    const float py = (float)(ho * g.sh - g.ph + ti * g.dh) + dy;
+    const float px = (float)(wo * g.sw - g.pw + tj * g.dw) + dx;
+    const bool inside = (py > -1.0f) && (px > -1.0f) && (py < (float)g.H) && (px < (float)g.W);
+
+    float acc_m = 0.0f, acc_y = 0.0f, acc_x = 0.0f;
+    if (inside) {
+      const float fy = floorf(py), fx = floorf(px);
+      const int y0 = (int)fy, x0 = (int)fx, y1 = y0 + 1, x1 = x0 + 1;
+      const float ly = py - fy, lx = px - fx, hy = 1.0f - ly, hx = 1.0f - lx;
+      const bool ok00 = y0 >= 0 && x0 >= 0, ok01 = y0 >= 0 && x1 <= g.W - 1;
+      const bool ok10 = y1 <= g.H - 1 && x0 >= 0, ok11 = y1 <= g.H - 1 && x1 <= g.W - 1;
+      const long o00 = (long)y0 * g.W + x0, o01 = o00 + 1, o10 = o00 + g.W, o11 = o10 + 1;
+
+      const int c_begin = dgi * g.ch_per_dg, c_end = c_begin + g.ch_per_dg;
+      for (int c0 = c_begin; c0 < c_end;) {
+        // a chunk stays inside one convolution group
+        const int grp = c0 / g.cin_g;
+        const int cn = min(kBwdChunk, min(c_end, (grp + 1) * g.cin_g) - c0);
+        float d[kBwdChunk];
+#pragma unroll
+        for (int cc = 0; cc < kBwdChunk; ++cc) d[cc] = 0.0f;
+        const E *grow = gout + ((long)n * g.Cout + (long)grp * g.cout_g) * plane_out + pix;
+        const E *wrow = weight + ((long)grp * g.cout_g * g.cin_g + (c0 - grp * g.cin_g)) * g.taps + tap;
+        for (int co = 0; co < g.cout_g; ++co) {
+          const float gv = to_f32(grow[(long)co * plane_out]);
+          const E *wc = wrow + (long)co * g.cin_g * g.taps;
+#pragma unroll
+          for (int cc = 0; cc < kBwdChunk; ++cc)
+            if (cc < cn) d[cc] += to_f32(wc[(long)cc * g.taps]) * gv;
+        }
+#pragma unroll
+        for (int cc = 0; cc < kBwdChunk; ++cc) {
+          if (cc < cn) {
+            const int c = c0 + cc;
+            const E *im = input + ((long)n * g.Cin + c) * plane_in;
+            const float v00 = ok00 ? to_f32(im[o00]) : 0.0f, v01 = ok01 ? to_f32(im[o01]) : 0.0f;
+            const float v10 = ok10 ? to_f32(im[o10]) : 0.0f, v11 = ok11 ? to_f32(im[o11]) : 0.0f;
+            const float dc = d[cc];
+            acc_m += dc * ((hy * hx) * v00 + (hy * lx) * v01 + (ly * hx) * v10 + (ly * lx) * v11);
+            acc_y += dc * (hx * (v10 - v00) + lx * (v11 - v01));
+            acc_x += dc * (hy * (v01 - v00) + ly * (v11 - v10));
+            const float t = dc * m;
+            float *gi = gin32 + ((long)n * g.Cin + c) * plane_in;
+            if (ok00) unsafeAtomicAdd(gi + o00, (hy * hx) * t);
+            if (ok01) unsafeAtomicAdd(gi + o01, (hy * lx) * t);
+            if (ok10) unsafeAtomicAdd(gi + o10, (ly * hx) * t);
+            if (ok11) unsafeAtomicAdd(gi + o11, (ly * lx) * t);
+          }
+        }
+        c0 += cn;
+      }
+    }
+    const long ob = ((long)n * g.DG + dgi) * 2 * g.taps;
+    goff[(ob + 2 * tap) * plane_out + pix] = from_f32<E>(acc_y * m);
+    goff[(ob + 2 * tap + 1) * plane_out + pix] = from_f32<E>(acc_x * m);
+    if (gmask) gmask[(((long)n * g.DG + dgi) * g.taps + tap) * plane_out + pix] = from_f32<E>(acc_m);
+  }
+}
+
+struct BwdWeightArgs {
+  Geom g;
+  const void *input;
+  OffMaskView om;
+  const void *gout;
+  float *gw32;       // (Cout, cin_g, kh, kw) fp32, zero before the launch
+  int k_tiles;       // ceil(cin_g * taps / 64)
+  int co_tiles;      // ceil(cout_g / 256)
+  int px_chunks;     // 64-pixel chunks per image
+  int splits;        // workgroups sharing the (image, chunk) range of one tile
+  int g_vec_ok;      // grad_output rows may be read 16 bytes at a time
+};
+
+// grad_weight[co, k] += sum_pixels grad_output[co, pixel] * col[k, pixel], k = (channel, tap)
+// of one group.  Workgroup = 256 output channels x 64 k of one group, for a share
+// of the (image, 64-pixel chunk) range; wave w owns channels 64w..64w+63 as 2x2
+// MFMA blocks.  Per chunk the 256 threads sample the 64 x 64 columns tile into
+// LDS (element type E, rows of 64 pixels, 16-byte chunks swizzled by row), then
+// A fragments (channel row, 16 bytes of pixels) come straight from grad_output
+// and B fragments (k row, 16 bytes of pixels) from LDS.  The partial sums leave
+// through fp32 atomics.
+template <typename E>
+__global__ __launch_bounds__(256) void bwd_weight_kernel(BwdWeightArgs a) {
+  using TR = ElemTraits<E>;
+  constexpr int ES = (int)sizeof(E);
+  constexpr int PXC = 16 / ES;          // pixels per 16-byte chunk
+  constexpr int NCH = 64 / PXC;         // chunks per 64-pixel row
+  __shared__ uint4 colT[64 * NCH];
+  const Geom &g = a.g;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int frow = lane & 31, fhalf = lane >> 5;
+  const long plane_out = (long)g.Ho * g.Wo;
+  const long plane_in = (long)g.H * g.W;
+  const int k_g = g.cin_g * g.taps;
+
+  int b = blockIdx.x;
+  const int kt = b % a.k_tiles;
+  b /= a.k_tiles;
+  const int ct = b % a.co_tiles;
+  const int grp = b / a.co_tiles;
+  const int split = blockIdx.y;
+
+  // the 16 columns rows this thread samples: k = kbase + tid / 64 + 4 * i
+  const int kbase = kt * 64;
+  const int spx = tid & 63;  // ... at pixel spx of the chunk
+  int s_c[16], s_tap[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int k = kbase + (tid >> 6) + 4 * i;
+    s_c[i] = k < k_g ? grp * g.cin_g + k / g.taps : -1;
+    s_tap[i] = k < k_g ? k % g.taps : 0;
+  }
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  const int co_base = ct * 256 + wave * 64;  // within the group
+  const E *gout = (const E *)a.gout;
+  const long work = (long)g.N * a.px_chunks;
+  for (long wi = split; wi < work; wi += a.splits) {
+    const int n = (int)(wi / a.px_chunks);
+    const int p0 = (int)(wi - (long)n * a.px_chunks) * 64;
+    // ---- columns tile -> LDS ----
+    {
+      const int p = p0 + spx;
+      const bool pv = p < plane_out;
+      const int ho = pv ? p / g.Wo : 0, wo = pv ? p - ho * g.Wo : 0;
+      E *c16 = (E *)colT;
+#pragma unroll 4
+      for (int i = 0; i < 16; ++i) {
+        const int kk = (tid >> 6) + 4 * i;
+        float v = 0.0f;
+        if (pv && s_c[i] >= 0) {
+          const int c = s_c[i], tap = s_tap[i];
+          const int dgi = c / g.ch_per_dg;
+          const int ti = tap / g.kw, tj = tap - ti * g.kw;
+          const E *off = (const E *)a.om.off + (long)n * a.om.off_n + (long)p * a.om.off_px +
+                         (long)(dgi * 2 * g.taps) * a.om.off_ch;
+          const E *msk = (const E *)a.om.msk + (long)n * a.om.msk_n + (long)p * a.om.msk_px +
+                         (long)(dgi * g.taps) * a.om.msk_ch;
+          const TapSample s = make_tap_sample(
+              ho * g.sh - g.ph + ti * g.dh, wo * g.sw - g.pw + tj * g.dw,
+              to_f32(off[(long)(2 * tap) * a.om.off_ch]), to_f32(off[(long)(2 * tap + 1) * a.om.off_ch]),
+              mask_value<E>(msk[(long)tap * a.om.msk_ch], a.om.logit), g.H, g.W);
+          if (s.inside) {
+            const E *im = (const E *)a.input + ((long)n * g.Cin + c) * plane_in;
+            const int y1 = s.y0 + 1, x1 = s.x0 + 1;
+            if (s.y0 >= 0 && s.x0 >= 0) v += s.w00 * to_f32(im[s.y0 * g.W + s.x0]);
+            if (s.y0 >= 0 && x1 <= g.W - 1) v += s.w01 * to_f32(im[s.y0 * g.W + x1]);
+            if (y1 <= g.H - 1 && s.x0 >= 0) v += s.w10 * to_f32(im[y1 * g.W + s.x0]);
+            if (y1 <= g.H - 1 && x1 <= g.W - 1) v += s.w11 * to_f32(im[y1 * g.W + x1]);
+          }
+        }
+        const int chunk = (spx / PXC) ^ (kk & (NCH - 1) & 7);
+        c16[(kk * NCH + chunk) * PXC + (spx % PXC)] = from_f32<E>(v);
+      }
+    }
+    __syncthreads();
+    // ---- MFMA over the 64 pixels ----
+#pragma unroll
+    for (int step = 0; step < NCH / 2; ++step) {
+      const int ch = step * 2 + fhalf;
+      uint4 af[2], bf[2];
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb) {
+        const int co = co_base + mb * 32 + frow;
+        const int p = p0 + ch * PXC;
+        af[mb] = make_uint4(0u, 0u, 0u, 0u);
+        if (co < g.cout_g) {
+          const E *row = gout + ((long)n * g.Cout + (long)grp * g.cout_g + co) * plane_out + p;
+          if (a.g_vec_ok && p + PXC <= plane_out) {
+            af[mb] = *(const uint4 *)row;
+          } else {
+            alignas(16) E tmp[PXC];
+#pragma unroll
+            for (int e = 0; e < PXC; ++e) tmp[e] = (p + e < plane_out) ? row[e] : from_f32<E>(0.0f);
+            af[mb] = *(const uint4 *)tmp;
+          }
+        }
+      }
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb) {
+        const int kk = nb * 32 + frow;
+        bf[nb] = colT[kk * NCH + (ch ^ (kk & (NCH - 1) & 7))];
+      }
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) TR::mma(acc[mb][nb], af[mb], bf[nb]);
+    }
+    __syncthreads();
+  }
+
+  // A rows = output channels, B rows = k: register r of lane l holds
+  //   channel = (r/4)*8 + (l/32)*4 + r%4,  k = l%32   of its block.
+#pragma unroll
+  for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int co = co_base + mb * 32 + (r >> 2) * 8 + fhalf * 4 + (r & 3);
+        const int k = kbase + nb * 32 + frow;
+        if (co < g.cout_g && k < k_g)
+          unsafeAtomicAdd(a.gw32 + ((long)grp * g.cout_g + co) * k_g + k, acc[mb][nb][r]);
+      }
+}
+
+}  // namespace mdcn

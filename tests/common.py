@@ -209,3 +209,38 @@ def capi_pack_forward(case, own_conv=True, raw=None, want_raw=False, path=capi.P
     assert rc == 0, capi.status_string(rc)
     torch.cuda.synchronize()
     return out, raw_out
+
+
+def capi_backward(case, grad_output, want_bias=True):
+    """mdcn_backward through ctypes on device tensors of `case` (mask None:
+    unmodulated); returns (grad_input, grad_offset, grad_mask or None, grad_weight,
+    grad_bias or None)."""
+    lib = capi.load()
+    x, off, msk, w = (case[k] for k in ('input', 'offset', 'mask', 'weight'))
+    N, Cin, H, W = x.shape
+    Cout, _, kh, kw = w.shape
+    bp = capi.MdcnBwdParams()
+    bp.conv = capi.make_params(DT[x.dtype], N, Cin, H, W, Cout, kh, kw, case['stride'], case['padding'],
+                               case['dilation'], case['groups'], case['deform_groups'])
+    p = bp.conv
+    keep = [t.contiguous() for t in (x, off, w, grad_output)]
+    p.input, p.offset, p.weight, bp.grad_output = (t.data_ptr() for t in keep)
+    g_in, g_off, g_w = torch.full_like(x, 7.0), torch.full_like(off, 7.0), torch.full_like(w, 7.0)
+    bp.grad_input, bp.grad_offset, bp.grad_weight = g_in.data_ptr(), g_off.data_ptr(), g_w.data_ptr()
+    g_mask = g_b = None
+    if msk is not None:
+        keep.append(msk.contiguous())
+        p.mask = keep[-1].data_ptr()
+        g_mask = torch.full_like(msk, 7.0)
+        bp.grad_mask = g_mask.data_ptr()
+    if want_bias:
+        g_b = torch.full((Cout,), 7.0, dtype=x.dtype, device=x.device)
+        bp.grad_bias = g_b.data_ptr()
+    ws_bytes = lib.mdcn_backward_workspace_bytes(ctypes.byref(bp))
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=x.device)
+    p.workspace = ws.data_ptr() if ws_bytes else None
+    p.workspace_bytes = ws_bytes
+    rc = lib.mdcn_backward(ctypes.byref(bp), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0, capi.status_string(rc)
+    torch.cuda.synchronize()
+    return g_in, g_off, g_mask, g_w, g_b

@@ -110,11 +110,11 @@ def test_module_behaviour():
     with torch.no_grad():
         ys = small(xs, torch.zeros(1, 18, 2, 5, device='cuda'))
     assert ys.shape == (1, 8, 2, 5)
-    # gradients are not implemented: the reference sequence runs and backward raises
+    # a gradient-requiring call takes the reference's two differentiable steps
     pack = DeformConv2dPack(64, 8, 3, padding=1).cuda()
-    out = pack(x.requires_grad_(True))
-    with pytest.raises(RuntimeError, match='forward pass only'):
-        out.sum().backward()
+    xg = x.clone().requires_grad_(True)
+    pack(xg).sum().backward()
+    assert xg.grad is not None and pack.weight.grad is not None and pack.conv_offset.bias.grad is not None
     # CPU tensors are refused
     with pytest.raises(RuntimeError, match='implementation for device cpu not found'):
         deform_conv2d(x.detach().cpu(), offset.cpu(), layer.weight.detach().cpu(), 1, 1, 1, 1, 2, False, 4)

@@ -145,10 +145,10 @@ def test_device_and_shape_errors():
     with pytest.raises(RuntimeError, match='not implemented for'):
         modulated_deform_conv2d(case['input'].double(), case['offset'].double(),
                                 case['mask'].double(), case['weight'].double(), None, 1, 1)
-    with pytest.raises(RuntimeError, match='forward pass only'):
-        x = case['input'].clone().requires_grad_(True)
-        modulated_deform_conv2d(x, case['offset'], case['mask'], case['weight'],
-                                None, 1, 1).sum().backward()
+    # gradients flow (their values are checked in test_gpu_backward.py)
+    x = case['input'].clone().requires_grad_(True)
+    modulated_deform_conv2d(x, case['offset'], case['mask'], case['weight'], None, 1, 1).sum().backward()
+    assert x.grad is not None and torch.isfinite(x.grad).all()
 
 
 # ---- the benchmark configurations at full size ----------------------------------

@@ -95,11 +95,13 @@ def test_module_fused_modes_agree():
         err = rel_err(_np(outs[mode]), _np(outs['none']))
         print(f'  fuse={mode}: {err:.2e}', flush=True)
         assert err <= TOL[torch.float32]
-    # a gradient-requiring call takes the reference sequence (and backward raises)
+    # a gradient-requiring call takes the reference sequence of differentiable ops
     layer.fuse = 'full'
-    y = layer(x.requires_grad_(True))
-    with pytest.raises(RuntimeError, match='forward pass only'):
-        y.sum().backward()
+    xg = x.clone().requires_grad_(True)
+    y = layer(xg)
+    assert rel_err(_np(y.detach()), _np(outs['none'])) == 0.0
+    y.sum().backward()
+    assert xg.grad is not None and layer.conv_offset.weight.grad is not None and layer.weight.grad is not None
 
 
 def test_zero_init_pack_is_plain_conv():
