@@ -459,10 +459,11 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
     float *gin32 = pl.gin_bytes ? (float *)ws : (float *)bp->grad_input;
     hipLaunchKernelGGL(fill_zero_kernel<float>, dim3(blocks_for(n_in)), dim3(256), 0, st, gin32, n_in);
     check();
-    const long total = (long)g.N * g.DG * g.taps * plane_out;
-    hipLaunchKernelGGL(bwd_data_kernel<E>, dim3(blocks_for(total)), dim3(256), 0, st, g,
-                       (const E *)p->input, om, (const E *)p->weight, (const E *)bp->grad_output,
-                       gin32, (E *)bp->grad_offset, (E *)bp->grad_mask, total);
+    const int rows = g.N * g.DG * g.taps;  // (image, deformable group, tap)
+    const dim3 grid((unsigned)((plane_out + 255) / 256), (unsigned)std::min(rows, 65535));
+    hipLaunchKernelGGL(bwd_data_kernel<E>, grid, dim3(256), 0, st, g, (const E *)p->input, om,
+                       (const E *)p->weight, (const E *)bp->grad_output, gin32,
+                       (E *)bp->grad_offset, (E *)bp->grad_mask, rows);
     check();
     if (pl.gin_bytes) {
       hipLaunchKernelGGL(round_kernel<E>, dim3(blocks_for(n_in)), dim3(256), 0, st, gin32,
@@ -516,7 +517,7 @@ int check_bwd(const mdcn_bwd_params *bp, Geom *g, bool need_ptrs) {
   const bool data = bp->grad_input != nullptr;
   if (data != (bp->grad_offset != nullptr)) return MDCN_ERR_NULL;
   if (p->mask ? (data != (bp->grad_mask != nullptr)) : (bp->grad_mask != nullptr)) return MDCN_ERR_NULL;
-  if ((uint64_t)g->N * g->DG * g->taps * g->Ho * g->Wo > 0x7fffffffffffull) return MDCN_ERR_TOO_LARGE;
+  if ((uint64_t)g->N * g->DG * g->taps > 0x7fffffffull) return MDCN_ERR_TOO_LARGE;
   return MDCN_OK;
 }
 

@@ -6,7 +6,7 @@
 // kernels and two library GEMMs over it; here nothing of column size reaches
 // memory:
 //   bwd_data_kernel    one thread per (image, deformable group, tap, output
-//                      pixel): builds the column gradients of its channels on
+//                      pixel), a workgroup sharing (image, group, tap): builds the column gradients of its channels on
 //                      the fly and turns them into grad_offset, grad_mask (plain
 //                      stores, every element has one owner) and grad_input
 //                      (fp32 atomics, four corners per channel),
@@ -59,32 +59,40 @@ __global__ __launch_bounds__(256) void bwd_bias_kernel(Geom g, const E *__restri
 
 // Channels whose column gradient a thread of bwd_data_kernel holds at a time.
 constexpr int kBwdChunk = 16;
+// Output channels of one weight slice staged in LDS at a time.
+constexpr int kBwdCoTile = 256;
 
-// One thread per (n, dg, tap, pixel).  For its channels, kBwdChunk at a time:
+// One workgroup per (n, dg, tap) and run of 256 output pixels, one thread per
+// pixel.  For the channels of the deformable group, kBwdChunk at a time:
 //   d[c] = sum_co weight[co, c, tap] * grad_output[n, co, pixel]    (the column gradient)
 //   grad_mask   += d[c] * bilinear(x[c], pos)
 //   grad_offset += d[c] * mask * d(bilinear)/d(pos)                  (y, then x)
 //   grad_input[c, corner] += d[c] * mask * corner weight             (atomics)
 // with the forward's sampling rule: nothing for a position outside (-1,H)x(-1,W),
 // no contribution from a corner outside the image
-// (cpu/modulated_deform_conv.cpp:34-107,170-320).
+// (cpu/modulated_deform_conv.cpp:34-107,170-320).  The weight slice
+// [co tile][chunk] of the workgroup's tap goes through LDS as fp32 and is read
+// back as broadcasts, so the inner loop costs one grad_output load and four LDS
+// reads per 16 multiply-adds.
 template <typename E>
 __global__ __launch_bounds__(256) void bwd_data_kernel(Geom g, const E *__restrict__ input,
                                                        OffMaskView om, const E *__restrict__ weight,
                                                        const E *__restrict__ gout,
                                                        float *__restrict__ gin32, E *__restrict__ goff,
-                                                       E *__restrict__ gmask, long total) {
+                                                       E *__restrict__ gmask, int rows) {
+  __shared__ float4 wl[kBwdCoTile][kBwdChunk / 4];
   const long plane_out = (long)g.Ho * g.Wo;
   const long plane_in = (long)g.H * g.W;
-  for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
-       idx += (long)gridDim.x * blockDim.x) {
-    const long pix = idx % plane_out;
-    long r = idx / plane_out;
-    const int tap = (int)(r % g.taps);
-    r /= g.taps;
-    const int dgi = (int)(r % g.DG);
-    const int n = (int)(r / g.DG);
-    const int ho = (int)(pix / g.Wo), wo = (int)(pix - (long)ho * g.Wo);
+  const int tid = threadIdx.x;
+  const long pix_raw = (long)blockIdx.x * 256 + tid;
+  const bool valid = pix_raw < plane_out;
+  const long pix = valid ? pix_raw : 0;
+  const int ho = (int)(pix / g.Wo), wo = (int)(pix - (long)ho * g.Wo);
+
+  for (int row = blockIdx.y; row < rows; row += gridDim.y) {  // row = (n, dg, tap), workgroup uniform
+    const int tap = row % g.taps;
+    const int dgi = (row / g.taps) % g.DG;
+    const int n = row / (g.taps * g.DG);
     const int ti = tap / g.kw, tj = tap - ti * g.kw;
 
     const E *off = (const E *)om.off + (long)n * om.off_n + pix * om.off_px +
@@ -96,34 +104,55 @@ __global__ __launch_bounds__(256) void bwd_data_kernel(Geom g, const E *__restri
     const float m = mask_value<E>(msk[(long)tap * om.msk_ch], om.logit);
     const float py = (float)(ho * g.sh - g.ph + ti * g.dh) + dy;
     const float px = (float)(wo * g.sw - g.pw + tj * g.dw) + dx;
-    const bool inside = (py > -1.0f) && (px > -1.0f) && (py < (float)g.H) && (px < (float)g.W);
+    const bool inside =
+        valid && (py > -1.0f) && (px > -1.0f) && (py < (float)g.H) && (px < (float)g.W);
+    const float fy = floorf(py), fx = floorf(px);
+    const int y0 = inside ? (int)fy : 0, x0 = inside ? (int)fx : 0, y1 = y0 + 1, x1 = x0 + 1;
+    const float ly = py - fy, lx = px - fx, hy = 1.0f - ly, hx = 1.0f - lx;
+    const bool ok00 = inside && y0 >= 0 && x0 >= 0, ok01 = inside && y0 >= 0 && x1 <= g.W - 1;
+    const bool ok10 = inside && y1 <= g.H - 1 && x0 >= 0, ok11 = inside && y1 <= g.H - 1 && x1 <= g.W - 1;
+    const long o00 = (long)y0 * g.W + x0, o01 = o00 + 1, o10 = o00 + g.W, o11 = o10 + 1;
 
     float acc_m = 0.0f, acc_y = 0.0f, acc_x = 0.0f;
-    if (inside) {
-      const float fy = floorf(py), fx = floorf(px);
-      const int y0 = (int)fy, x0 = (int)fx, y1 = y0 + 1, x1 = x0 + 1;
-      const float ly = py - fy, lx = px - fx, hy = 1.0f - ly, hx = 1.0f - lx;
-      const bool ok00 = y0 >= 0 && x0 >= 0, ok01 = y0 >= 0 && x1 <= g.W - 1;
-      const bool ok10 = y1 <= g.H - 1 && x0 >= 0, ok11 = y1 <= g.H - 1 && x1 <= g.W - 1;
-      const long o00 = (long)y0 * g.W + x0, o01 = o00 + 1, o10 = o00 + g.W, o11 = o10 + 1;
-
-      const int c_begin = dgi * g.ch_per_dg, c_end = c_begin + g.ch_per_dg;
-      for (int c0 = c_begin; c0 < c_end;) {
-        // a chunk stays inside one convolution group
-        const int grp = c0 / g.cin_g;
-        const int cn = min(kBwdChunk, min(c_end, (grp + 1) * g.cin_g) - c0);
-        float d[kBwdChunk];
+    const int c_begin = dgi * g.ch_per_dg, c_end = c_begin + g.ch_per_dg;
+    for (int c0 = c_begin; c0 < c_end;) {
+      // a chunk stays inside one convolution group
+      const int grp = c0 / g.cin_g;
+      const int cn = min(kBwdChunk, min(c_end, (grp + 1) * g.cin_g) - c0);
+      float d[kBwdChunk];
 #pragma unroll
-        for (int cc = 0; cc < kBwdChunk; ++cc) d[cc] = 0.0f;
-        const E *grow = gout + ((long)n * g.Cout + (long)grp * g.cout_g) * plane_out + pix;
-        const E *wrow = weight + ((long)grp * g.cout_g * g.cin_g + (c0 - grp * g.cin_g)) * g.taps + tap;
-        for (int co = 0; co < g.cout_g; ++co) {
-          const float gv = to_f32(grow[(long)co * plane_out]);
-          const E *wc = wrow + (long)co * g.cin_g * g.taps;
+      for (int cc = 0; cc < kBwdChunk; ++cc) d[cc] = 0.0f;
+      const E *grow = gout + ((long)n * g.Cout + (long)grp * g.cout_g) * plane_out + pix;
+      const E *wrow = weight + ((long)grp * g.cout_g * g.cin_g + (c0 - grp * g.cin_g)) * g.taps + tap;
+      for (int cot = 0; cot < g.cout_g; cot += kBwdCoTile) {
+        const int ncot = min(kBwdCoTile, g.cout_g - cot);
+        __syncthreads();  // the previous slice has been read
+        {
+          float w16[kBwdChunk];
+          const E *wc = wrow + (long)(cot + min(tid, ncot - 1)) * g.cin_g * g.taps;
 #pragma unroll
           for (int cc = 0; cc < kBwdChunk; ++cc)
-            if (cc < cn) d[cc] += to_f32(wc[(long)cc * g.taps]) * gv;
+            w16[cc] = (cc < cn && tid < ncot) ? to_f32(wc[(long)cc * g.taps]) : 0.0f;
+#pragma unroll
+          for (int q = 0; q < kBwdChunk / 4; ++q)
+            wl[tid][q] = make_float4(w16[4 * q], w16[4 * q + 1], w16[4 * q + 2], w16[4 * q + 3]);
         }
+        __syncthreads();
+        if (inside) {
+          for (int co = 0; co < ncot; ++co) {
+            const float gv = to_f32(grow[(long)(cot + co) * plane_out]);
+#pragma unroll
+            for (int q = 0; q < kBwdChunk / 4; ++q) {
+              const float4 w4 = wl[co][q];
+              d[4 * q] += w4.x * gv;
+              d[4 * q + 1] += w4.y * gv;
+              d[4 * q + 2] += w4.z * gv;
+              d[4 * q + 3] += w4.w * gv;
+            }
+          }
+        }
+      }
+      if (inside) {
 #pragma unroll
         for (int cc = 0; cc < kBwdChunk; ++cc) {
           if (cc < cn) {
@@ -143,13 +172,15 @@ __global__ __launch_bounds__(256) void bwd_data_kernel(Geom g, const E *__restri
             if (ok11) unsafeAtomicAdd(gi + o11, (ly * lx) * t);
           }
         }
-        c0 += cn;
       }
+      c0 += cn;
     }
-    const long ob = ((long)n * g.DG + dgi) * 2 * g.taps;
-    goff[(ob + 2 * tap) * plane_out + pix] = from_f32<E>(acc_y * m);
-    goff[(ob + 2 * tap + 1) * plane_out + pix] = from_f32<E>(acc_x * m);
-    if (gmask) gmask[(((long)n * g.DG + dgi) * g.taps + tap) * plane_out + pix] = from_f32<E>(acc_m);
+    if (valid) {
+      const long ob = ((long)n * g.DG + dgi) * 2 * g.taps;
+      goff[(ob + 2 * tap) * plane_out + pix] = from_f32<E>(acc_y * m);
+      goff[(ob + 2 * tap + 1) * plane_out + pix] = from_f32<E>(acc_x * m);
+      if (gmask) gmask[(((long)n * g.DG + dgi) * g.taps + tap) * plane_out + pix] = from_f32<E>(acc_m);
+    }
   }
 }
 
