@@ -73,17 +73,23 @@ template <typename E>
 struct ElemTraits;
 
 // ---- 16-bit element types ---------------------------------------------------
-// A 32-bit word of gathered data holds two channels and is fed to the blend
-// instruction unchanged (no unpacking).
+// A 32-bit word of gathered data holds two channels.  The two horizontal
+// neighbours of a row are paired channel by channel with v_perm_b32 and one
+// v_dot2 applies both of their weights: (v(x0), v(x0+1)) . (w_left, w_right).
+// The perms run on the integer pipe, which keeps working while the other wave
+// of the SIMD streams MFMAs; floating-point VALU work does not (measured: it is
+// starved completely), so halving the number of dot instructions matters more
+// than the instruction count says.  The table keeps the weight pairs
+// (w00, w01) and (w10, w11), rounded to the element type.
 template <typename E>
 struct Half16Traits {
   static constexpr int KC = 64;  // channels per K step (128 bytes)
 
   static __device__ __forceinline__ void table_weights(const TapSample &s, uint32_t (&tw)[4]) {
-    tw[0] = ElemTraits<E>::pack2(s.w00, 0.0f);
-    tw[1] = ElemTraits<E>::pack2(s.w01, 0.0f);
-    tw[2] = ElemTraits<E>::pack2(s.w10, 0.0f);
-    tw[3] = ElemTraits<E>::pack2(s.w11, 0.0f);
+    tw[0] = ElemTraits<E>::pack2(s.w00, s.w01);
+    tw[1] = ElemTraits<E>::pack2(s.w10, s.w11);
+    tw[2] = 0u;
+    tw[3] = 0u;
   }
 
   // four consecutive pixels of one output channel, rounded, to the staging row
@@ -93,32 +99,27 @@ struct Half16Traits {
   }
 
   // 16 bytes (8 channels) of one pixel from the same 16 bytes at its 4 corners
+  // (v0, v1: upper row left/right; v2, v3: lower row)
   static __device__ __forceinline__ uint4 blend(const uint4 &v0, const uint4 &v1, const uint4 &v2,
                                                 const uint4 &v3, const uint4 &w) {
-    const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
-    const uint4 v[4] = {v0, v1, v2, v3};
-    float acc[8];
+    const uint32_t t0[4] = {v0.x, v0.y, v0.z, v0.w}, t1[4] = {v1.x, v1.y, v1.z, v1.w};
+    const uint32_t b0[4] = {v2.x, v2.y, v2.z, v2.w}, b1[4] = {v3.x, v3.y, v3.z, v3.w};
+    uint32_t o[4];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const uint32_t d[4] = {v[q].x, v[q].y, v[q].z, v[q].w};
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        if (q == 0) {
-          acc[2 * j] = ElemTraits<E>::dot_lo0(d[j], ww[q]);
-          acc[2 * j + 1] = ElemTraits<E>::dot_hi0(d[j], ww[q]);
-        } else {
-          acc[2 * j] = ElemTraits<E>::dot_lo(d[j], ww[q], acc[2 * j]);
-          acc[2 * j + 1] = ElemTraits<E>::dot_hi(d[j], ww[q], acc[2 * j + 1]);
-        }
-      }
+    for (int j = 0; j < 4; ++j) {
+      // low channel of word j: bytes 0,1 of both neighbours; high channel: bytes 2,3
+      const uint32_t top_lo = __builtin_amdgcn_perm(t1[j], t0[j], 0x05040100u);
+      const uint32_t top_hi = __builtin_amdgcn_perm(t1[j], t0[j], 0x07060302u);
+      const uint32_t bot_lo = __builtin_amdgcn_perm(b1[j], b0[j], 0x05040100u);
+      const uint32_t bot_hi = __builtin_amdgcn_perm(b1[j], b0[j], 0x07060302u);
+      const float lo = ElemTraits<E>::dot2(bot_lo, w.y, ElemTraits<E>::dot2(top_lo, w.x, 0.0f));
+      const float hi = ElemTraits<E>::dot2(bot_hi, w.y, ElemTraits<E>::dot2(top_hi, w.x, 0.0f));
+      o[j] = ElemTraits<E>::pack2(lo, hi);
     }
-    return make_uint4(ElemTraits<E>::pack2(acc[0], acc[1]), ElemTraits<E>::pack2(acc[2], acc[3]),
-                      ElemTraits<E>::pack2(acc[4], acc[5]), ElemTraits<E>::pack2(acc[6], acc[7]));
+    return make_uint4(o[0], o[1], o[2], o[3]);
   }
 };
 
-// bf16: v_dot2 on the raw pair.  The table keeps the weight word (w, 0); the
-// word for the high channel, (0, w), is that shifted left by 16.
 template <>
 struct ElemTraits<bf16_t> : Half16Traits<bf16_t> {
   static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
@@ -127,20 +128,11 @@ struct ElemTraits<bf16_t> : Half16Traits<bf16_t> {
     p.y = (bf16_t)hi;
     return __builtin_bit_cast(uint32_t, p);
   }
-  // (builtins, not inline assembly: the compiler must see the DOT instruction
+  // (the builtin, not inline assembly: the compiler must see the DOT instruction
   // to insert the wait states its result needs before another VALU reads it)
-  static __device__ __forceinline__ float dot_lo(uint32_t d, uint32_t w, float c) {
+  static __device__ __forceinline__ float dot2(uint32_t d, uint32_t w, float c) {
     return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, d),
                                            __builtin_bit_cast(bf16x2, w), c, false);
-  }
-  static __device__ __forceinline__ float dot_hi(uint32_t d, uint32_t w, float c) {
-    return dot_lo(d, w << 16, c);
-  }
-  static __device__ __forceinline__ float dot_lo0(uint32_t d, uint32_t w) {
-    return dot_lo(d, w, 0.0f);
-  }
-  static __device__ __forceinline__ float dot_hi0(uint32_t d, uint32_t w) {
-    return dot_lo(d, w << 16, 0.0f);
   }
   // 16 bytes = 8 consecutive K elements of one row per lane.
   static __device__ __forceinline__ void mma(f32x16 &c, const uint4 &a, const uint4 &b) {
@@ -149,8 +141,6 @@ struct ElemTraits<bf16_t> : Half16Traits<bf16_t> {
   }
 };
 
-// fp16: mixed-precision FMA (v_fma_mix_f32): one source is read as the low or
-// high fp16 half of the gathered word, the bilinear weight stays fp32.
 template <>
 struct ElemTraits<f16_t> : Half16Traits<f16_t> {
   static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
@@ -159,24 +149,8 @@ struct ElemTraits<f16_t> : Half16Traits<f16_t> {
     p.y = (f16_t)hi;
     return __builtin_bit_cast(uint32_t, p);
   }
-  static __device__ __forceinline__ void table_weights(const TapSample &s, uint32_t (&tw)[4]) {
-    tw[0] = __float_as_uint(s.w00);
-    tw[1] = __float_as_uint(s.w01);
-    tw[2] = __float_as_uint(s.w10);
-    tw[3] = __float_as_uint(s.w11);
-  }
-  // fma(fpext(half), w, c): the compiler selects v_fma_mix_f32 with op_sel
-  static __device__ __forceinline__ float dot_lo(uint32_t d, uint32_t w, float c) {
-    return __builtin_fmaf((float)__builtin_bit_cast(f16x2, d).x, __uint_as_float(w), c);
-  }
-  static __device__ __forceinline__ float dot_hi(uint32_t d, uint32_t w, float c) {
-    return __builtin_fmaf((float)__builtin_bit_cast(f16x2, d).y, __uint_as_float(w), c);
-  }
-  static __device__ __forceinline__ float dot_lo0(uint32_t d, uint32_t w) {
-    return (float)__builtin_bit_cast(f16x2, d).x * __uint_as_float(w);
-  }
-  static __device__ __forceinline__ float dot_hi0(uint32_t d, uint32_t w) {
-    return (float)__builtin_bit_cast(f16x2, d).y * __uint_as_float(w);
+  static __device__ __forceinline__ float dot2(uint32_t d, uint32_t w, float c) {
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, d), __builtin_bit_cast(f16x2, w), c, false);
   }
   static __device__ __forceinline__ void mma(f32x16 &c, const uint4 &a, const uint4 &b) {
     c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
