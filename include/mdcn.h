@@ -85,6 +85,10 @@ typedef struct mdcn_params {
   int32_t Cout, kh, kw;
   int32_t sh, sw, ph, pw, dh, dw;
   int32_t groups, dgroups;
+  int32_t input_nhwc;     /* 0: input is dense (N, Cin, H, W).  1: input is dense channels-last, (N, H, W, Cin)
+                             in memory (torch.channels_last); the fused kernel then reads it in place, without
+                             the re-laid-out copy.  Fused path of mdcn_forward() only (H, W >= 2); every
+                             other tensor keeps its layout. */
 } mdcn_params;
 
 /* ABI version of the loaded library (== MDCN_ABI_VERSION it was built with). */

@@ -115,7 +115,17 @@ void prepare(Prepared &pr, const Tensor &input, const Tensor &weight,
     pr.keep.push_back(t.contiguous());
     return pr.keep.back().data_ptr();
   };
-  p.input = dense(input);
+  // a channels-last input is read in place when the fused kernel covers the shape
+  p.input = nullptr;
+  if (!input.is_contiguous() && input.is_contiguous(at::MemoryFormat::ChannelsLast)) {
+    p.input = input.data_ptr();
+    p.input_nhwc = 1;
+    if (!mdcn_fused_eligible(&p) || g_path == MDCN_PATH_DIRECT) {
+      p.input = nullptr;
+      p.input_nhwc = 0;
+    }
+  }
+  if (!p.input) p.input = dense(input);
   p.offset = dense(offset);
   p.mask = dense(mask);
   p.weight = dense(weight);

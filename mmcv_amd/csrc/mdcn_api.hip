@@ -71,6 +71,7 @@ inline int pick_ct(int cout_g, int taps) {
 
 bool fused_ok(const mdcn_params *p, const Geom &g) {
   const int KC = slab_channels(p->dtype);
+  if (p->input_nhwc && (g.H < 2 || g.W < 2 || ((uintptr_t)p->input % 16) != 0)) return false;
   if (g.cin_g % KC || g.ch_per_dg % KC) return false;
   if (g.taps > kTapsLarge) return false;
   if (fused_lds_bytes(pick_ct(g.cout_g, g.taps), table_capacity(g.taps)) > kMaxLds) return false;
@@ -116,6 +117,7 @@ struct PackExtra {
 int make_plan(const mdcn_params *p, const Geom &g, Plan *pl) {
   const bool ok = fused_ok(p, g);
   if (p->path == MDCN_PATH_FUSED && !ok) return MDCN_ERR_PATH;
+  if (p->input_nhwc && (!ok || p->path == MDCN_PATH_DIRECT)) return MDCN_ERR_PATH;  // in-place reads: fused kernel only
   pl->fused = ok && p->path != MDCN_PATH_DIRECT;
   pl->CT = pl->KC = pl->n_ctiles = pl->slabs = pl->n_chunk = 0;
   pl->xt_bytes = pl->wp_bytes = pl->owp_bytes = pl->raw_bytes = 0;
@@ -130,7 +132,7 @@ int make_plan(const mdcn_params *p, const Geom &g, Plan *pl) {
   pl->slabs = g.cin_g / pl->KC;
   const uint64_t img = (uint64_t)g.Hp * g.Wp * g.Cin * es;
   pl->n_chunk = (int)std::min<uint64_t>((uint64_t)g.N, std::max<uint64_t>(1, kMaxXtBytes / img));
-  pl->xt_bytes = align_up((size_t)img * pl->n_chunk);
+  pl->xt_bytes = p->input_nhwc ? 0 : align_up((size_t)img * pl->n_chunk);
   pl->wp_bytes = align_up((size_t)g.G * pl->n_ctiles * pl->slabs * g.taps * pl->CT * pl->KC * es);
   return MDCN_OK;
 }
@@ -139,6 +141,7 @@ int make_plan(const mdcn_params *p, const Geom &g, Plan *pl) {
 // the direct one (nothing when the caller's own raw buffer serves).
 int make_pack_plan(const mdcn_pack_params *pp, const Geom &g, Plan *pl) {
   const mdcn_params *p = &pp->conv;
+  if (p->input_nhwc) return MDCN_ERR_PATH;
   const int rc = make_plan(p, g, pl);
   if (rc != MDCN_OK) return rc;
   if (pp->unmodulated) {
@@ -200,36 +203,40 @@ hipError_t launch_oconv(OconvArgs oa, hipStream_t st) {
 }
 
 template <typename E, int CT, int TMAX, bool MULTI_DG>
-hipError_t launch_fused_ct(const FusedArgs &fa, hipStream_t st) {
+hipError_t launch_fused_ct(const FusedArgs &fa, bool unbordered, hipStream_t st) {
   // persistent workgroups: one per CU, a multiple of the 8 XCDs
   const int total_wg = fa.n_ptiles * fa.n_ctiles * fa.g.G;
   const int per_xcd = std::max(1, std::min((total_wg + 7) / 8, num_cus() / 8));
-  hipLaunchKernelGGL((fused_kernel<E, CT, TMAX, MULTI_DG>), dim3(per_xcd * 8), dim3(kThreads), 0,
-                     st, fa);
+  if (unbordered)
+    hipLaunchKernelGGL((fused_kernel<E, CT, TMAX, MULTI_DG, true>), dim3(per_xcd * 8), dim3(kThreads),
+                       0, st, fa);
+  else
+    hipLaunchKernelGGL((fused_kernel<E, CT, TMAX, MULTI_DG, false>), dim3(per_xcd * 8), dim3(kThreads),
+                       0, st, fa);
   return hipGetLastError();
 }
 
 template <typename E, int CT>
-hipError_t launch_fused_tm(const FusedArgs &fa, hipStream_t st) {
+hipError_t launch_fused_tm(const FusedArgs &fa, bool ub, hipStream_t st) {
   const bool small = fa.g.taps <= kTapsSmall;
   if constexpr (CT == 256) {  // (pick_ct never pairs the 256-wide tile with the large table)
-    return fa.g.DG > 1 ? launch_fused_ct<E, CT, kTapsSmall, true>(fa, st)
-                       : launch_fused_ct<E, CT, kTapsSmall, false>(fa, st);
+    return fa.g.DG > 1 ? launch_fused_ct<E, CT, kTapsSmall, true>(fa, ub, st)
+                       : launch_fused_ct<E, CT, kTapsSmall, false>(fa, ub, st);
   } else {
     if (fa.g.DG > 1)
-      return small ? launch_fused_ct<E, CT, kTapsSmall, true>(fa, st)
-                   : launch_fused_ct<E, CT, kTapsLarge, true>(fa, st);
-    return small ? launch_fused_ct<E, CT, kTapsSmall, false>(fa, st)
-                 : launch_fused_ct<E, CT, kTapsLarge, false>(fa, st);
+      return small ? launch_fused_ct<E, CT, kTapsSmall, true>(fa, ub, st)
+                   : launch_fused_ct<E, CT, kTapsLarge, true>(fa, ub, st);
+    return small ? launch_fused_ct<E, CT, kTapsSmall, false>(fa, ub, st)
+                 : launch_fused_ct<E, CT, kTapsLarge, false>(fa, ub, st);
   }
 }
 
 template <typename E>
-hipError_t launch_fused(const FusedArgs &fa, int CT, hipStream_t st) {
+hipError_t launch_fused(const FusedArgs &fa, int CT, bool ub, hipStream_t st) {
   switch (CT) {
-    case 64: return launch_fused_tm<E, 64>(fa, st);
-    case 128: return launch_fused_tm<E, 128>(fa, st);
-    default: return launch_fused_tm<E, 256>(fa, st);
+    case 64: return launch_fused_tm<E, 64>(fa, ub, st);
+    case 128: return launch_fused_tm<E, 128>(fa, ub, st);
+    default: return launch_fused_tm<E, 256>(fa, ub, st);
   }
 }
 
@@ -325,7 +332,8 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
       Geom gc = g;
       gc.N = std::min(pl.n_chunk, g.N - n0);
       const E *in = (const E *)p->input + (size_t)n0 * g.Cin * g.H * g.W;
-      {
+      const bool nhwc = p->input_nhwc != 0;
+      if (!nhwc) {
         // runs of 128 pixels of the image plane
         const int n_pchunks = (gc.H * gc.W + 127) / 128;
         const long blocks = (long)gc.N * (gc.Cin / pl.KC) * n_pchunks;
@@ -339,8 +347,19 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
       }
       FusedArgs fa;
       fa.g = gc;
-      fa.xt = xt;
+      fa.xt = nhwc ? (const void *)in : (const void *)xt;
       fa.wp = wp;
+      if (nhwc) {
+        fa.px_bytes = (uint32_t)(g.Cin * es);
+        fa.row_bytes = (uint32_t)g.W * fa.px_bytes;
+        fa.slab_bytes = (uint32_t)kRowB;
+        fa.img_bytes = (uint32_t)g.H * fa.row_bytes;
+      } else {
+        fa.px_bytes = (uint32_t)kRowB;
+        fa.row_bytes = (uint32_t)g.Wp * (uint32_t)kRowB;
+        fa.slab_bytes = (uint32_t)(g.Hp * g.Wp) * (uint32_t)kRowB;
+        fa.img_bytes = (uint32_t)(g.Cin / pl.KC) * fa.slab_bytes;
+      }
       if (own_oconv) {
         OconvArgs oa;
         oa.g = gc;
@@ -390,10 +409,9 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
       fa.slabs = pl.slabs;
       fa.slabs_total = g.Cin / pl.KC;
       fa.plane_px = g.Hp * g.Wp;
-      fa.row_bytes = (uint32_t)g.Wp * (uint32_t)kRowB;
       fa.out_vec_ok = (plane_out % (long)(16 / es) == 0) && (((uintptr_t)fa.out % 16) == 0);
       tic();
-      if (launch_fused<E>(fa, pl.CT, st) != hipSuccess) rc = MDCN_ERR_LAUNCH;
+      if (launch_fused<E>(fa, pl.CT, nhwc, st) != hipSuccess) rc = MDCN_ERR_LAUNCH;
       toc(2);
     }
   }
@@ -511,6 +529,7 @@ int check_bwd(const mdcn_bwd_params *bp, Geom *g, bool need_ptrs) {
   const mdcn_params *p = &bp->conv;
   int rc = check_params(p, g, false);
   if (rc != MDCN_OK) return rc;
+  if (p->input_nhwc) return MDCN_ERR_PATH;
   if (!need_ptrs) return MDCN_OK;
   if (!p->input || !p->offset || !p->weight || !bp->grad_output) return MDCN_ERR_NULL;
   // grad_input and the offset/mask gradients come out of one kernel

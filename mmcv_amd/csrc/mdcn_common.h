@@ -68,6 +68,24 @@ __device__ __forceinline__ TapSample make_tap_sample(int base_y, int base_x,
   return s;
 }
 
+// For reading the four corners from a tensor without a zero border (needs
+// H, W >= 2): move the 2x2 block into the image and give the corners that fell
+// outside weight 0; the corners that stay valid keep their weight, at their new
+// place in the block.  Positions outside (-1,H)x(-1,W) already have zero weights
+// and y0 = x0 = 0.
+__device__ __forceinline__ void clamp_to_image(TapSample &s, int H, int W) {
+  if (s.x0 < 0) {            // only the right column (x0 + 1 == 0) is inside: it becomes the left one
+    s.w00 = s.w01; s.w10 = s.w11; s.w01 = 0.0f; s.w11 = 0.0f; s.x0 = 0;
+  } else if (s.x0 > W - 2) { // only the left column (x0 == W - 1) is inside: it becomes the right one
+    s.w01 = s.w00; s.w11 = s.w10; s.w00 = 0.0f; s.w10 = 0.0f; s.x0 = W - 2;
+  }
+  if (s.y0 < 0) {
+    s.w00 = s.w10; s.w01 = s.w11; s.w10 = 0.0f; s.w11 = 0.0f; s.y0 = 0;
+  } else if (s.y0 > H - 2) {
+    s.w10 = s.w00; s.w11 = s.w01; s.w00 = 0.0f; s.w01 = 0.0f; s.y0 = H - 2;
+  }
+}
+
 // Where the offsets and the mask of one output pixel live, in elements: image n,
 // pixel rem = ho * Wo + wo, channel c sits at base + n * _n + rem * _px + c * _ch.
 // The reference op takes two dense NCHW tensors (_px = 1, _ch = Ho * Wo); the

@@ -54,7 +54,7 @@ constexpr int kTapGroups = kProducerWaves / 2;           // producer lanes per p
 
 struct FusedArgs {
   Geom g;
-  const void *xt;      // zero-bordered slab-major input copy
+  const void *xt;      // zero-bordered slab-major input copy, or the caller's channels-last input itself
   const void *wp;      // packed weights
   OffMaskView om;      // offsets and mask of the images of this launch
   const void *bias;    // may be null
@@ -64,7 +64,10 @@ struct FusedArgs {
   int slabs_total;     // Cin / KC
   int plane_px;        // Hp * Wp
   int out_vec_ok;      // (Ho*Wo) % (16/sizeof(E)) == 0 and the output pointer is 16-byte aligned
-  uint32_t row_bytes;  // Wp * kRowB
+  uint32_t row_bytes;  // bytes between vertically adjacent pixels: Wp * kRowB (copy) or W * Cin * sizeof(E)
+  uint32_t px_bytes;   // bytes between horizontally adjacent pixels: kRowB (copy) or Cin * sizeof(E)
+  uint32_t slab_bytes; // bytes between channel slabs of one pixel: plane_px * kRowB (copy) or kRowB
+  uint32_t img_bytes;  // bytes between images
 };
 
 typedef __attribute__((address_space(3))) void *lptr_t;
@@ -287,7 +290,11 @@ __device__ __forceinline__ int tile_chunk(int r, int c) { return r * kRowChunks 
 // K loop.  Kept out of the single-group instantiation because a conditional
 // block with loads inside the step loop makes the compiler drain the gather
 // prefetch (vmcnt(0)) at every step.
-template <typename E, int CT, int TMAX, bool MULTI_DG>
+// UNBORDERED: a.xt is the caller's dense channels-last (N, H, W, Cin) input, read
+// in place: no copy, no zero border.  The table then clamps each 2x2 corner block
+// into the image and moves the weights of the corners that fell outside to zero
+// (clamp_to_image), which keeps the reference's per-corner rule.
+template <typename E, int CT, int TMAX, bool MULTI_DG, bool UNBORDERED>
 __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
   using TR = ElemTraits<E>;
   constexpr int PT = kPT;
@@ -301,7 +308,7 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
 
   __shared__ uint4 Xs[2][PT * kRowChunks];                // sample tiles
   __shared__ uint4 Ws[kWeightSlots][CT * kRowChunks];     // weight tiles
-  __shared__ int32_t tpix[PT * TMAX];                     // (pixel, tap) table, [tap][PT]: corner
+  __shared__ uint32_t tpix[PT * TMAX];                    // (pixel, tap) table, [tap][PT]: corner byte offset
   __shared__ uint4 tws[PT * TMAX];                        // ... and the four weights
 
   const Geom &g = a.g;
@@ -346,6 +353,8 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
       const int q = ptid & 3;          // this lane handles 16-byte chunks q and q + 4 of a row
       const int pxl = ptid >> 2;       // ... of pixels pxl and pxl + 64 of the tile
       const unsigned char *xt = (const unsigned char *)a.xt;
+      // horizontal neighbour: an instruction offset for the copy, a register otherwise
+      const uint32_t pxb = UNBORDERED ? a.px_bytes : (uint32_t)kRowB;
 
       // -- (pixel, tap) table of one deformable group; lane serves pixel ptid%128
       const int tb_pl = ptid & (PT - 1);
@@ -378,12 +387,19 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
           const int tap = (ptid >> 7) + kTapGroups * i;
           if (tap < taps) {
             const int ti = tap / g.kw, tj = tap - ti * g.kw;
-            const TapSample sm =
+            TapSample sm =
                 make_tap_sample(tb_ho * g.sh - g.ph + ti * g.dh, tb_wo * g.sw - g.pw + tj * g.dw,
                                 to_f32(rdy[i]), to_f32(rdx[i]), mask_value<E>(rm[i], a.om.logit), g.H, g.W);
-            // +1: coordinates in the zero-bordered copy (y0, x0 >= -1 when inside,
-            // 0 with zero weights otherwise); slab 0 of image tb_n.
-            int32_t pix = tb_n * a.slabs_total * a.plane_px + (sm.y0 + 1) * g.Wp + (sm.x0 + 1);
+            // byte offset of the upper left corner, slab 0 of image tb_n
+            uint32_t pix;
+            if (UNBORDERED) {
+              clamp_to_image(sm, g.H, g.W);
+              pix = (uint32_t)tb_n * a.img_bytes + (uint32_t)sm.y0 * a.row_bytes + (uint32_t)sm.x0 * a.px_bytes;
+            } else {
+              // +1: coordinates in the zero-bordered copy (y0, x0 >= -1 when inside,
+              // 0 with zero weights otherwise)
+              pix = (uint32_t)tb_n * a.img_bytes + (uint32_t)(sm.y0 + 1) * a.row_bytes + (uint32_t)(sm.x0 + 1) * kRowB;
+            }
             uint32_t tw[4];
             TR::table_weights(sm, tw);
             if (!tb_valid) {
@@ -411,22 +427,22 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
           build_table((ch0 + cur.slab * KC) / g.ch_per_dg);
           MDCN_BARRIER_LDS();  // R: new table visible (the consumers join)
         }
-        const int sbase = (slab0 + cur.slab) * a.plane_px;
+        const uint32_t sbase = (uint32_t)(slab0 + cur.slab) * a.slab_bytes + (uint32_t)q * 16u;
 #pragma unroll
         for (int h = 0; h < kPxPerLane; ++h) {
           const int e = cur.tap * PT + pxl + (PT / kPxPerLane) * h;
-          const uint32_t o = ((uint32_t)(tpix[e] + sbase) << 7) + (uint32_t)q * 16u;
+          const uint32_t o = tpix[e] + sbase;
           w[h] = tws[e];
           const unsigned char *top = xt + o;
           const unsigned char *bot = top + a.row_bytes;
           v[h][0][0] = *(const uint4 *)(top);
           v[h][0][1] = *(const uint4 *)(top + 64);
-          v[h][1][0] = *(const uint4 *)(top + 128);
-          v[h][1][1] = *(const uint4 *)(top + 192);
+          v[h][1][0] = *(const uint4 *)(top + pxb);
+          v[h][1][1] = *(const uint4 *)(top + pxb + 64);
           v[h][2][0] = *(const uint4 *)(bot);
           v[h][2][1] = *(const uint4 *)(bot + 64);
-          v[h][3][0] = *(const uint4 *)(bot + 128);
-          v[h][3][1] = *(const uint4 *)(bot + 192);
+          v[h][3][0] = *(const uint4 *)(bot + pxb);
+          v[h][3][1] = *(const uint4 *)(bot + pxb + 64);
         }
         cur.advance(nk, taps, spd);
       };
@@ -440,13 +456,13 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
           build_table((ch0 + cur.slab * KC) / g.ch_per_dg);
           MDCN_BARRIER_LDS();  // R
         }
-        const int sbase = (slab0 + cur.slab) * a.plane_px;
+        const uint32_t sbase = (uint32_t)(slab0 + cur.slab) * a.slab_bytes + (uint32_t)q * 16u;
         uint32_t o[kPxPerLane];
         uint4 wn[kPxPerLane];
 #pragma unroll
         for (int h = 0; h < kPxPerLane; ++h) {
           const int e = cur.tap * PT + pxl + (PT / kPxPerLane) * h;
-          o[h] = ((uint32_t)(tpix[e] + sbase) << 7) + (uint32_t)q * 16u;
+          o[h] = tpix[e] + sbase;
           wn[h] = tws[e];
         }
 #pragma unroll
@@ -459,9 +475,9 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
             const unsigned char *top = xt + o[h] + half * 64;
             const unsigned char *bot = top + a.row_bytes;
             v[h][0][half] = *(const uint4 *)(top);
-            v[h][1][half] = *(const uint4 *)(top + 128);
+            v[h][1][half] = *(const uint4 *)(top + pxb);
             v[h][2][half] = *(const uint4 *)(bot);
-            v[h][3][half] = *(const uint4 *)(bot + 128);
+            v[h][3][half] = *(const uint4 *)(bot + pxb);
             __builtin_amdgcn_sched_barrier(0);
           }
           w[h] = wn[h];

@@ -88,6 +88,9 @@ def capi_forward(case, path=capi.PATH_AUTO, timed=False):
     ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=x.device)
     keep = [t.contiguous() for t in (x, off, w)]
     p.input, p.offset, p.weight = (t.data_ptr() for t in keep)
+    if case.get('input_nhwc'):  # hand the library the channels-last bytes of the input
+        keep.append(x.permute(0, 2, 3, 1).contiguous())
+        p.input, p.input_nhwc = keep[-1].data_ptr(), 1
     if msk is not None:  # None: unmodulated (DCNv1)
         keep.append(msk.contiguous())
         p.mask = keep[-1].data_ptr()
