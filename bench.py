@@ -250,6 +250,20 @@ def main():
     log(f'{a.workload} {dname}: step {ms_per_step:.4f} ms (events {ev_ms:.4f}, wall {wall_ms:.4f}); '
         f'stages relayout {stage[0]:.4f} pack {stage[1]:.4f} main {stage[2]:.4f} ms')
 
+    # the same step with the input handed over channels-last (read in place, no re-layout)
+    x_cl = x.contiguous(memory_format=torch.channels_last)
+    step_cl = lambda: ext_module.modulated_deform_conv_forward(x_cl, w, b, empty, off, msk, out, empty, **kwargs)
+    for _ in range(a.warmup):
+        step_cl()
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(a.steps):
+        step_cl()
+    e1.record()
+    torch.cuda.synchronize()
+    cl_ms = e0.elapsed_time(e1) / a.steps
+    log(f'channels-last input: step {cl_ms:.4f} ms')
+
     value = flops / (ms_per_step * 1e-3) / 1e12
     achieved = flops / (main_ms * 1e-3) / 1e12
     peak = PEAK_TFLOPS[dname]
@@ -279,6 +293,8 @@ def main():
         'stage_ms': {'relayout': round(stage[0], 4), 'weight_pack': round(stage[1], 4),
                      'main': round(stage[2], 4)},
         'hbm_GBs_algorithmic': round(alg_bytes / (ms_per_step * 1e-3) / 1e9, 1),
+        'channels_last_input': {'ms_per_step': round(cl_ms, 4),
+                                'TFLOPs': round(flops / (cl_ms * 1e-3) / 1e12, 2)},
         'roofline': {
             'bound': 'mfma',
             'kernel': f'fused_kernel<{dname}>',
