@@ -24,6 +24,8 @@ HIPCC_FLAGS = [
     '--offload-arch=gfx950', '-O3', '-std=c++17', '-fPIC', '-shared',
     # packed-fp32 VALU forms are kept out of the generated code
     '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
+    # '#pragma unroll' loops whose bodies index register arrays must unroll whatever their size
+    '-mllvm', '-pragma-unroll-threshold=100000',
     '-Wno-unused-command-line-argument',
 ]
 

@@ -477,11 +477,38 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
     float *gin32 = pl.gin_bytes ? (float *)ws : (float *)bp->grad_input;
     hipLaunchKernelGGL(fill_zero_kernel<float>, dim3(blocks_for(n_in)), dim3(256), 0, st, gin32, n_in);
     check();
-    const int rows = g.N * g.DG * g.taps;  // (image, deformable group, tap)
-    const dim3 grid((unsigned)((plane_out + 255) / 256), (unsigned)std::min(rows, 65535));
-    hipLaunchKernelGGL(bwd_data_kernel<E>, grid, dim3(256), 0, st, g, (const E *)p->input, om,
-                       (const E *)p->weight, (const E *)bp->grad_output, gin32,
-                       (E *)bp->grad_offset, (E *)bp->grad_mask, rows);
+    // window of the tiled kernel: the tile's undeformed footprint plus a margin R on every side
+    const int base_h = (kBwdTile - 1) * g.sh + (g.kh - 1) * g.dh + 2;
+    const int base_w = (kBwdTile - 1) * g.sw + (g.kw - 1) * g.dw + 2;
+    const int max_px = kBwdWindowBytes / (4 * kBwdChunk);
+    int R = -1;
+    while (R < 8 && (base_h + 2 * (R + 1)) * (base_w + 2 * (R + 1)) <= max_px) ++R;
+    // (small problems keep the per-tap kernel: it has taps x more workgroups)
+    const long n_tiles = (long)g.N * g.DG * ((g.Ho + kBwdTile - 1) / kBwdTile) * ((g.Wo + kBwdTile - 1) / kBwdTile);
+    if (g.taps <= kBwdTapsMax && R >= 1 && n_tiles >= 2L * num_cus()) {
+      BwdDataTiledArgs da;
+      da.g = g;
+      da.input = p->input;
+      da.om = om;
+      da.weight = p->weight;
+      da.gout = bp->grad_output;
+      da.gin32 = gin32;
+      da.goff = bp->grad_offset;
+      da.gmask = bp->grad_mask;
+      da.tiles_x = (g.Wo + kBwdTile - 1) / kBwdTile;
+      da.tiles_y = (g.Ho + kBwdTile - 1) / kBwdTile;
+      da.R = R;
+      da.WH = base_h + 2 * R;
+      da.WW = base_w + 2 * R;
+      const long blocks = (long)g.N * g.DG * da.tiles_y * da.tiles_x;
+      hipLaunchKernelGGL(bwd_data_tiled_kernel<E>, dim3((unsigned)blocks), dim3(256), 0, st, da);
+    } else {
+      const int rows = g.N * g.DG * g.taps;  // (image, deformable group, tap)
+      const dim3 grid((unsigned)((plane_out + 255) / 256), (unsigned)std::min(rows, 65535));
+      hipLaunchKernelGGL(bwd_data_kernel<E>, grid, dim3(256), 0, st, g, (const E *)p->input, om,
+                         (const E *)p->weight, (const E *)bp->grad_output, gin32,
+                         (E *)bp->grad_offset, (E *)bp->grad_mask, rows);
+    }
     check();
     if (pl.gin_bytes) {
       hipLaunchKernelGGL(round_kernel<E>, dim3(blocks_for(n_in)), dim3(256), 0, st, gin32,

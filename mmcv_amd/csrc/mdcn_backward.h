@@ -184,6 +184,199 @@ __global__ __launch_bounds__(256) void bwd_data_kernel(Geom g, const E *__restri
   }
 }
 
+// Tiled variant of bwd_data_kernel for kernels of up to 9 taps: a workgroup owns a
+// 16 x 16 tile of output pixels of one (image, deformable group) and walks all
+// taps itself, so that the scatter into grad_input can be summed in LDS first.
+// The taps of a tile and of neighbouring pixels hit the same few input pixels
+// again and again (256 pixels x 9 taps x 4 corners land in a window of roughly
+// (16 + 2R)^2 pixels): per chunk of kBwdChunk channels the workgroup keeps an fp32
+// window [kBwdChunk][WH][WW] of grad_input around its tile, adds into it with LDS
+// atomics, and flushes the non-zero entries with one global atomic each; corners
+// outside the window go to global memory directly.  grad_offset / grad_mask sums
+// stay in registers per (pixel, tap) across the channel chunks.
+constexpr int kBwdTile = 16;
+constexpr int kBwdTapsMax = 9;
+constexpr int kBwdWindowBytes = 48 * 1024;
+
+struct BwdDataTiledArgs {
+  Geom g;
+  const void *input;
+  OffMaskView om;
+  const void *weight;
+  const void *gout;
+  float *gin32;
+  void *goff;
+  void *gmask;  // null when unmodulated
+  int tiles_x, tiles_y;
+  int WH, WW;   // window size in input pixels
+  int R;        // margin of the window around the tile's undeformed footprint
+};
+
+// Output channels of one all-taps weight slice in LDS.
+constexpr int kBwdTiledCoTile = 16;
+
+template <typename E>
+__global__ __launch_bounds__(256, 2) void bwd_data_tiled_kernel(BwdDataTiledArgs a) {
+  // weight slice [co][tap][chunk] of the current channel chunk, fp32
+  __shared__ float4 wl[kBwdTiledCoTile][kBwdTapsMax][kBwdChunk / 4];
+  __shared__ float win[kBwdWindowBytes / 4];
+  const Geom &g = a.g;
+  const long plane_out = (long)g.Ho * g.Wo;
+  const long plane_in = (long)g.H * g.W;
+  const int tid = threadIdx.x;
+  int b = blockIdx.x;
+  const int tx = b % a.tiles_x;
+  b /= a.tiles_x;
+  const int ty = b % a.tiles_y;
+  b /= a.tiles_y;
+  const int dgi = b % g.DG;
+  const int n = b / g.DG;
+  const int ho = ty * kBwdTile + (tid >> 4), wo = tx * kBwdTile + (tid & 15);
+  const bool valid = ho < g.Ho && wo < g.Wo;
+  const long pix = valid ? (long)ho * g.Wo + wo : 0;
+  // window origin in input coordinates
+  const int wy0 = ty * kBwdTile * g.sh - g.ph - a.R, wx0 = tx * kBwdTile * g.sw - g.pw - a.R;
+  const int win_px = a.WH * a.WW;
+
+  const E *input = (const E *)a.input, *weight = (const E *)a.weight, *gout = (const E *)a.gout;
+  const E *off = (const E *)a.om.off + (long)n * a.om.off_n + pix * a.om.off_px +
+                 (long)(dgi * 2 * g.taps) * a.om.off_ch;
+  const E *msk = (const E *)a.om.msk + (long)n * a.om.msk_n + pix * a.om.msk_px +
+                 (long)(dgi * g.taps) * a.om.msk_ch;
+
+  float acc_m[kBwdTapsMax], acc_y[kBwdTapsMax], acc_x[kBwdTapsMax];
+#pragma unroll
+  for (int t = 0; t < kBwdTapsMax; ++t) acc_m[t] = acc_y[t] = acc_x[t] = 0.0f;
+
+  const int c_begin = dgi * g.ch_per_dg, c_end = c_begin + g.ch_per_dg;
+  for (int c0 = c_begin; c0 < c_end;) {
+    const int grp = c0 / g.cin_g;  // a chunk stays inside one convolution group
+    const int cn = min(kBwdChunk, min(c_end, (grp + 1) * g.cin_g) - c0);
+    __syncthreads();  // the previous chunk's flush is done
+    for (int i = tid; i < win_px * kBwdChunk; i += 256) win[i] = 0.0f;
+    // (the barriers of the slice loop order the zeroing before any add)
+
+    // ---- column gradients of the chunk for every tap: one grad_output load per
+    //      (output channel, pixel) feeds taps x chunk multiply-adds ----
+    static_assert(kBwdChunk == 16, "one 16-float vector per tap");
+    f32x16 d[kBwdTapsMax];  // (vectors, so that the compiler keeps them in registers)
+#pragma unroll
+    for (int t = 0; t < kBwdTapsMax; ++t)
+#pragma unroll
+      for (int cc = 0; cc < kBwdChunk; ++cc) d[t][cc] = 0.0f;
+    const E *grow = gout + ((long)n * g.Cout + (long)grp * g.cout_g) * plane_out + pix;
+    const E *wrow = weight + ((long)grp * g.cout_g * g.cin_g + (c0 - grp * g.cin_g)) * g.taps;
+    for (int cot = 0; cot < g.cout_g; cot += kBwdTiledCoTile) {
+      const int ncot = min(kBwdTiledCoTile, g.cout_g - cot);
+      __syncthreads();  // the previous slice has been read
+      // slice element (co, tap, cc) <- weight[cot + co][c0 + cc][tap]; 16 * 9 * 16 = 2304 elements
+      for (int i = tid; i < kBwdTiledCoTile * kBwdTapsMax * kBwdChunk; i += 256) {
+        const int cc = i % kBwdChunk, t = (i / kBwdChunk) % kBwdTapsMax, co = i / (kBwdChunk * kBwdTapsMax);
+        float v = 0.0f;
+        if (co < ncot && t < g.taps && cc < cn)
+          v = to_f32(wrow[((long)(cot + co) * g.cin_g + cc) * g.taps + t]);
+        ((float *)wl)[i] = v;
+      }
+      __syncthreads();
+      if (valid) {
+        for (int co = 0; co < ncot; ++co) {
+          const float gv = to_f32(grow[(long)(cot + co) * plane_out]);
+#pragma unroll
+          for (int t = 0; t < kBwdTapsMax; ++t)
+#pragma unroll
+            for (int q = 0; q < kBwdChunk / 4; ++q) {
+              const float4 w4 = wl[co][t][q];
+              d[t][4 * q] += w4.x * gv;
+              d[t][4 * q + 1] += w4.y * gv;
+              d[t][4 * q + 2] += w4.z * gv;
+              d[t][4 * q + 3] += w4.w * gv;
+            }
+        }
+      }
+    }
+
+    // ---- per tap: offset / mask sums and the scatter ----
+#pragma unroll
+    for (int tap = 0; tap < kBwdTapsMax; ++tap) {
+      if (tap < g.taps) {
+        const int ti = tap / g.kw, tj = tap - ti * g.kw;
+        const float dy = to_f32(off[(long)(2 * tap) * a.om.off_ch]);
+        const float dx = to_f32(off[(long)(2 * tap + 1) * a.om.off_ch]);
+        const float m = mask_value<E>(msk[(long)tap * a.om.msk_ch], a.om.logit);
+        const float py = (float)(ho * g.sh - g.ph + ti * g.dh) + dy;
+        const float px = (float)(wo * g.sw - g.pw + tj * g.dw) + dx;
+        const bool inside =
+            valid && (py > -1.0f) && (px > -1.0f) && (py < (float)g.H) && (px < (float)g.W);
+        if (inside) {
+          const float fy = floorf(py), fx = floorf(px);
+          const int y0 = (int)fy, x0 = (int)fx, y1 = y0 + 1, x1 = x0 + 1;
+          const float ly = py - fy, lx = px - fx, hy = 1.0f - ly, hx = 1.0f - lx;
+          const bool ok00 = y0 >= 0 && x0 >= 0, ok01 = y0 >= 0 && x1 <= g.W - 1;
+          const bool ok10 = y1 <= g.H - 1 && x0 >= 0, ok11 = y1 <= g.H - 1 && x1 <= g.W - 1;
+          const long o00 = (long)y0 * g.W + x0, o01 = o00 + 1, o10 = o00 + g.W, o11 = o10 + 1;
+          // the 2x2 block inside the window?  (then all four corners are)
+          const int ry = y0 - wy0, rx = x0 - wx0;
+          const bool in_win = ry >= 0 && ry + 1 < a.WH && rx >= 0 && rx + 1 < a.WW;
+          const int wbase = ry * a.WW + rx;  // window is [channel][WH][WW]: neighbouring pixels, neighbouring banks
+          float am = 0.0f, ay = 0.0f, ax = 0.0f;
+#pragma unroll
+          for (int cc = 0; cc < kBwdChunk; ++cc) {
+            if (cc < cn) {
+              const int c = c0 + cc;
+              const E *im = input + ((long)n * g.Cin + c) * plane_in;
+              const float v00 = ok00 ? to_f32(im[o00]) : 0.0f, v01 = ok01 ? to_f32(im[o01]) : 0.0f;
+              const float v10 = ok10 ? to_f32(im[o10]) : 0.0f, v11 = ok11 ? to_f32(im[o11]) : 0.0f;
+              const float dc = d[tap][cc];
+              am += dc * ((hy * hx) * v00 + (hy * lx) * v01 + (ly * hx) * v10 + (ly * lx) * v11);
+              ay += dc * (hx * (v10 - v00) + lx * (v11 - v01));
+              ax += dc * (hy * (v01 - v00) + ly * (v11 - v10));
+              const float t = dc * m;
+              if (in_win) {
+                float *wp = win + cc * win_px + wbase;
+                if (ok00) atomicAdd(wp, (hy * hx) * t);
+                if (ok01) atomicAdd(wp + 1, (hy * lx) * t);
+                if (ok10) atomicAdd(wp + a.WW, (ly * hx) * t);
+                if (ok11) atomicAdd(wp + a.WW + 1, (ly * lx) * t);
+              } else {
+                float *gi = a.gin32 + ((long)n * g.Cin + c) * plane_in;
+                if (ok00) unsafeAtomicAdd(gi + o00, (hy * hx) * t);
+                if (ok01) unsafeAtomicAdd(gi + o01, (hy * lx) * t);
+                if (ok10) unsafeAtomicAdd(gi + o10, (ly * hx) * t);
+                if (ok11) unsafeAtomicAdd(gi + o11, (ly * lx) * t);
+              }
+            }
+          }
+          acc_m[tap] += am;
+          acc_y[tap] += ay * m;
+          acc_x[tap] += ax * m;
+        }
+      }
+    }
+    __syncthreads();  // every add into the window has landed
+    for (int i = tid; i < win_px * kBwdChunk; i += 256) {
+      const float v = win[i];
+      if (v != 0.0f) {
+        const int cc = i / win_px, q = i - cc * win_px;
+        const int y = wy0 + q / a.WW, x = wx0 + q % a.WW;  // in the image: only valid corners were added
+        unsafeAtomicAdd(a.gin32 + ((long)n * g.Cin + c0 + cc) * plane_in + (long)y * g.W + x, v);
+      }
+    }
+    c0 += cn;
+  }
+  if (valid) {
+    E *goff = (E *)a.goff, *gmask = (E *)a.gmask;
+    const long ob = ((long)n * g.DG + dgi) * 2 * g.taps;
+#pragma unroll
+    for (int tap = 0; tap < kBwdTapsMax; ++tap) {
+      if (tap < g.taps) {
+        goff[(ob + 2 * tap) * plane_out + pix] = from_f32<E>(acc_y[tap]);
+        goff[(ob + 2 * tap + 1) * plane_out + pix] = from_f32<E>(acc_x[tap]);
+        if (gmask) gmask[(((long)n * g.DG + dgi) * g.taps + tap) * plane_out + pix] = from_f32<E>(acc_m[tap]);
+      }
+    }
+  }
+}
+
 struct BwdWeightArgs {
   Geom g;
   const void *input;
