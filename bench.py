@@ -304,7 +304,7 @@ def main():
             'frac': round(achieved / peak, 4),
             # HBM bytes per launch of the fused kernel on cfg4/bf16 from rocprofv3 FETCH_SIZE and
             # WRITE_SIZE, scaled by a copy kernel (profiles/fused_kernel_bf16_cfg4.md)
-            'traffic': 394.2e6 if a.workload == 'cfg4' else None,
+            'traffic': 378.3e6 if a.workload == 'cfg4' else None,
         },
     }
     if not a.no_cpu:
