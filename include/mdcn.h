@@ -191,8 +191,15 @@ typedef struct mdcn_bwd_params {
   void *grad_bias;
 } mdcn_bwd_params;
 
-/* Bytes of device scratch mdcn_backward() needs (fp32 staging of grad_input and
- * grad_weight for 16-bit tensors); may be 0. */
+/* Bytes of device scratch mdcn_backward() needs for *p as it will be passed to
+ * mdcn_backward() (gradient pointers set: which gradients are asked for decides
+ * what is staged): fp32 staging of grad_input and grad_weight for 16-bit
+ * tensors and, for shapes whose column gradient runs on the matrix cores,
+ * pixel-major copies of input and grad_output, the transposed weights and the
+ * column gradient of up to 1.5 GiB of images at a time; may be 0.
+ * conv.path: MDCN_PATH_AUTO picks by shape and size; MDCN_PATH_FUSED asks for
+ * the tiled kernels whatever the problem size (MDCN_ERR_PATH if the shape rules
+ * them out); MDCN_PATH_DIRECT keeps the one-workgroup-per-tap kernel. */
 size_t mdcn_backward_workspace_bytes(const mdcn_bwd_params *p);
 
 /* Enqueue the backward on `hip_stream`.  Returns an mdcn_status. */

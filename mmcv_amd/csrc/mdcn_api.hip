@@ -10,6 +10,7 @@
 #include "mdcn_common.h"
 #include "mdcn_direct.h"
 #include "mdcn_backward.h"
+#include "mdcn_backward_gemm.h"
 #include "mdcn_fused.h"
 #include "mdcn_oconv.h"
 #include "mdcn_prepass.h"
@@ -452,14 +453,60 @@ int run(const mdcn_params *p, void *stream, float *ms, const mdcn_pack_params *p
   }
 }
 
+// Column gradient held in memory per pass of the matrix-core data path.
+constexpr size_t kBwdColGradCap = (size_t)3 << 29;  // 1.5 GiB
+
 struct BwdPlan {
   size_t gin_bytes, gw_bytes;  // fp32 staging (0 for fp32 tensors)
+  // grad_input / grad_offset / grad_mask:
+  bool tiled;      // 16 x 16 pixel tiles with an LDS window (else one workgroup per tap)
+  int R, WH, WW;   // window margin and size
+  bool gemm;       // column gradient by bwd_colgrad_kernel, handed over through the workspace
+  int n_chunk;     // images per pass of that path
+  int M_pad;       // rows of the transposed weight matrix per group
+  size_t xt_bytes, gt_bytes, wt_bytes, d_bytes;
+  size_t total() const { return gin_bytes + gw_bytes + xt_bytes + gt_bytes + wt_bytes + d_bytes; }
 };
 
 void make_bwd_plan(const mdcn_bwd_params *bp, const Geom &g, BwdPlan *pl) {
   const bool staged = bp->conv.dtype != MDCN_F32;
+  const size_t es = elem_size(bp->conv.dtype);
   pl->gin_bytes = (staged && bp->grad_input) ? align_up((size_t)g.N * g.Cin * g.H * g.W * 4) : 0;
   pl->gw_bytes = (staged && bp->grad_weight) ? align_up((size_t)g.Cout * g.cin_g * g.taps * 4) : 0;
+  pl->tiled = pl->gemm = false;
+  pl->xt_bytes = pl->gt_bytes = pl->wt_bytes = pl->d_bytes = 0;
+  pl->n_chunk = g.N;
+  pl->M_pad = 0;
+  pl->R = -1;
+  pl->WH = pl->WW = 0;
+  if (!bp->grad_input) return;
+  // window of the tiled kernels: the tile's undeformed footprint plus a margin R on every side
+  const long base_h = (long)(kBwdTile - 1) * g.sh + (long)(g.kh - 1) * g.dh + 2;
+  const long base_w = (long)(kBwdTile - 1) * g.sw + (long)(g.kw - 1) * g.dw + 2;
+  const long max_px = kBwdWindowBytes / (4 * kBwdChunk);
+  int R = -1;
+  while (R < 8 && (base_h + 2 * (R + 1)) * (base_w + 2 * (R + 1)) <= max_px) ++R;
+  // (small problems keep the per-tap kernel: it has taps x more workgroups)
+  const long n_tiles = (long)g.N * g.DG * ((g.Ho + kBwdTile - 1) / kBwdTile) * ((g.Wo + kBwdTile - 1) / kBwdTile);
+  const int path = bp->conv.path;
+  if (path == MDCN_PATH_DIRECT) return;
+  if (!(g.taps <= kBwdTapsMax && R >= 1 && (n_tiles >= 512 || path == MDCN_PATH_FUSED))) return;
+  pl->tiled = true;
+  pl->R = R;
+  pl->WH = (int)base_h + 2 * R;
+  pl->WW = (int)base_w + 2 * R;
+  const int KC = (int)(128 / es);
+  if (g.Cin % KC || g.cout_g % KC || g.cin_g % 32 || g.ch_per_dg % kBwdChunk) return;
+  const size_t plane_out = (size_t)g.Ho * g.Wo;
+  const size_t d_img = (size_t)g.taps * g.Cin * plane_out * es;
+  if (d_img > kBwdColGradCap || plane_out > (size_t)1 << 30) return;
+  pl->gemm = true;
+  pl->n_chunk = (int)std::min<size_t>((size_t)g.N, kBwdColGradCap / d_img);
+  pl->M_pad = (g.taps * g.cin_g + kCgTile - 1) / kCgTile * kCgTile;
+  pl->xt_bytes = align_up((size_t)g.N * (g.Cin / KC) * g.Hp * g.Wp * 128);
+  pl->gt_bytes = align_up((size_t)g.N * (g.Cout / KC) * plane_out * 128);
+  pl->wt_bytes = align_up((size_t)g.G * pl->M_pad * g.cout_g * es);
+  pl->d_bytes = align_up(d_img * pl->n_chunk);
 }
 
 template <typename E>
@@ -477,15 +524,74 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
     float *gin32 = pl.gin_bytes ? (float *)ws : (float *)bp->grad_input;
     hipLaunchKernelGGL(fill_zero_kernel<float>, dim3(blocks_for(n_in)), dim3(256), 0, st, gin32, n_in);
     check();
-    // window of the tiled kernel: the tile's undeformed footprint plus a margin R on every side
-    const int base_h = (kBwdTile - 1) * g.sh + (g.kh - 1) * g.dh + 2;
-    const int base_w = (kBwdTile - 1) * g.sw + (g.kw - 1) * g.dw + 2;
-    const int max_px = kBwdWindowBytes / (4 * kBwdChunk);
-    int R = -1;
-    while (R < 8 && (base_h + 2 * (R + 1)) * (base_w + 2 * (R + 1)) <= max_px) ++R;
-    // (small problems keep the per-tap kernel: it has taps x more workgroups)
-    const long n_tiles = (long)g.N * g.DG * ((g.Ho + kBwdTile - 1) / kBwdTile) * ((g.Wo + kBwdTile - 1) / kBwdTile);
-    if (g.taps <= kBwdTapsMax && R >= 1 && n_tiles >= 2L * num_cus()) {
+    const int tiles_x = (g.Wo + kBwdTile - 1) / kBwdTile, tiles_y = (g.Ho + kBwdTile - 1) / kBwdTile;
+    if (pl.gemm) {
+      constexpr int KC = 128 / (int)sizeof(E);
+      unsigned char *xt = ws + pl.gin_bytes + pl.gw_bytes;
+      unsigned char *gT = xt + pl.xt_bytes;
+      unsigned char *wT = gT + pl.gt_bytes;
+      unsigned char *D = wT + pl.wt_bytes;
+      {  // pixel-major copies of the input (zero border) and of grad_output (plain)
+        const int n_pchunks = (g.H * g.W + 127) / 128;
+        const int words_ok = ((g.H * g.W) % 2 == 0) && (((uintptr_t)p->input % 4) == 0);
+        hipLaunchKernelGGL(relayout_kernel<E>, dim3((unsigned)((long)g.N * (g.Cin / KC) * n_pchunks)),
+                           dim3(256), 0, st, g, (const E *)p->input, (E *)xt, n_pchunks, words_ok);
+        check();
+        Geom gg = g;
+        gg.Cin = g.Cout;
+        gg.H = g.Ho;
+        gg.W = g.Wo;
+        const int o_pchunks = (int)((plane_out + 127) / 128);
+        const int o_words_ok = (plane_out % 2 == 0) && (((uintptr_t)bp->grad_output % 4) == 0);
+        hipLaunchKernelGGL((relayout_kernel<E, false>), dim3((unsigned)((long)g.N * (g.Cout / KC) * o_pchunks)),
+                           dim3(256), 0, st, gg, (const E *)bp->grad_output, (E *)gT, o_pchunks, o_words_ok);
+        check();
+        const long wtotal = (long)g.G * pl.M_pad * g.cout_g;
+        hipLaunchKernelGGL(pack_weight_t_kernel<E>, dim3(blocks_for(wtotal)), dim3(256), 0, st, g,
+                           (const E *)p->weight, (E *)wT, pl.M_pad, wtotal);
+        check();
+      }
+      for (int n0 = 0; n0 < g.N; n0 += pl.n_chunk) {
+        const int nb = std::min(pl.n_chunk, g.N - n0);
+        ColGradArgs ca;
+        ca.wT = wT;
+        ca.gT = gT;
+        ca.D = D;
+        ca.P = (int)plane_out;
+        ca.px_tiles = (int)((plane_out + kCgTile - 1) / kCgTile);
+        ca.m_tiles = pl.M_pad / kCgTile;
+        ca.M = g.taps * g.cin_g;
+        ca.M_pad = pl.M_pad;
+        ca.cin_g = g.cin_g;
+        ca.cout_g = g.cout_g;
+        ca.taps = g.taps;
+        ca.G = g.G;
+        ca.Cin = g.Cin;
+        ca.Cout = g.Cout;
+        ca.kslabs = g.cout_g / KC;
+        ca.n0 = n0;
+        const long cblocks = (long)nb * g.G * ca.px_tiles * ca.m_tiles;
+        hipLaunchKernelGGL(bwd_colgrad_kernel<E>, dim3((unsigned)cblocks), dim3(256), 0, st, ca);
+        check();
+        BwdScatterArgs sa;
+        sa.g = g;
+        sa.xt = xt;
+        sa.om = om;
+        sa.D = D;
+        sa.gin32 = gin32;
+        sa.goff = bp->grad_offset;
+        sa.gmask = bp->grad_mask;
+        sa.tiles_x = tiles_x;
+        sa.tiles_y = tiles_y;
+        sa.R = pl.R;
+        sa.WH = pl.WH;
+        sa.WW = pl.WW;
+        sa.n0 = n0;
+        const long sblocks = (long)nb * g.DG * tiles_y * tiles_x;
+        hipLaunchKernelGGL(bwd_scatter_kernel<E>, dim3((unsigned)sblocks), dim3(256), 0, st, sa);
+        check();
+      }
+    } else if (pl.tiled) {
       BwdDataTiledArgs da;
       da.g = g;
       da.input = p->input;
@@ -495,11 +601,11 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
       da.gin32 = gin32;
       da.goff = bp->grad_offset;
       da.gmask = bp->grad_mask;
-      da.tiles_x = (g.Wo + kBwdTile - 1) / kBwdTile;
-      da.tiles_y = (g.Ho + kBwdTile - 1) / kBwdTile;
-      da.R = R;
-      da.WH = base_h + 2 * R;
-      da.WW = base_w + 2 * R;
+      da.tiles_x = tiles_x;
+      da.tiles_y = tiles_y;
+      da.R = pl.R;
+      da.WH = pl.WH;
+      da.WW = pl.WW;
       const long blocks = (long)g.N * g.DG * da.tiles_y * da.tiles_x;
       hipLaunchKernelGGL(bwd_data_tiled_kernel<E>, dim3((unsigned)blocks), dim3(256), 0, st, da);
     } else {
@@ -564,6 +670,11 @@ int check_bwd(const mdcn_bwd_params *bp, Geom *g, bool need_ptrs) {
   if (data != (bp->grad_offset != nullptr)) return MDCN_ERR_NULL;
   if (p->mask ? (data != (bp->grad_mask != nullptr)) : (bp->grad_mask != nullptr)) return MDCN_ERR_NULL;
   if ((uint64_t)g->N * g->DG * g->taps > 0x7fffffffull) return MDCN_ERR_TOO_LARGE;
+  if (p->path == MDCN_PATH_FUSED && data) {  // asked for the tiled kernels: the shape must allow them
+    BwdPlan pl;
+    make_bwd_plan(bp, *g, &pl);
+    if (!pl.tiled) return MDCN_ERR_PATH;
+  }
   return MDCN_OK;
 }
 
@@ -637,7 +748,7 @@ size_t mdcn_backward_workspace_bytes(const mdcn_bwd_params *bp) {
   if (check_bwd(bp, &g, false) != MDCN_OK) return 0;
   BwdPlan pl;
   make_bwd_plan(bp, g, &pl);
-  return pl.gin_bytes + pl.gw_bytes;
+  return pl.total();
 }
 
 int mdcn_backward(const mdcn_bwd_params *bp, void *hip_stream) {
@@ -646,7 +757,7 @@ int mdcn_backward(const mdcn_bwd_params *bp, void *hip_stream) {
   if (rc != MDCN_OK) return rc;
   BwdPlan pl;
   make_bwd_plan(bp, g, &pl);
-  const size_t need = pl.gin_bytes + pl.gw_bytes;
+  const size_t need = pl.total();
   const mdcn_params *p = &bp->conv;
   if (need > 0 && (!p->workspace || p->workspace_bytes < need || ((uintptr_t)p->workspace % kAlign) != 0))
     return MDCN_ERR_WORKSPACE;

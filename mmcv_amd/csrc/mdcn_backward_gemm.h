@@ -1,0 +1,363 @@
+// Backward, data side, for channel counts that fill MFMA tiles: the column
+// gradient  d[pixel, (tap, c)] = sum_co grad_output[co, pixel] * weight[co, c, tap]
+// (the reference's first GEMM, mmcv/ops/csrc/pytorch/modulated_deform_conv.cpp:199-206)
+// is a plain matrix product, so it runs on the matrix cores
+// (bwd_colgrad_kernel) and is handed to the scatter kernel through memory in a
+// layout made for that kernel: d[image][16-channel chunk][tap][pixel][16].  The
+// scatter kernel (bwd_scatter_kernel) then is the reference's three element-wise
+// kernels in one pass (cpu/modulated_deform_conv.cpp:34-107,170-320): a thread
+// owns an output pixel, reads 16 channels of d and of the four corners (from the
+// zero-bordered pixel-major input copy, 32 or 64 contiguous bytes per corner),
+// forms its share of grad_offset / grad_mask in registers, and adds the
+// grad_input contributions into an fp32 LDS window around its 16 x 16 pixel
+// tile, which is flushed with one global atomic per non-zero entry.
+// Both operands of the product are pixel-major / K-contiguous copies written by
+// small pre-passes (relayout_kernel<E, false> for grad_output,
+// pack_weight_t_kernel for the weights).
+#pragma once
+
+#include "mdcn_backward.h"
+
+namespace mdcn {
+
+// Rows of either operand per workgroup tile of the column-gradient product.
+constexpr int kCgTile = 128;
+
+// weight[Cout][cin_g][taps] -> wT[G][M_pad][cout_g], row m = tap * cin_g + c,
+// zero rows from taps * cin_g up to M_pad (a multiple of kCgTile).
+template <typename E>
+__global__ __launch_bounds__(256) void pack_weight_t_kernel(Geom g, const E *__restrict__ w,
+                                                            E *__restrict__ wT, int M_pad, long total) {
+  for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (long)gridDim.x * blockDim.x) {
+    long r = idx;
+    const int co = (int)(r % g.cout_g);
+    r /= g.cout_g;
+    const int m = (int)(r % M_pad);
+    const int grp = (int)(r / M_pad);
+    E v = from_f32<E>(0.0f);
+    if (m < g.taps * g.cin_g) {
+      const int tap = m / g.cin_g, c = m - tap * g.cin_g;
+      v = w[((long)(grp * g.cout_g + co) * g.cin_g + c) * g.taps + tap];
+    }
+    wT[idx] = v;
+  }
+}
+
+struct ColGradArgs {
+  const void *wT;  // [G][M_pad][cout_g]
+  const void *gT;  // [N][Cout / KC][P][KC], KC = 128 bytes of channels
+  void *D;         // [images of the pass][Cin / 16][taps][P][16]
+  int P;           // output pixels per image
+  int px_tiles, m_tiles;
+  int M, M_pad;    // taps * cin_g and its padded size
+  int cin_g, cout_g, taps, G, Cin, Cout;
+  int kslabs;      // cout_g / KC
+  int n0;          // first image of the pass
+};
+
+// Workgroup = 128 rows of wT (one group) x 128 pixels of one image, reduction
+// over the group's output channels in slabs of 128 bytes; 4 waves as 2 x 2, each
+// 2 x 2 MFMA blocks of 32 x 32.  Both operand tiles of a slab go to LDS with
+// 16-byte direct-to-LDS copies (rows of 128 bytes, the 16-byte chunks of a row
+// swizzled by the row number on the source side, so that fragment reads are
+// conflict free), double buffered.  A rows = (tap, channel), B rows = pixels:
+// a lane ends up with 4 x 4 consecutive channels of one pixel, which is what the
+// d layout wants (8- or 16-byte stores).
+template <typename E>
+__global__ __launch_bounds__(256, 2) void bwd_colgrad_kernel(ColGradArgs a) {
+  using TR = ElemTraits<E>;
+  constexpr int ES = (int)sizeof(E);
+  constexpr int KC = 128 / ES;
+  __shared__ uint4 As[2][kCgTile * 8];
+  __shared__ uint4 Bs[2][kCgTile * 8];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int frow = lane & 31, fhalf = lane >> 5;
+  const int wm = wave & 1, wn = wave >> 1;
+  int b = blockIdx.x;
+  const int mt = b % a.m_tiles;
+  b /= a.m_tiles;
+  const int pt = b % a.px_tiles;
+  b /= a.px_tiles;
+  const int grp = b % a.G;
+  const int nl = b / a.G;
+  const int n = a.n0 + nl;
+
+  // this lane's share of the copies: 4 of the 16 one-KiB blocks (8 rows) of each tile
+  const unsigned char *a_src[4], *b_src[4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const int row = (wave * 4 + c) * 8 + (lane >> 3);
+    const int ch = (lane & 7) ^ (row & 7);
+    a_src[c] = (const unsigned char *)a.wT +
+               ((long)grp * a.M_pad + (long)mt * kCgTile + row) * a.cout_g * ES + ch * 16;
+    // rows past the image repeat its last pixel; they are never stored
+    const int px = min(pt * kCgTile + row, a.P - 1);
+    b_src[c] = (const unsigned char *)a.gT +
+               (((long)n * (a.Cout / KC) + (long)grp * a.kslabs) * a.P + px) * 128 + ch * 16;
+  }
+  const long b_step = (long)a.P * 128;
+  const uint32_t lds_a = (uint32_t)(uintptr_t)(lptr_t)(&As[0][0]) +
+                         (uint32_t)__builtin_amdgcn_readfirstlane(wave) * 4096u;
+  const uint32_t lds_b = (uint32_t)(uintptr_t)(lptr_t)(&Bs[0][0]) +
+                         (uint32_t)__builtin_amdgcn_readfirstlane(wave) * 4096u;
+  auto issue = [&](int ks, int buf) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      copy16_global_to_lds(a_src[c] + (long)ks * 128, lds_a + (uint32_t)buf * 16384u + (uint32_t)c * 1024u);
+      copy16_global_to_lds(b_src[c] + (long)ks * b_step, lds_b + (uint32_t)buf * 16384u + (uint32_t)c * 1024u);
+    }
+  };
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  issue(0, 0);
+  for (int ks = 0; ks < a.kslabs; ++ks) {
+    const int buf = ks & 1;
+    if (ks + 1 < a.kslabs) {
+      issue(ks + 1, buf ^ 1);  // (its buffer was last read before the barrier that ended step ks - 1)
+      asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    __syncthreads();
+#pragma unroll
+    for (int ksub = 0; ksub < 4; ++ksub) {
+      uint4 af[2], bf[2];
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb) {
+        const int row = wm * 64 + mb * 32 + frow;
+        af[mb] = As[buf][row * 8 + ((ksub * 2 + fhalf) ^ (row & 7))];
+      }
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb) {
+        const int row = wn * 64 + nb * 32 + frow;
+        bf[nb] = Bs[buf][row * 8 + ((ksub * 2 + fhalf) ^ (row & 7))];
+      }
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) TR::mma(acc[mb][nb], af[mb], bf[nb]);
+    }
+    __syncthreads();
+  }
+
+  // register r of lane l: A row (r/4)*8 + (l/32)*4 + r%4 of the block, B row l%32
+  E *D = (E *)a.D;
+  const int chunks = a.Cin / 16;
+#pragma unroll
+  for (int mb = 0; mb < 2; ++mb) {
+    const int m0 = mt * kCgTile + wm * 64 + mb * 32;  // a block = one tap, 32 consecutive channels
+    if (m0 >= a.M) continue;
+    const int tap = m0 / a.cin_g;
+    const int cb = grp * a.cin_g + (m0 - tap * a.cin_g);
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) {
+      const int px = pt * kCgTile + wn * 64 + nb * 32 + frow;
+      if (px >= a.P) continue;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int c = cb + j * 8 + fhalf * 4;
+        E *dst = D + ((((long)nl * chunks + (c >> 4)) * a.taps + tap) * a.P + px) * 16 + (c & 15);
+        TR::store4((unsigned char *)dst, acc[mb][nb][4 * j], acc[mb][nb][4 * j + 1],
+                   acc[mb][nb][4 * j + 2], acc[mb][nb][4 * j + 3]);
+      }
+    }
+  }
+}
+
+// 16 consecutive channels (32 or 64 bytes) as floats.
+template <typename E>
+struct Vec16 {
+  static constexpr int NV = (int)sizeof(E);  // 16-byte loads per 16 channels
+  uint4 raw[NV];
+  __device__ __forceinline__ void load(const E *p) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) raw[i] = ((const uint4 *)p)[i];
+  }
+  __device__ __forceinline__ void unpack(float (&out)[16]) const;
+};
+template <>
+__device__ __forceinline__ void Vec16<float>::unpack(float (&out)[16]) const {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    out[4 * i] = __uint_as_float(raw[i].x);
+    out[4 * i + 1] = __uint_as_float(raw[i].y);
+    out[4 * i + 2] = __uint_as_float(raw[i].z);
+    out[4 * i + 3] = __uint_as_float(raw[i].w);
+  }
+}
+template <>
+__device__ __forceinline__ void Vec16<bf16_t>::unpack(float (&out)[16]) const {
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const uint32_t w[4] = {raw[i].x, raw[i].y, raw[i].z, raw[i].w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      out[8 * i + 2 * j] = __uint_as_float(w[j] << 16);
+      out[8 * i + 2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+    }
+  }
+}
+template <>
+__device__ __forceinline__ void Vec16<f16_t>::unpack(float (&out)[16]) const {
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const uint32_t w[4] = {raw[i].x, raw[i].y, raw[i].z, raw[i].w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const f16x2 p = __builtin_bit_cast(f16x2, w[j]);
+      out[8 * i + 2 * j] = (float)p.x;
+      out[8 * i + 2 * j + 1] = (float)p.y;
+    }
+  }
+}
+
+struct BwdScatterArgs {
+  Geom g;
+  const void *xt;  // zero-bordered pixel-major input copy [N][Cin / KC][H + 2][W + 2][KC]
+  OffMaskView om;
+  const void *D;   // column gradient of the pass, layout of ColGradArgs::D
+  float *gin32;
+  void *goff;
+  void *gmask;     // null when unmodulated
+  int tiles_x, tiles_y;
+  int WH, WW;      // window size in input pixels
+  int R;           // margin of the window around the tile's undeformed footprint
+  int n0;          // first image of the pass
+};
+
+template <typename E>
+__global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
+  constexpr int KC = 128 / (int)sizeof(E);
+  __shared__ float win[kBwdWindowBytes / 4];
+  const Geom &g = a.g;
+  const long plane_out = (long)g.Ho * g.Wo;
+  const long plane_in = (long)g.H * g.W;
+  const long slab_px = (long)g.Hp * g.Wp;
+  const int tid = threadIdx.x;
+  int b = blockIdx.x;
+  const int tx = b % a.tiles_x;
+  b /= a.tiles_x;
+  const int ty = b % a.tiles_y;
+  b /= a.tiles_y;
+  const int dgi = b % g.DG;
+  const int nl = b / g.DG;
+  const int n = a.n0 + nl;
+  const int ho = ty * kBwdTile + (tid >> 4), wo = tx * kBwdTile + (tid & 15);
+  const bool valid = ho < g.Ho && wo < g.Wo;
+  const long pix = valid ? (long)ho * g.Wo + wo : 0;
+  const int wy0 = ty * kBwdTile * g.sh - g.ph - a.R, wx0 = tx * kBwdTile * g.sw - g.pw - a.R;
+  const int win_px = a.WH * a.WW;
+
+  const E *off = (const E *)a.om.off + (long)n * a.om.off_n + pix * a.om.off_px +
+                 (long)(dgi * 2 * g.taps) * a.om.off_ch;
+  const E *msk = (const E *)a.om.msk + (long)n * a.om.msk_n + pix * a.om.msk_px +
+                 (long)(dgi * g.taps) * a.om.msk_ch;
+
+  float acc_m[kBwdTapsMax], acc_y[kBwdTapsMax], acc_x[kBwdTapsMax];
+#pragma unroll
+  for (int t = 0; t < kBwdTapsMax; ++t) acc_m[t] = acc_y[t] = acc_x[t] = 0.0f;
+
+  const int c_begin = dgi * g.ch_per_dg, c_end = c_begin + g.ch_per_dg;
+  for (int c0 = c_begin; c0 < c_end; c0 += kBwdChunk) {
+    __syncthreads();  // the previous chunk's flush is done
+    for (int i = tid; i < win_px * kBwdChunk; i += 256) win[i] = 0.0f;
+    __syncthreads();
+    const E *dbase = (const E *)a.D + (((long)nl * (g.Cin / 16) + (c0 >> 4)) * g.taps) * plane_out * 16 + pix * 16;
+    const E *xbase = (const E *)a.xt + (((long)n * (g.Cin / KC) + c0 / KC) * slab_px) * KC + (c0 % KC);
+#pragma unroll
+    for (int tap = 0; tap < kBwdTapsMax; ++tap) {
+      if (tap < g.taps) {
+        const int ti = tap / g.kw, tj = tap - ti * g.kw;
+        const float dy = to_f32(off[(long)(2 * tap) * a.om.off_ch]);
+        const float dx = to_f32(off[(long)(2 * tap + 1) * a.om.off_ch]);
+        const float m = mask_value<E>(msk[(long)tap * a.om.msk_ch], a.om.logit);
+        const float py = (float)(ho * g.sh - g.ph + ti * g.dh) + dy;
+        const float px = (float)(wo * g.sw - g.pw + tj * g.dw) + dx;
+        const bool inside =
+            valid && (py > -1.0f) && (px > -1.0f) && (py < (float)g.H) && (px < (float)g.W);
+        if (inside) {
+          const float fy = floorf(py), fx = floorf(px);
+          const int y0 = (int)fy, x0 = (int)fx, y1 = y0 + 1, x1 = x0 + 1;
+          const float ly = py - fy, lx = px - fx, hy = 1.0f - ly, hx = 1.0f - lx;
+          const bool ok00 = y0 >= 0 && x0 >= 0, ok01 = y0 >= 0 && x1 <= g.W - 1;
+          const bool ok10 = y1 <= g.H - 1 && x0 >= 0, ok11 = y1 <= g.H - 1 && x1 <= g.W - 1;
+          // corners outside the image read the copy's zero border
+          const E *xp = xbase + ((long)(y0 + 1) * g.Wp + (x0 + 1)) * KC;
+          Vec16<E> rd, r00, r01, r10, r11;
+          rd.load(dbase + (long)tap * plane_out * 16);
+          r00.load(xp);
+          r01.load(xp + KC);
+          r10.load(xp + (long)g.Wp * KC);
+          r11.load(xp + (long)(g.Wp + 1) * KC);
+          float d[16], v00[16], v01[16], v10[16], v11[16];
+          rd.unpack(d);
+          r00.unpack(v00);
+          r01.unpack(v01);
+          r10.unpack(v10);
+          r11.unpack(v11);
+          const int ry = y0 - wy0, rx = x0 - wx0;
+          const bool in_win = ry >= 0 && ry + 1 < a.WH && rx >= 0 && rx + 1 < a.WW;
+          const int wbase = ry * a.WW + rx;  // window is [channel][WH][WW]: neighbouring pixels, neighbouring banks
+          const long o00 = (long)y0 * g.W + x0, o01 = o00 + 1, o10 = o00 + g.W, o11 = o10 + 1;
+          const float w00 = hy * hx, w01 = hy * lx, w10 = ly * hx, w11 = ly * lx;
+          float am = 0.0f, ay = 0.0f, ax = 0.0f;
+#pragma unroll
+          for (int cc = 0; cc < kBwdChunk; ++cc) {
+            const float dc = d[cc];
+            am += dc * (w00 * v00[cc] + w01 * v01[cc] + w10 * v10[cc] + w11 * v11[cc]);
+            ay += dc * (hx * (v10[cc] - v00[cc]) + lx * (v11[cc] - v01[cc]));
+            ax += dc * (hy * (v01[cc] - v00[cc]) + ly * (v11[cc] - v10[cc]));
+            const float t = dc * m;
+            if (in_win) {
+              float *wp = win + cc * win_px + wbase;
+              if (ok00) atomicAdd(wp, w00 * t);
+              if (ok01) atomicAdd(wp + 1, w01 * t);
+              if (ok10) atomicAdd(wp + a.WW, w10 * t);
+              if (ok11) atomicAdd(wp + a.WW + 1, w11 * t);
+            } else {
+              float *gi = a.gin32 + ((long)n * g.Cin + c0 + cc) * plane_in;
+              if (ok00) unsafeAtomicAdd(gi + o00, w00 * t);
+              if (ok01) unsafeAtomicAdd(gi + o01, w01 * t);
+              if (ok10) unsafeAtomicAdd(gi + o10, w10 * t);
+              if (ok11) unsafeAtomicAdd(gi + o11, w11 * t);
+            }
+          }
+          acc_m[tap] += am;
+          acc_y[tap] += ay * m;
+          acc_x[tap] += ax * m;
+        }
+      }
+    }
+    __syncthreads();  // every add into the window has landed
+    for (int i = tid; i < win_px * kBwdChunk; i += 256) {
+      const float v = win[i];
+      if (v != 0.0f) {
+        const int cc = i / win_px, q = i - cc * win_px;
+        const int y = wy0 + q / a.WW, x = wx0 + q % a.WW;  // in the image: only valid corners were added
+        unsafeAtomicAdd(a.gin32 + ((long)n * g.Cin + c0 + cc) * plane_in + (long)y * g.W + x, v);
+      }
+    }
+  }
+  if (valid) {
+    E *goff = (E *)a.goff, *gmask = (E *)a.gmask;
+    const long ob = ((long)n * g.DG + dgi) * 2 * g.taps;
+#pragma unroll
+    for (int tap = 0; tap < kBwdTapsMax; ++tap) {
+      if (tap < g.taps) {
+        goff[(ob + 2 * tap) * plane_out + pix] = from_f32<E>(acc_y[tap]);
+        goff[(ob + 2 * tap + 1) * plane_out + pix] = from_f32<E>(acc_x[tap]);
+        if (gmask) gmask[(((long)n * g.DG + dgi) * g.taps + tap) * plane_out + pix] = from_f32<E>(acc_m[tap]);
+      }
+    }
+  }
+}
+
+}  // namespace mdcn

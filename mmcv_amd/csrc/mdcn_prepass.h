@@ -19,7 +19,9 @@ namespace mdcn {
 // image row also zeroes the two border pixels that follow it in the copy (right
 // border of its row, left border of the next); the first block of a plane
 // zeroes the top border row and the pixel after it, the last one the bottom row.
-template <typename E>
+// BORDER = false writes the plain pixel-major copy [N][Cin/KC][H*W][KC] instead
+// (the backward's pixel-major grad_output).
+template <typename E, bool BORDER = true>
 __global__ __launch_bounds__(256) void relayout_kernel(Geom g, const E *__restrict__ in,
                                                        E *__restrict__ xt, int n_pchunks,
                                                        int words_ok) {
@@ -74,7 +76,7 @@ __global__ __launch_bounds__(256) void relayout_kernel(Geom g, const E *__restri
   }
   __syncthreads();
   unsigned char *dst_slab =
-      (unsigned char *)xt + (((long)n * slabs_total + slab) * g.Hp * g.Wp) * 128;
+      (unsigned char *)xt + (((long)n * slabs_total + slab) * (BORDER ? (long)g.Hp * g.Wp : (long)plane)) * 128;
   const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
 #pragma unroll
   for (int it = 0; it < 4; ++it) {
@@ -85,14 +87,15 @@ __global__ __launch_bounds__(256) void relayout_kernel(Geom g, const E *__restri
       const int y = p / g.W;
       const int x = p - y * g.W;
       const uint32_t *t = tile + lp * ROWW + q * 4;
-      unsigned char *d = dst_slab + ((long)(y + 1) * g.Wp + (x + 1)) * 128 + q * 16;
+      unsigned char *d = dst_slab + (BORDER ? (long)(y + 1) * g.Wp + (x + 1) : (long)p) * 128 + q * 16;
       *(uint4 *)d = make_uint4(t[0], t[1], t[2], t[3]);
-      if (x == g.W - 1) {
+      if (BORDER && x == g.W - 1) {
         *(uint4 *)(d + 128) = zero;
         *(uint4 *)(d + 256) = zero;
       }
     }
   }
+  if (!BORDER) return;
   if (pc == 0)  // top border row and the left border pixel of the first image row
     for (int i = tid; i < (g.Wp + 1) * 8; i += 256) *(uint4 *)(dst_slab + (long)i * 16) = zero;
   if (pc == n_pchunks - 1)  // bottom border row

@@ -214,7 +214,7 @@ def capi_pack_forward(case, own_conv=True, raw=None, want_raw=False, path=capi.P
     return out, raw_out
 
 
-def capi_backward(case, grad_output, want_bias=True):
+def capi_backward(case, grad_output, want_bias=True, path=0):
     """mdcn_backward through ctypes on device tensors of `case` (mask None:
     unmodulated); returns (grad_input, grad_offset, grad_mask or None, grad_weight,
     grad_bias or None)."""
@@ -226,6 +226,7 @@ def capi_backward(case, grad_output, want_bias=True):
     bp.conv = capi.make_params(DT[x.dtype], N, Cin, H, W, Cout, kh, kw, case['stride'], case['padding'],
                                case['dilation'], case['groups'], case['deform_groups'])
     p = bp.conv
+    p.path = path
     keep = [t.contiguous() for t in (x, off, w, grad_output)]
     p.input, p.offset, p.weight, bp.grad_output = (t.data_ptr() for t in keep)
     g_in, g_off, g_w = torch.full_like(x, 7.0), torch.full_like(off, 7.0), torch.full_like(w, 7.0)

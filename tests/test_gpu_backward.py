@@ -6,6 +6,7 @@ import pytest
 import torch
 
 import oracle
+from mmcv_amd import capi
 from common import TOL, capi_backward, cast_case, make_case, rel_err
 
 pytestmark = pytest.mark.gpu
@@ -106,6 +107,47 @@ def test_reference_known_answer_dcnv1_module():
         assert np.allclose(_np(model.weight.grad) / batch, [[[[3.62, 0.], [0.40, 0.18]]]], wthr, wthr)
 
 
+# shapes the matrix-core column-gradient path covers (channels in whole 128-byte
+# slabs, 32-channel blocks per tap), forced onto the tiled kernels at test size
+TILED_CASES = [
+    ('c64', dict(N=2, Cin=64, Cout=64, H=20, W=19, sigma=2.0)),
+    ('c128_g2_dg2', dict(N=1, Cin=128, Cout=128, H=18, W=21, groups=2, deform_groups=2, sigma=2.5)),
+    ('c64_co192', dict(N=2, Cin=64, Cout=192, H=23, W=17, sigma=1.5)),
+    ('c64_dil2_dg4', dict(N=1, Cin=64, Cout=64, H=17, W=17, padding=2, dilation=2, deform_groups=4, sigma=3.0)),
+    ('c192_k1x3', dict(N=1, Cin=192, Cout=64, H=9, W=33, k=(1, 3), padding=(0, 1), sigma=1.0)),
+    ('c96_f32_only', dict(N=1, Cin=96, Cout=32, H=16, W=16, sigma=6.0)),
+    ('c40_window_only', dict(N=2, Cin=40, Cout=24, H=18, W=17, deform_groups=2, sigma=2.0)),
+]
+
+
+@pytest.mark.parametrize('modulated', [True, False], ids=['dcnv2', 'dcnv1'])
+@pytest.mark.parametrize('dtype', DTYPES, ids=['f32', 'bf16', 'f16'])
+@pytest.mark.parametrize('name,kw', TILED_CASES, ids=[c[0] for c in TILED_CASES])
+def test_tiled_backward_against_oracle(name, kw, dtype, modulated):
+    case = cast_case(make_case(900 + len(name), **kw), dtype)
+    if not modulated:
+        case['mask'] = torch.ones_like(case['mask'])
+    g = torch.Generator().manual_seed(11)
+    Ho, Wo = case['offset'].shape[2:]
+    gy = torch.randn(case['input'].shape[0], case['weight'].shape[0], Ho, Wo, generator=g).to(dtype)
+    geo = dict(stride=case['stride'], padding=case['padding'], dilation=case['dilation'],
+               groups=case['groups'], deform_groups=case['deform_groups'])
+    ref = oracle.backward(*[case[k].float().numpy() for k in ('input', 'offset', 'mask', 'weight')],
+                          gy.float().numpy(), True, **geo)
+    dev = cast_case(case, dtype, 'cuda')
+    if not modulated:
+        dev['mask'] = None
+    got = capi_backward(dev, gy.cuda(), path=capi.PATH_FUSED)
+    direct = capi_backward(dev, gy.cuda(), path=capi.PATH_DIRECT)
+    for nm, r, o, d in zip(NAMES, ref, got, direct):
+        if o is None:
+            assert nm == 'grad_mask' and not modulated
+            continue
+        err, err_d = rel_err(_np(o), r), rel_err(_np(d), r)
+        print(f'  {name} {dtype} {nm}: tiled {err:.2e} per-tap {err_d:.2e}', flush=True)
+        assert err <= TOL[dtype] and err_d <= TOL[dtype], (nm, err, err_d)
+
+
 def test_full_size_layer_gradients_spot_check():
     """cfg-4-like layer at reduced batch (bf16, 256 channels, 100x152): first image
     of the batch against the oracle."""
@@ -113,7 +155,7 @@ def test_full_size_layer_gradients_spot_check():
     case = cast_case(make_case(4242, N=2, Cin=256, Cout=256, H=100, W=152, sigma=2.0), dtype)
     g = torch.Generator().manual_seed(1)
     gy = torch.randn(2, 256, 100, 152, generator=g).to(dtype)
-    got = capi_backward(cast_case(case, dtype, 'cuda'), gy.cuda())
+    got = capi_backward(cast_case(case, dtype, 'cuda'), gy.cuda(), path=capi.PATH_FUSED)
     sub = {k: (case[k][:1] if k in ('input', 'offset', 'mask') else case[k]) for k in case}
     ref = oracle.backward(*[sub[k].float().numpy() for k in ('input', 'offset', 'mask', 'weight')],
                           gy[:1].float().numpy(), True, stride=(1, 1), padding=(1, 1), dilation=(1, 1), groups=1,
