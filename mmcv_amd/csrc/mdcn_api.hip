@@ -453,19 +453,38 @@ int run(const mdcn_params *p, void *stream, float *ms, const mdcn_pack_params *p
   }
 }
 
-// Column gradient held in memory per pass of the matrix-core data path.
-constexpr size_t kBwdColGradCap = (size_t)3 << 29;  // 1.5 GiB
+// Column gradient (and columns) held in memory per pass of the matrix-core paths.
+constexpr size_t kBwdColGradCap = (size_t)3 << 29;  // 1.5 GiB each
+
+// Largest margin R (up to 8) for which the LDS window of a th x tw output-pixel
+// tile fits max_px pixels; -1 if even R = 0 does not.
+int window_margin(const Geom &g, int th, int tw, long max_px, int *WH, int *WW) {
+  const long base_h = (long)(th - 1) * g.sh + (long)(g.kh - 1) * g.dh + 2;
+  const long base_w = (long)(tw - 1) * g.sw + (long)(g.kw - 1) * g.dw + 2;
+  int R = -1;
+  while (R < 8 && (base_h + 2 * (R + 1)) * (base_w + 2 * (R + 1)) <= max_px) ++R;
+  *WH = (int)base_h + 2 * std::max(R, 0);
+  *WW = (int)base_w + 2 * std::max(R, 0);
+  return R;
+}
 
 struct BwdPlan {
   size_t gin_bytes, gw_bytes;  // fp32 staging (0 for fp32 tensors)
-  // grad_input / grad_offset / grad_mask:
-  bool tiled;      // 16 x 16 pixel tiles with an LDS window (else one workgroup per tap)
-  int R, WH, WW;   // window margin and size
-  bool gemm;       // column gradient by bwd_colgrad_kernel, handed over through the workspace
-  int n_chunk;     // images per pass of that path
+  // grad_input / grad_offset / grad_mask by bwd_data_tiled_kernel (else, without
+  // `gemm`, one workgroup per tap):
+  bool tiled;
+  int R, WH, WW;   // its window margin and size
+  // matrix-core paths (bwd_colgrad_kernel + bwd_scatter_kernel, bwd_wgrad_kernel):
+  bool gemm;       // data gradients
+  bool wgemm;      // grad_weight from stored columns
+  int sR, sWH, sWW;  // window of the scatter kernel
+  int n_chunk;     // images per pass
   int M_pad;       // rows of the transposed weight matrix per group
-  size_t xt_bytes, gt_bytes, wt_bytes, d_bytes;
-  size_t total() const { return gin_bytes + gw_bytes + xt_bytes + gt_bytes + wt_bytes + d_bytes; }
+  long P_pad;      // row pitch of the columns matrix
+  size_t xt_bytes, gt_bytes, wt_bytes, d_bytes, col_bytes;
+  size_t total() const {
+    return gin_bytes + gw_bytes + xt_bytes + gt_bytes + wt_bytes + d_bytes + col_bytes;
+  }
 };
 
 void make_bwd_plan(const mdcn_bwd_params *bp, const Geom &g, BwdPlan *pl) {
@@ -473,86 +492,119 @@ void make_bwd_plan(const mdcn_bwd_params *bp, const Geom &g, BwdPlan *pl) {
   const size_t es = elem_size(bp->conv.dtype);
   pl->gin_bytes = (staged && bp->grad_input) ? align_up((size_t)g.N * g.Cin * g.H * g.W * 4) : 0;
   pl->gw_bytes = (staged && bp->grad_weight) ? align_up((size_t)g.Cout * g.cin_g * g.taps * 4) : 0;
-  pl->tiled = pl->gemm = false;
-  pl->xt_bytes = pl->gt_bytes = pl->wt_bytes = pl->d_bytes = 0;
+  pl->tiled = pl->gemm = pl->wgemm = false;
+  pl->xt_bytes = pl->gt_bytes = pl->wt_bytes = pl->d_bytes = pl->col_bytes = 0;
   pl->n_chunk = g.N;
   pl->M_pad = 0;
-  pl->R = -1;
-  pl->WH = pl->WW = 0;
-  if (!bp->grad_input) return;
-  // window of the tiled kernels: the tile's undeformed footprint plus a margin R on every side
-  const long base_h = (long)(kBwdTile - 1) * g.sh + (long)(g.kh - 1) * g.dh + 2;
-  const long base_w = (long)(kBwdTile - 1) * g.sw + (long)(g.kw - 1) * g.dw + 2;
-  const long max_px = kBwdWindowBytes / (4 * kBwdChunk);
-  int R = -1;
-  while (R < 8 && (base_h + 2 * (R + 1)) * (base_w + 2 * (R + 1)) <= max_px) ++R;
-  // (small problems keep the per-tap kernel: it has taps x more workgroups)
-  const long n_tiles = (long)g.N * g.DG * ((g.Ho + kBwdTile - 1) / kBwdTile) * ((g.Wo + kBwdTile - 1) / kBwdTile);
+  pl->P_pad = 0;
+  pl->R = pl->sR = -1;
+  pl->WH = pl->WW = pl->sWH = pl->sWW = 0;
   const int path = bp->conv.path;
-  if (path == MDCN_PATH_DIRECT) return;
-  if (!(g.taps <= kBwdTapsMax && R >= 1 && (n_tiles >= 512 || path == MDCN_PATH_FUSED))) return;
-  pl->tiled = true;
-  pl->R = R;
-  pl->WH = (int)base_h + 2 * R;
-  pl->WW = (int)base_w + 2 * R;
-  const int KC = (int)(128 / es);
-  if (g.Cin % KC || g.cout_g % KC || g.cin_g % 32 || g.ch_per_dg % kBwdChunk) return;
+  if (path == MDCN_PATH_DIRECT || g.taps > kBwdTapsMax) return;
+  const bool forced = path == MDCN_PATH_FUSED;
   const size_t plane_out = (size_t)g.Ho * g.Wo;
+
+  // matrix-core paths: channels in whole 128-byte slabs, 32-channel blocks per tap
+  const int KC = (int)(128 / es);
   const size_t d_img = (size_t)g.taps * g.Cin * plane_out * es;
-  if (d_img > kBwdColGradCap || plane_out > (size_t)1 << 30) return;
-  pl->gemm = true;
-  pl->n_chunk = (int)std::min<size_t>((size_t)g.N, kBwdColGradCap / d_img);
-  pl->M_pad = (g.taps * g.cin_g + kCgTile - 1) / kCgTile * kCgTile;
-  pl->xt_bytes = align_up((size_t)g.N * (g.Cin / KC) * g.Hp * g.Wp * 128);
-  pl->gt_bytes = align_up((size_t)g.N * (g.Cout / KC) * plane_out * 128);
-  pl->wt_bytes = align_up((size_t)g.G * pl->M_pad * g.cout_g * es);
-  pl->d_bytes = align_up(d_img * pl->n_chunk);
+  pl->sR = window_margin(g, kScTH, kScTW, kBwdWindowBytes / (8 * kScChunk), &pl->sWH, &pl->sWW);
+  const long s_tiles = (long)g.N * g.DG * ((g.Ho + kScTH - 1) / kScTH) * ((g.Wo + kScTW - 1) / kScTW);
+  const bool mfma_ok = g.Cin % KC == 0 && g.cout_g % KC == 0 && g.cin_g % 32 == 0 &&
+                       g.ch_per_dg % kScChunk == 0 && pl->sR >= 1 && (s_tiles >= 512 || forced) &&
+                       d_img <= kBwdColGradCap && plane_out <= ((size_t)1 << 30);
+  if (mfma_ok) {
+    pl->gemm = bp->grad_input != nullptr;
+    // (grad_output rows are copied to LDS 16 bytes at a time)
+    pl->wgemm = bp->grad_weight != nullptr && plane_out % (16 / es) == 0;
+  }
+  if (pl->gemm || pl->wgemm) {
+    pl->n_chunk = (int)std::min<size_t>((size_t)g.N, kBwdColGradCap / d_img);
+    pl->xt_bytes = align_up((size_t)g.N * (g.Cin / KC) * g.Hp * g.Wp * 128);
+  }
+  if (pl->gemm) {
+    pl->M_pad = (g.taps * g.cin_g + kCgTile - 1) / kCgTile * kCgTile;
+    pl->gt_bytes = align_up((size_t)g.N * (g.Cout / KC) * plane_out * 128);
+    pl->wt_bytes = align_up((size_t)g.G * pl->M_pad * g.cout_g * es);
+    pl->d_bytes = align_up(d_img * pl->n_chunk);
+  }
+  if (pl->wgemm) {
+    const long kpx = 128 / (long)es;  // pixels per K step
+    pl->P_pad = ((long)plane_out + kpx - 1) / kpx * kpx;
+    pl->col_bytes = align_up((size_t)pl->n_chunk * g.taps * g.Cin * pl->P_pad * es);
+  }
+  if (bp->grad_input && !pl->gemm) {
+    // (small problems keep the per-tap kernel: it has taps x more workgroups)
+    pl->R = window_margin(g, kBwdTile, kBwdTile, kBwdWindowBytes / (4 * kBwdChunk), &pl->WH, &pl->WW);
+    const long n_tiles = (long)g.N * g.DG * ((g.Ho + kBwdTile - 1) / kBwdTile) * ((g.Wo + kBwdTile - 1) / kBwdTile);
+    pl->tiled = pl->R >= 1 && (n_tiles >= 512 || forced);
+  }
 }
 
 template <typename E>
 int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &pl, hipStream_t st) {
   const mdcn_params *p = &bp->conv;
+  constexpr int KC = 128 / (int)sizeof(E);
   const long plane_out = (long)g.Ho * g.Wo;
   const OffMaskView om = dense_view(p->offset, p->mask, g);
   unsigned char *ws = (unsigned char *)p->workspace;
-  auto blocks_for = [](long n) { return (int)std::min<long>((n + 255) / 256, 1L << 20); };
+  auto blocks_for = [](long n) { return (int)std::max<long>(1, std::min<long>((n + 255) / 256, 1L << 20)); };
   int rc = MDCN_OK;
   auto check = [&]() { if (hipGetLastError() != hipSuccess) rc = MDCN_ERR_LAUNCH; };
 
+  const long n_in = (long)g.N * g.Cin * g.H * g.W;
+  const long n_w = (long)g.Cout * g.cin_g * g.taps;
+  float *gin32 = pl.gin_bytes ? (float *)ws : (float *)bp->grad_input;
+  float *gw32 = pl.gw_bytes ? (float *)(ws + pl.gin_bytes) : (float *)bp->grad_weight;
+  unsigned char *xt = ws + pl.gin_bytes + pl.gw_bytes;
+  unsigned char *gT = xt + pl.xt_bytes;
+  unsigned char *wT = gT + pl.gt_bytes;
+  unsigned char *D = wT + pl.wt_bytes;
+  unsigned char *col = D + pl.d_bytes;
+  // the weight-gradient product copies grad_output rows 16 bytes at a time
+  const bool wgemm = pl.wgemm && ((uintptr_t)bp->grad_output % 16) == 0;
+  const bool gemm = pl.gemm;
+
   if (bp->grad_input) {
-    const long n_in = (long)g.N * g.Cin * g.H * g.W;
-    float *gin32 = pl.gin_bytes ? (float *)ws : (float *)bp->grad_input;
     hipLaunchKernelGGL(fill_zero_kernel<float>, dim3(blocks_for(n_in)), dim3(256), 0, st, gin32, n_in);
     check();
-    const int tiles_x = (g.Wo + kBwdTile - 1) / kBwdTile, tiles_y = (g.Ho + kBwdTile - 1) / kBwdTile;
-    if (pl.gemm) {
-      constexpr int KC = 128 / (int)sizeof(E);
-      unsigned char *xt = ws + pl.gin_bytes + pl.gw_bytes;
-      unsigned char *gT = xt + pl.xt_bytes;
-      unsigned char *wT = gT + pl.gt_bytes;
-      unsigned char *D = wT + pl.wt_bytes;
-      {  // pixel-major copies of the input (zero border) and of grad_output (plain)
-        const int n_pchunks = (g.H * g.W + 127) / 128;
-        const int words_ok = ((g.H * g.W) % 2 == 0) && (((uintptr_t)p->input % 4) == 0);
-        hipLaunchKernelGGL(relayout_kernel<E>, dim3((unsigned)((long)g.N * (g.Cin / KC) * n_pchunks)),
-                           dim3(256), 0, st, g, (const E *)p->input, (E *)xt, n_pchunks, words_ok);
-        check();
-        Geom gg = g;
-        gg.Cin = g.Cout;
-        gg.H = g.Ho;
-        gg.W = g.Wo;
-        const int o_pchunks = (int)((plane_out + 127) / 128);
-        const int o_words_ok = (plane_out % 2 == 0) && (((uintptr_t)bp->grad_output % 4) == 0);
-        hipLaunchKernelGGL((relayout_kernel<E, false>), dim3((unsigned)((long)g.N * (g.Cout / KC) * o_pchunks)),
-                           dim3(256), 0, st, gg, (const E *)bp->grad_output, (E *)gT, o_pchunks, o_words_ok);
-        check();
-        const long wtotal = (long)g.G * pl.M_pad * g.cout_g;
-        hipLaunchKernelGGL(pack_weight_t_kernel<E>, dim3(blocks_for(wtotal)), dim3(256), 0, st, g,
-                           (const E *)p->weight, (E *)wT, pl.M_pad, wtotal);
-        check();
-      }
-      for (int n0 = 0; n0 < g.N; n0 += pl.n_chunk) {
-        const int nb = std::min(pl.n_chunk, g.N - n0);
+  }
+  if (bp->grad_weight) {
+    hipLaunchKernelGGL(fill_zero_kernel<float>, dim3(blocks_for(n_w)), dim3(256), 0, st, gw32, n_w);
+    check();
+  }
+
+  if (gemm || wgemm) {
+    {  // zero-bordered pixel-major copy of the input
+      const int n_pchunks = (g.H * g.W + 127) / 128;
+      const int words_ok = ((g.H * g.W) % 2 == 0) && (((uintptr_t)p->input % 4) == 0);
+      hipLaunchKernelGGL(relayout_kernel<E>, dim3((unsigned)((long)g.N * (g.Cin / KC) * n_pchunks)),
+                         dim3(256), 0, st, g, (const E *)p->input, (E *)xt, n_pchunks, words_ok);
+      check();
+    }
+    if (gemm) {  // pixel-major grad_output, transposed weights
+      Geom gg = g;
+      gg.Cin = g.Cout;
+      gg.H = g.Ho;
+      gg.W = g.Wo;
+      const int o_pchunks = (int)((plane_out + 127) / 128);
+      const int o_words_ok = (plane_out % 2 == 0) && (((uintptr_t)bp->grad_output % 4) == 0);
+      hipLaunchKernelGGL((relayout_kernel<E, false>), dim3((unsigned)((long)g.N * (g.Cout / KC) * o_pchunks)),
+                         dim3(256), 0, st, gg, (const E *)bp->grad_output, (E *)gT, o_pchunks, o_words_ok);
+      check();
+      const long wtotal = (long)g.G * pl.M_pad * g.cout_g;
+      hipLaunchKernelGGL(pack_weight_t_kernel<E>, dim3(blocks_for(wtotal)), dim3(256), 0, st, g,
+                         (const E *)p->weight, (E *)wT, pl.M_pad, wtotal);
+      check();
+    }
+    if (wgemm && pl.P_pad > plane_out) {
+      const long rows = (long)pl.n_chunk * g.taps * g.Cin;
+      hipLaunchKernelGGL(zero_col_pad_kernel<E>, dim3(blocks_for(rows * (pl.P_pad - plane_out))), dim3(256), 0, st,
+                         (E *)col, rows, (int)plane_out, pl.P_pad);
+      check();
+    }
+    for (int n0 = 0; n0 < g.N; n0 += pl.n_chunk) {
+      const int nb = std::min(pl.n_chunk, g.N - n0);
+      if (gemm) {
         ColGradArgs ca;
         ca.wT = wT;
         ca.gT = gT;
@@ -573,24 +625,57 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
         const long cblocks = (long)nb * g.G * ca.px_tiles * ca.m_tiles;
         hipLaunchKernelGGL(bwd_colgrad_kernel<E>, dim3((unsigned)cblocks), dim3(256), 0, st, ca);
         check();
-        BwdScatterArgs sa;
-        sa.g = g;
-        sa.xt = xt;
-        sa.om = om;
-        sa.D = D;
-        sa.gin32 = gin32;
-        sa.goff = bp->grad_offset;
-        sa.gmask = bp->grad_mask;
-        sa.tiles_x = tiles_x;
-        sa.tiles_y = tiles_y;
-        sa.R = pl.R;
-        sa.WH = pl.WH;
-        sa.WW = pl.WW;
-        sa.n0 = n0;
-        const long sblocks = (long)nb * g.DG * tiles_y * tiles_x;
-        hipLaunchKernelGGL(bwd_scatter_kernel<E>, dim3((unsigned)sblocks), dim3(256), 0, st, sa);
+      }
+      BwdScatterArgs sa;
+      sa.g = g;
+      sa.xt = xt;
+      sa.om = om;
+      sa.D = gemm ? D : nullptr;
+      sa.gin32 = gin32;
+      sa.goff = bp->grad_offset;
+      sa.gmask = bp->grad_mask;
+      sa.col = wgemm ? col : nullptr;
+      sa.P_pad = pl.P_pad;
+      sa.tiles_x = (g.Wo + kScTW - 1) / kScTW;
+      sa.tiles_y = (g.Ho + kScTH - 1) / kScTH;
+      sa.R = pl.sR;
+      sa.WH = pl.sWH;
+      sa.WW = pl.sWW;
+      sa.n0 = n0;
+      const long sblocks = (long)nb * g.DG * sa.tiles_y * sa.tiles_x;
+      hipLaunchKernelGGL(bwd_scatter_kernel<E>, dim3((unsigned)sblocks), dim3(256), 0, st, sa);
+      check();
+      if (wgemm) {
+        WGradArgs wa;
+        wa.gout = bp->grad_output;
+        wa.col = col;
+        wa.gw32 = gw32;
+        wa.P = (int)plane_out;
+        wa.P_pad = pl.P_pad;
+        wa.ksteps = (int)(pl.P_pad / KC);
+        wa.nb = nb;
+        wa.n0 = n0;
+        wa.M = g.taps * g.cin_g;
+        wa.cin_g = g.cin_g;
+        wa.cout_g = g.cout_g;
+        wa.taps = g.taps;
+        wa.G = g.G;
+        wa.Cin = g.Cin;
+        wa.Cout = g.Cout;
+        wa.co_tiles = (g.cout_g + kCgTile - 1) / kCgTile;
+        wa.m_tiles = (wa.M + kCgTile - 1) / kCgTile;
+        const long tiles = (long)g.G * wa.co_tiles * wa.m_tiles;
+        const long work = (long)nb * wa.ksteps;
+        wa.splits = (int)std::max<long>(1, std::min<long>(std::min<long>(work, 65535), (4L * num_cus() + tiles - 1) / tiles));
+        hipLaunchKernelGGL(bwd_wgrad_kernel<E>, dim3((unsigned)tiles, (unsigned)wa.splits), dim3(256), 0, st, wa);
         check();
       }
+    }
+  }
+
+  if (bp->grad_input) {
+    if (gemm) {
+      // done above
     } else if (pl.tiled) {
       BwdDataTiledArgs da;
       da.g = g;
@@ -601,21 +686,22 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
       da.gin32 = gin32;
       da.goff = bp->grad_offset;
       da.gmask = bp->grad_mask;
-      da.tiles_x = tiles_x;
-      da.tiles_y = tiles_y;
+      da.tiles_x = (g.Wo + kBwdTile - 1) / kBwdTile;
+      da.tiles_y = (g.Ho + kBwdTile - 1) / kBwdTile;
       da.R = pl.R;
       da.WH = pl.WH;
       da.WW = pl.WW;
       const long blocks = (long)g.N * g.DG * da.tiles_y * da.tiles_x;
       hipLaunchKernelGGL(bwd_data_tiled_kernel<E>, dim3((unsigned)blocks), dim3(256), 0, st, da);
+      check();
     } else {
       const int rows = g.N * g.DG * g.taps;  // (image, deformable group, tap)
       const dim3 grid((unsigned)((plane_out + 255) / 256), (unsigned)std::min(rows, 65535));
       hipLaunchKernelGGL(bwd_data_kernel<E>, grid, dim3(256), 0, st, g, (const E *)p->input, om,
                          (const E *)p->weight, (const E *)bp->grad_output, gin32,
                          (E *)bp->grad_offset, (E *)bp->grad_mask, rows);
+      check();
     }
-    check();
     if (pl.gin_bytes) {
       hipLaunchKernelGGL(round_kernel<E>, dim3(blocks_for(n_in)), dim3(256), 0, st, gin32,
                          (E *)bp->grad_input, n_in);
@@ -623,26 +709,24 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
     }
   }
   if (bp->grad_weight) {
-    const long n_w = (long)g.Cout * g.cin_g * g.taps;
-    float *gw32 = pl.gw_bytes ? (float *)(ws + pl.gin_bytes) : (float *)bp->grad_weight;
-    hipLaunchKernelGGL(fill_zero_kernel<float>, dim3(blocks_for(n_w)), dim3(256), 0, st, gw32, n_w);
-    check();
-    BwdWeightArgs wa;
-    wa.g = g;
-    wa.input = p->input;
-    wa.om = om;
-    wa.gout = bp->grad_output;
-    wa.gw32 = gw32;
-    wa.k_tiles = (g.cin_g * g.taps + 63) / 64;
-    wa.co_tiles = (g.cout_g + 255) / 256;
-    wa.px_chunks = (int)((plane_out + 63) / 64);
-    const long tiles = (long)wa.k_tiles * wa.co_tiles * g.G;
-    const long work = (long)g.N * wa.px_chunks;
-    wa.splits = (int)std::max<long>(1, std::min<long>(work, (4L * num_cus() + tiles - 1) / tiles));
-    wa.g_vec_ok = (plane_out % (16 / (long)sizeof(E)) == 0) && (((uintptr_t)bp->grad_output % 16) == 0);
-    hipLaunchKernelGGL(bwd_weight_kernel<E>, dim3((unsigned)tiles, (unsigned)wa.splits), dim3(256), 0,
-                       st, wa);
-    check();
+    if (!wgemm) {
+      BwdWeightArgs wa;
+      wa.g = g;
+      wa.input = p->input;
+      wa.om = om;
+      wa.gout = bp->grad_output;
+      wa.gw32 = gw32;
+      wa.k_tiles = (g.cin_g * g.taps + 63) / 64;
+      wa.co_tiles = (g.cout_g + 255) / 256;
+      wa.px_chunks = (int)((plane_out + 63) / 64);
+      const long tiles = (long)wa.k_tiles * wa.co_tiles * g.G;
+      const long work = (long)g.N * wa.px_chunks;
+      wa.splits = (int)std::max<long>(1, std::min<long>(work, (4L * num_cus() + tiles - 1) / tiles));
+      wa.g_vec_ok = (plane_out % (16 / (long)sizeof(E)) == 0) && (((uintptr_t)bp->grad_output % 16) == 0);
+      hipLaunchKernelGGL(bwd_weight_kernel<E>, dim3((unsigned)tiles, (unsigned)wa.splits), dim3(256), 0,
+                         st, wa);
+      check();
+    }
     if (pl.gw_bytes) {
       hipLaunchKernelGGL(round_kernel<E>, dim3(blocks_for(n_w)), dim3(256), 0, st, gw32,
                          (E *)bp->grad_weight, n_w);
@@ -670,10 +754,10 @@ int check_bwd(const mdcn_bwd_params *bp, Geom *g, bool need_ptrs) {
   if (data != (bp->grad_offset != nullptr)) return MDCN_ERR_NULL;
   if (p->mask ? (data != (bp->grad_mask != nullptr)) : (bp->grad_mask != nullptr)) return MDCN_ERR_NULL;
   if ((uint64_t)g->N * g->DG * g->taps > 0x7fffffffull) return MDCN_ERR_TOO_LARGE;
-  if (p->path == MDCN_PATH_FUSED && data) {  // asked for the tiled kernels: the shape must allow them
+  if (p->path == MDCN_PATH_FUSED) {  // asked for the tiled kernels: the shape must allow them
     BwdPlan pl;
     make_bwd_plan(bp, *g, &pl);
-    if (!pl.tiled) return MDCN_ERR_PATH;
+    if ((data && !pl.tiled && !pl.gemm) || (!data && bp->grad_weight && !pl.wgemm)) return MDCN_ERR_PATH;
   }
   return MDCN_OK;
 }

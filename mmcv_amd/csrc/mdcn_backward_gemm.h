@@ -6,11 +6,13 @@
 // layout made for that kernel: d[image][16-channel chunk][tap][pixel][16].  The
 // scatter kernel (bwd_scatter_kernel) then is the reference's three element-wise
 // kernels in one pass (cpu/modulated_deform_conv.cpp:34-107,170-320): a thread
-// owns an output pixel, reads 16 channels of d and of the four corners (from the
-// zero-bordered pixel-major input copy, 32 or 64 contiguous bytes per corner),
+// owns an output pixel, reads 8 channels of d and of the four corners (from the
+// zero-bordered pixel-major input copy, 16 or 32 contiguous bytes per corner),
 // forms its share of grad_offset / grad_mask in registers, and adds the
-// grad_input contributions into an fp32 LDS window around its 16 x 16 pixel
-// tile, which is flushed with one global atomic per non-zero entry.
+// grad_input contributions into an LDS window around its 8 x 32 pixel tile,
+// which is flushed with one global atomic per non-zero entry.  On the way it can
+// store the forward's columns, from which grad_weight is a second plain product
+// (bwd_wgrad_kernel).
 // Both operands of the product are pixel-major / K-contiguous copies written by
 // small pre-passes (relayout_kernel<E, false> for grad_output,
 // pack_weight_t_kernel for the weights).
@@ -222,14 +224,22 @@ __device__ __forceinline__ void VecCh<f16_t>::unpack(float (&out)[kScChunk]) con
   }
 }
 
+// Output-pixel tile of the scatter kernel: 8 rows x 32 columns, one thread per
+// pixel (rows of 32 keep the loads of d and the stores of the columns in 64-byte
+// or longer runs, and the window around it stays under 48 KiB for a margin of 3).
+constexpr int kScTH = 8;
+constexpr int kScTW = 32;
+
 struct BwdScatterArgs {
   Geom g;
   const void *xt;  // zero-bordered pixel-major input copy [N][Cin / KC][H + 2][W + 2][KC]
   OffMaskView om;
-  const void *D;   // column gradient of the pass, layout of ColGradArgs::D
+  const void *D;   // column gradient of the pass, layout of ColGradArgs::D; null: columns only
   float *gin32;
   void *goff;
   void *gmask;     // null when unmodulated
+  void *col;       // columns of the pass [image][group][tap][channel of the group][P_pad], or null
+  long P_pad;      // row pitch of col in elements
   int tiles_x, tiles_y;
   int WH, WW;      // window size in input pixels
   int R;           // margin of the window around the tile's undeformed footprint
@@ -239,11 +249,14 @@ struct BwdScatterArgs {
 // The window is kept in double precision: LDS double-precision atomic adds run
 // several times faster than single-precision ones on this hardware (measured:
 // 26 against 170 clocks per wavefront instruction per CU), so the window holds
-// kScChunk channels of 8 bytes where the fp32 design held 16 of 4.
+// kScChunk channels of 8 bytes where an fp32 window would hold 16 of 4.
+// With a.col the kernel also stores the forward's columns (mask * bilinear
+// sample, rounded to E as the reference's columns tensor is) for the
+// weight-gradient product; with a.D == null that is all it does.
 template <typename E>
 __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
   constexpr int KC = 128 / (int)sizeof(E);
-  static_assert(kScChunk * 8 == kBwdChunk * 4, "same window size in pixels as the fp32 window");
+  static_assert(kScTH * kScTW == 256, "one thread per pixel of the tile");
   __shared__ double win[kBwdWindowBytes / 8];
   const Geom &g = a.g;
   const long plane_out = (long)g.Ho * g.Wo;
@@ -258,11 +271,12 @@ __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
   const int dgi = b % g.DG;
   const int nl = b / g.DG;
   const int n = a.n0 + nl;
-  const int ho = ty * kBwdTile + (tid >> 4), wo = tx * kBwdTile + (tid & 15);
+  const int ho = ty * kScTH + tid / kScTW, wo = tx * kScTW + tid % kScTW;
   const bool valid = ho < g.Ho && wo < g.Wo;
   const long pix = valid ? (long)ho * g.Wo + wo : 0;
-  const int wy0 = ty * kBwdTile * g.sh - g.ph - a.R, wx0 = tx * kBwdTile * g.sw - g.pw - a.R;
+  const int wy0 = ty * kScTH * g.sh - g.ph - a.R, wx0 = tx * kScTW * g.sw - g.pw - a.R;
   const int win_px = a.WH * a.WW;
+  const bool data = a.D != nullptr;  // workgroup uniform
 
   const E *off = (const E *)a.om.off + (long)n * a.om.off_n + pix * a.om.off_px +
                  (long)(dgi * 2 * g.taps) * a.om.off_ch;
@@ -275,12 +289,17 @@ __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
 
   const int c_begin = dgi * g.ch_per_dg, c_end = c_begin + g.ch_per_dg;
   for (int c0 = c_begin; c0 < c_end; c0 += kScChunk) {
-    __syncthreads();  // the previous chunk's flush is done
-    for (int i = tid; i < win_px * kScChunk; i += 256) win[i] = 0.0;
-    __syncthreads();
+    if (data) {
+      __syncthreads();  // the previous chunk's flush is done
+      for (int i = tid; i < win_px * kScChunk; i += 256) win[i] = 0.0;
+      __syncthreads();
+    }
     const E *dbase = (const E *)a.D + (((long)nl * (g.Cin / 16) + (c0 >> 4)) * g.taps) * plane_out * 16 + pix * 16 +
                      (c0 & 15);
     const E *xbase = (const E *)a.xt + (((long)n * (g.Cin / KC) + c0 / KC) * slab_px) * KC + (c0 % KC);
+    // row of the columns matrix of channel c0 at tap 0 (a chunk stays inside one group)
+    const int grp = c0 / g.cin_g;
+    E *cbase = (E *)a.col + (((long)nl * g.Cin + (long)grp * g.cin_g) * g.taps + (c0 - grp * g.cin_g)) * a.P_pad + pix;
 #pragma unroll
     for (int tap = 0; tap < kBwdTapsMax; ++tap) {
       if (tap < g.taps) {
@@ -292,6 +311,7 @@ __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
         const float px = (float)(wo * g.sw - g.pw + tj * g.dw) + dx;
         const bool inside =
             valid && (py > -1.0f) && (px > -1.0f) && (py < (float)g.H) && (px < (float)g.W);
+        E *crow = cbase + (long)tap * g.cin_g * a.P_pad;
         if (inside) {
           const float fy = floorf(py), fx = floorf(px);
           const int y0 = (int)fy, x0 = (int)fx, y1 = y0 + 1, x1 = x0 + 1;
@@ -300,62 +320,77 @@ __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
           const bool ok10 = y1 <= g.H - 1 && x0 >= 0, ok11 = y1 <= g.H - 1 && x1 <= g.W - 1;
           // corners outside the image read the copy's zero border
           const E *xp = xbase + ((long)(y0 + 1) * g.Wp + (x0 + 1)) * KC;
-          VecCh<E> rd, r00, r01, r10, r11;
-          rd.load(dbase + (long)tap * plane_out * 16);
+          VecCh<E> r00, r01, r10, r11;
           r00.load(xp);
           r01.load(xp + KC);
           r10.load(xp + (long)g.Wp * KC);
           r11.load(xp + (long)(g.Wp + 1) * KC);
-          float d[kScChunk], v00[kScChunk], v01[kScChunk], v10[kScChunk], v11[kScChunk];
-          rd.unpack(d);
+          float v00[kScChunk], v01[kScChunk], v10[kScChunk], v11[kScChunk];
           r00.unpack(v00);
           r01.unpack(v01);
           r10.unpack(v10);
           r11.unpack(v11);
-          const int ry = y0 - wy0, rx = x0 - wx0;
-          const bool in_win = ry >= 0 && ry + 1 < a.WH && rx >= 0 && rx + 1 < a.WW;
-          const int wbase = ry * a.WW + rx;  // window is [channel][WH][WW]: neighbouring pixels, neighbouring banks
-          const long o00 = (long)y0 * g.W + x0, o01 = o00 + 1, o10 = o00 + g.W, o11 = o10 + 1;
           const float w00 = hy * hx, w01 = hy * lx, w10 = ly * hx, w11 = ly * lx;
-          float am = 0.0f, ay = 0.0f, ax = 0.0f;
+          if (a.col) {
 #pragma unroll
-          for (int cc = 0; cc < kScChunk; ++cc) {
-            const float dc = d[cc];
-            am += dc * (w00 * v00[cc] + w01 * v01[cc] + w10 * v10[cc] + w11 * v11[cc]);
-            ay += dc * (hx * (v10[cc] - v00[cc]) + lx * (v11[cc] - v01[cc]));
-            ax += dc * (hy * (v01[cc] - v00[cc]) + ly * (v11[cc] - v10[cc]));
-            const float t = dc * m;
-            if (in_win) {
-              double *wp = win + cc * win_px + wbase;
-              if (ok00) atomicAdd(wp, (double)(w00 * t));
-              if (ok01) atomicAdd(wp + 1, (double)(w01 * t));
-              if (ok10) atomicAdd(wp + a.WW, (double)(w10 * t));
-              if (ok11) atomicAdd(wp + a.WW + 1, (double)(w11 * t));
-            } else {
-              float *gi = a.gin32 + ((long)n * g.Cin + c0 + cc) * plane_in;
-              if (ok00) unsafeAtomicAdd(gi + o00, w00 * t);
-              if (ok01) unsafeAtomicAdd(gi + o01, w01 * t);
-              if (ok10) unsafeAtomicAdd(gi + o10, w10 * t);
-              if (ok11) unsafeAtomicAdd(gi + o11, w11 * t);
-            }
+            for (int cc = 0; cc < kScChunk; ++cc)
+              crow[(long)cc * a.P_pad] =
+                  from_f32<E>(m * (w00 * v00[cc] + w01 * v01[cc] + w10 * v10[cc] + w11 * v11[cc]));
           }
-          acc_m[tap] += am;
-          acc_y[tap] += ay * m;
-          acc_x[tap] += ax * m;
+          if (data) {
+            VecCh<E> rd;
+            rd.load(dbase + (long)tap * plane_out * 16);
+            float d[kScChunk];
+            rd.unpack(d);
+            const int ry = y0 - wy0, rx = x0 - wx0;
+            const bool in_win = ry >= 0 && ry + 1 < a.WH && rx >= 0 && rx + 1 < a.WW;
+            const int wbase = ry * a.WW + rx;  // window is [channel][WH][WW]: neighbouring pixels, neighbouring banks
+            const long o00 = (long)y0 * g.W + x0, o01 = o00 + 1, o10 = o00 + g.W, o11 = o10 + 1;
+            float am = 0.0f, ay = 0.0f, ax = 0.0f;
+#pragma unroll
+            for (int cc = 0; cc < kScChunk; ++cc) {
+              const float dc = d[cc];
+              am += dc * (w00 * v00[cc] + w01 * v01[cc] + w10 * v10[cc] + w11 * v11[cc]);
+              ay += dc * (hx * (v10[cc] - v00[cc]) + lx * (v11[cc] - v01[cc]));
+              ax += dc * (hy * (v01[cc] - v00[cc]) + ly * (v11[cc] - v10[cc]));
+              const float t = dc * m;
+              if (in_win) {
+                double *wp = win + cc * win_px + wbase;
+                if (ok00) atomicAdd(wp, (double)(w00 * t));
+                if (ok01) atomicAdd(wp + 1, (double)(w01 * t));
+                if (ok10) atomicAdd(wp + a.WW, (double)(w10 * t));
+                if (ok11) atomicAdd(wp + a.WW + 1, (double)(w11 * t));
+              } else {
+                float *gi = a.gin32 + ((long)n * g.Cin + c0 + cc) * plane_in;
+                if (ok00) unsafeAtomicAdd(gi + o00, w00 * t);
+                if (ok01) unsafeAtomicAdd(gi + o01, w01 * t);
+                if (ok10) unsafeAtomicAdd(gi + o10, w10 * t);
+                if (ok11) unsafeAtomicAdd(gi + o11, w11 * t);
+              }
+            }
+            acc_m[tap] += am;
+            acc_y[tap] += ay * m;
+            acc_x[tap] += ax * m;
+          }
+        } else if (valid && a.col) {  // a position outside the sampling range: a column of zeros
+#pragma unroll
+          for (int cc = 0; cc < kScChunk; ++cc) crow[(long)cc * a.P_pad] = from_f32<E>(0.0f);
         }
       }
     }
-    __syncthreads();  // every add into the window has landed
-    for (int i = tid; i < win_px * kScChunk; i += 256) {
-      const float v = (float)win[i];
-      if (v != 0.0f) {
-        const int cc = i / win_px, q = i - cc * win_px;
-        const int y = wy0 + q / a.WW, x = wx0 + q % a.WW;  // in the image: only valid corners were added
-        unsafeAtomicAdd(a.gin32 + ((long)n * g.Cin + c0 + cc) * plane_in + (long)y * g.W + x, v);
+    if (data) {
+      __syncthreads();  // every add into the window has landed
+      for (int i = tid; i < win_px * kScChunk; i += 256) {
+        const float v = (float)win[i];
+        if (v != 0.0f) {
+          const int cc = i / win_px, q = i - cc * win_px;
+          const int y = wy0 + q / a.WW, x = wx0 + q % a.WW;  // in the image: only valid corners were added
+          unsafeAtomicAdd(a.gin32 + ((long)n * g.Cin + c0 + cc) * plane_in + (long)y * g.W + x, v);
+        }
       }
     }
   }
-  if (valid) {
+  if (valid && data) {
     E *goff = (E *)a.goff, *gmask = (E *)a.gmask;
     const long ob = ((long)n * g.DG + dgi) * 2 * g.taps;
 #pragma unroll
@@ -367,6 +402,153 @@ __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
       }
     }
   }
+}
+
+// Zeroes the padding columns [P, P_pad) of every row of the columns matrix.
+template <typename E>
+__global__ __launch_bounds__(256) void zero_col_pad_kernel(E *col, long rows, int P, long P_pad) {
+  const int padn = (int)(P_pad - P);
+  const long total = rows * padn;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+    const long r = i / padn;
+    col[r * P_pad + P + (i - r * padn)] = from_f32<E>(0.0f);
+  }
+}
+
+struct WGradArgs {
+  const void *gout;  // [N][Cout][P]
+  const void *col;   // [images of the pass][G][taps][cin_g][P_pad]
+  float *gw32;       // (Cout, cin_g, kh, kw) fp32, zero before the first pass
+  int P;
+  long P_pad;
+  int ksteps;        // P_pad / (pixels per 128 bytes)
+  int nb, n0;        // images of the pass, first image
+  int M;             // taps * cin_g
+  int cin_g, cout_g, taps, G, Cin, Cout;
+  int co_tiles, m_tiles;
+  int splits;        // workgroups sharing the (image, K step) range of one tile
+};
+
+// grad_weight[co, (c, tap)] += sum over the pass's images and pixels of
+// grad_output[co, pixel] * col[(tap, c), pixel]: a plain product with the pixels
+// as reduction dimension (the reference's second GEMM,
+// mmcv/ops/csrc/pytorch/modulated_deform_conv.cpp:227-237).  Workgroup = 128
+// output channels x 128 column rows of one group over a share of the (image,
+// 128-byte pixel run) steps; both operand tiles go to LDS with direct copies as
+// in bwd_colgrad_kernel (grad_output is read in place: its rows are pixel
+// contiguous).  Runs of pixels past the end of an image read the row's last
+// 16 bytes again; the zero padding of col cancels them.  Rows past the group's
+// channels repeat its last row and are dropped at the end.  Partial sums leave
+// through fp32 atomics.
+template <typename E>
+__global__ __launch_bounds__(256, 2) void bwd_wgrad_kernel(WGradArgs a) {
+  using TR = ElemTraits<E>;
+  constexpr int ES = (int)sizeof(E);
+  constexpr int PXC = 16 / ES;  // pixels per 16-byte chunk
+  __shared__ uint4 As[2][kCgTile * 8];
+  __shared__ uint4 Bs[2][kCgTile * 8];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int frow = lane & 31, fhalf = lane >> 5;
+  const int wm = wave & 1, wn = wave >> 1;
+  int b = blockIdx.x;
+  const int mt = b % a.m_tiles;
+  b /= a.m_tiles;
+  const int ct = b % a.co_tiles;
+  const int grp = b / a.co_tiles;
+  const int split = blockIdx.y;
+
+  // this lane's rows and 16-byte chunk of the copies
+  long a_row[4], b_row[4];
+  int chunk[4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const int row = (wave * 4 + c) * 8 + (lane >> 3);
+    chunk[c] = (lane & 7) ^ (row & 7);
+    const int co = min(ct * kCgTile + row, a.cout_g - 1);
+    const int m = min(mt * kCgTile + row, a.M - 1);
+    a_row[c] = ((long)grp * a.cout_g + co) * a.P;            // + n * Cout * P
+    b_row[c] = ((long)grp * a.M + m) * a.P_pad;              // + nl * taps * Cin * P_pad
+  }
+  const uint32_t lds_a = (uint32_t)(uintptr_t)(lptr_t)(&As[0][0]) +
+                         (uint32_t)__builtin_amdgcn_readfirstlane(wave) * 4096u;
+  const uint32_t lds_b = (uint32_t)(uintptr_t)(lptr_t)(&Bs[0][0]) +
+                         (uint32_t)__builtin_amdgcn_readfirstlane(wave) * 4096u;
+  const E *gout = (const E *)a.gout, *col = (const E *)a.col;
+  const int last_chunk_px = a.P - PXC;  // (P is a multiple of PXC)
+  auto issue = [&](long wi, int buf) {
+    const int nl = (int)(wi / a.ksteps);
+    const int p0 = (int)(wi - (long)nl * a.ksteps) * (8 * PXC);
+    const E *ga = gout + (long)(a.n0 + nl) * a.Cout * a.P;
+    const E *cb = col + (long)nl * a.taps * a.Cin * a.P_pad;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int px = p0 + chunk[c] * PXC;
+      copy16_global_to_lds(ga + a_row[c] + min(px, last_chunk_px), lds_a + (uint32_t)buf * 16384u + (uint32_t)c * 1024u);
+      copy16_global_to_lds(cb + b_row[c] + px, lds_b + (uint32_t)buf * 16384u + (uint32_t)c * 1024u);
+    }
+  };
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  // this workgroup's contiguous share of the (image, K step) range
+  const long work = (long)a.nb * a.ksteps;
+  const long per = (work + a.splits - 1) / a.splits;
+  const long w_begin = (long)split * per, w_end = min(work, w_begin + per);
+  if (w_begin < w_end) {
+    issue(w_begin, 0);
+    int buf = 0;
+    for (long wi = w_begin; wi < w_end; ++wi, buf ^= 1) {
+      if (wi + 1 < w_end) {
+        issue(wi + 1, buf ^ 1);
+        asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+      } else {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      }
+      __syncthreads();
+#pragma unroll
+      for (int ksub = 0; ksub < 4; ++ksub) {
+        uint4 af[2], bf[2];
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb) {
+          const int row = wm * 64 + mb * 32 + frow;
+          af[mb] = As[buf][row * 8 + ((ksub * 2 + fhalf) ^ (row & 7))];
+        }
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) {
+          const int row = wn * 64 + nb * 32 + frow;
+          bf[nb] = Bs[buf][row * 8 + ((ksub * 2 + fhalf) ^ (row & 7))];
+        }
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+          for (int nb = 0; nb < 2; ++nb) TR::mma(acc[mb][nb], af[mb], bf[nb]);
+      }
+      __syncthreads();
+    }
+  }
+
+  // register r of lane l: A row (output channel) (r/4)*8 + (l/32)*4 + r%4 of the block, B row (column row) l%32
+  const int k_g = a.cin_g * a.taps;
+#pragma unroll
+  for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) {
+      const int m = mt * kCgTile + wn * 64 + nb * 32 + frow;
+      if (m >= a.M) continue;
+      const int tap = m / a.cin_g, cl = m - tap * a.cin_g;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int co = ct * kCgTile + wm * 64 + mb * 32 + (r >> 2) * 8 + fhalf * 4 + (r & 3);
+        if (co < a.cout_g)
+          unsafeAtomicAdd(a.gw32 + ((long)grp * a.cout_g + co) * k_g + (long)cl * a.taps + tap, acc[mb][nb][r]);
+      }
+    }
 }
 
 }  // namespace mdcn

@@ -214,7 +214,7 @@ def capi_pack_forward(case, own_conv=True, raw=None, want_raw=False, path=capi.P
     return out, raw_out
 
 
-def capi_backward(case, grad_output, want_bias=True, path=0):
+def capi_backward(case, grad_output, want_bias=True, path=0, want_data=True, want_weight=True):
     """mdcn_backward through ctypes on device tensors of `case` (mask None:
     unmodulated); returns (grad_input, grad_offset, grad_mask or None, grad_weight,
     grad_bias or None)."""
@@ -230,13 +230,17 @@ def capi_backward(case, grad_output, want_bias=True, path=0):
     keep = [t.contiguous() for t in (x, off, w, grad_output)]
     p.input, p.offset, p.weight, bp.grad_output = (t.data_ptr() for t in keep)
     g_in, g_off, g_w = torch.full_like(x, 7.0), torch.full_like(off, 7.0), torch.full_like(w, 7.0)
-    bp.grad_input, bp.grad_offset, bp.grad_weight = g_in.data_ptr(), g_off.data_ptr(), g_w.data_ptr()
+    if want_data:
+        bp.grad_input, bp.grad_offset = g_in.data_ptr(), g_off.data_ptr()
+    if want_weight:
+        bp.grad_weight = g_w.data_ptr()
     g_mask = g_b = None
     if msk is not None:
         keep.append(msk.contiguous())
         p.mask = keep[-1].data_ptr()
         g_mask = torch.full_like(msk, 7.0)
-        bp.grad_mask = g_mask.data_ptr()
+        if want_data:
+            bp.grad_mask = g_mask.data_ptr()
     if want_bias:
         g_b = torch.full((Cout,), 7.0, dtype=x.dtype, device=x.device)
         bp.grad_bias = g_b.data_ptr()

@@ -148,6 +148,24 @@ def test_tiled_backward_against_oracle(name, kw, dtype, modulated):
         assert err <= TOL[dtype] and err_d <= TOL[dtype], (nm, err, err_d)
 
 
+@pytest.mark.parametrize('dtype', DTYPES, ids=['f32', 'bf16', 'f16'])
+def test_tiled_backward_partial_requests(dtype):
+    """Only the data gradients, or only grad_weight (the two calls of the unmodulated
+    layer's backward): the same values as the full call, the rest untouched."""
+    case = cast_case(make_case(77, N=2, Cin=64, Cout=128, H=14, W=24, deform_groups=2, sigma=2.0), dtype, 'cuda')
+    gy = torch.randn(2, 128, 14, 24, generator=torch.Generator().manual_seed(3)).to(dtype).cuda()
+    full = capi_backward(case, gy, path=capi.PATH_FUSED)
+    data = capi_backward(case, gy, path=capi.PATH_FUSED, want_weight=False, want_bias=False)
+    wonly = capi_backward(case, gy, path=capi.PATH_FUSED, want_data=False)
+    tol = 1e-5 if dtype == torch.float32 else 4e-3  # (atomics: the order of the sums varies; one 16-bit ulp)
+    for i in range(3):
+        assert rel_err(_np(data[i]), _np(full[i])) <= tol
+        assert torch.all(wonly[i] == 7.0)
+    assert torch.all(data[3] == 7.0)
+    assert rel_err(_np(wonly[3]), _np(full[3])) <= tol
+    assert torch.equal(wonly[4], full[4])
+
+
 def test_full_size_layer_gradients_spot_check():
     """cfg-4-like layer at reduced batch (bf16, 256 channels, 100x152): first image
     of the batch against the oracle."""
