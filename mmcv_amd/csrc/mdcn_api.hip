@@ -481,9 +481,11 @@ struct BwdPlan {
   int n_chunk;     // images per pass
   int M_pad;       // rows of the transposed weight matrix per group
   long P_pad;      // row pitch of the columns matrix
-  size_t xt_bytes, gt_bytes, wt_bytes, d_bytes, col_bytes;
+  int parts;       // workgroups of the scatter kernel per tile (shares of the channels)
+  size_t xt_bytes, gt_bytes, wt_bytes, d_bytes, col_bytes, part_bytes;
+  size_t gb_bytes;  // fp32 sum of grad_bias (16-bit tensors)
   size_t total() const {
-    return gin_bytes + gw_bytes + xt_bytes + gt_bytes + wt_bytes + d_bytes + col_bytes;
+    return gin_bytes + gw_bytes + gb_bytes + xt_bytes + gt_bytes + wt_bytes + d_bytes + col_bytes + part_bytes;
   }
 };
 
@@ -492,8 +494,10 @@ void make_bwd_plan(const mdcn_bwd_params *bp, const Geom &g, BwdPlan *pl) {
   const size_t es = elem_size(bp->conv.dtype);
   pl->gin_bytes = (staged && bp->grad_input) ? align_up((size_t)g.N * g.Cin * g.H * g.W * 4) : 0;
   pl->gw_bytes = (staged && bp->grad_weight) ? align_up((size_t)g.Cout * g.cin_g * g.taps * 4) : 0;
+  pl->gb_bytes = (staged && bp->grad_bias) ? align_up((size_t)g.Cout * 4) : 0;
   pl->tiled = pl->gemm = pl->wgemm = false;
-  pl->xt_bytes = pl->gt_bytes = pl->wt_bytes = pl->d_bytes = pl->col_bytes = 0;
+  pl->xt_bytes = pl->gt_bytes = pl->wt_bytes = pl->d_bytes = pl->col_bytes = pl->part_bytes = 0;
+  pl->parts = 1;
   pl->n_chunk = g.N;
   pl->M_pad = 0;
   pl->P_pad = 0;
@@ -526,6 +530,10 @@ void make_bwd_plan(const mdcn_bwd_params *bp, const Geom &g, BwdPlan *pl) {
     pl->gt_bytes = align_up((size_t)g.N * (g.Cout / KC) * plane_out * 128);
     pl->wt_bytes = align_up((size_t)g.G * pl->M_pad * g.cout_g * es);
     pl->d_bytes = align_up(d_img * pl->n_chunk);
+    // enough workgroups for eight rounds or so of the chip's 2 x CUs slots
+    while (pl->parts < 8 && s_tiles * pl->parts < 4096 && g.ch_per_dg % (2 * pl->parts * kScChunk) == 0)
+      pl->parts *= 2;
+    if (pl->parts > 1) pl->part_bytes = align_up((size_t)pl->parts * g.N * g.DG * 3 * g.taps * plane_out * 4);
   }
   if (pl->wgemm) {
     const long kpx = 128 / (long)es;  // pixels per K step
@@ -555,11 +563,15 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
   const long n_w = (long)g.Cout * g.cin_g * g.taps;
   float *gin32 = pl.gin_bytes ? (float *)ws : (float *)bp->grad_input;
   float *gw32 = pl.gw_bytes ? (float *)(ws + pl.gin_bytes) : (float *)bp->grad_weight;
-  unsigned char *xt = ws + pl.gin_bytes + pl.gw_bytes;
+  float *gb32 = pl.gb_bytes ? (float *)(ws + pl.gin_bytes + pl.gw_bytes) : (float *)bp->grad_bias;
+  unsigned char *xt = ws + pl.gin_bytes + pl.gw_bytes + pl.gb_bytes;
   unsigned char *gT = xt + pl.xt_bytes;
   unsigned char *wT = gT + pl.gt_bytes;
   unsigned char *D = wT + pl.wt_bytes;
   unsigned char *col = D + pl.d_bytes;
+  const long off_total = (long)g.N * g.DG * 2 * g.taps * plane_out, mask_total = off_total / 2;
+  float *poff = (float *)(col + pl.col_bytes);
+  float *pmask = poff + (long)pl.parts * off_total;
   // the weight-gradient product copies grad_output rows 16 bytes at a time
   const bool wgemm = pl.wgemm && ((uintptr_t)bp->grad_output % 16) == 0;
   const bool gemm = pl.gemm;
@@ -642,8 +654,13 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
       sa.WH = pl.sWH;
       sa.WW = pl.sWW;
       sa.n0 = n0;
+      sa.parts = gemm ? pl.parts : 1;
+      sa.poff = poff;
+      sa.pmask = pmask;
+      sa.off_total = off_total;
+      sa.mask_total = mask_total;
       const long sblocks = (long)nb * g.DG * sa.tiles_y * sa.tiles_x;
-      hipLaunchKernelGGL(bwd_scatter_kernel<E>, dim3((unsigned)sblocks), dim3(256), 0, st, sa);
+      hipLaunchKernelGGL(bwd_scatter_kernel<E>, dim3((unsigned)sblocks, (unsigned)sa.parts), dim3(256), 0, st, sa);
       check();
       if (wgemm) {
         WGradArgs wa;
@@ -675,7 +692,16 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
 
   if (bp->grad_input) {
     if (gemm) {
-      // done above
+      if (pl.parts > 1) {
+        hipLaunchKernelGGL(combine_parts_kernel<E>, dim3(blocks_for(off_total)), dim3(256), 0, st, poff,
+                           (E *)bp->grad_offset, off_total, pl.parts);
+        check();
+        if (bp->grad_mask) {
+          hipLaunchKernelGGL(combine_parts_kernel<E>, dim3(blocks_for(mask_total)), dim3(256), 0, st, pmask,
+                             (E *)bp->grad_mask, mask_total, pl.parts);
+          check();
+        }
+      }
     } else if (pl.tiled) {
       BwdDataTiledArgs da;
       da.g = g;
@@ -734,9 +760,18 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
     }
   }
   if (bp->grad_bias) {
-    hipLaunchKernelGGL(bwd_bias_kernel<E>, dim3(g.Cout), dim3(256), 0, st, g,
-                       (const E *)bp->grad_output, (E *)bp->grad_bias);
+    hipLaunchKernelGGL(fill_zero_kernel<float>, dim3(blocks_for(g.Cout)), dim3(256), 0, st, gb32, (long)g.Cout);
     check();
+    const int runs = (int)((plane_out + kBiasRun - 1) / kBiasRun);
+    const int splits = (int)std::min<long>((long)g.N * runs, 64);
+    hipLaunchKernelGGL(bwd_bias_kernel<E>, dim3(g.Cout, splits), dim3(256), 0, st, g,
+                       (const E *)bp->grad_output, gb32, runs, splits);
+    check();
+    if (pl.gb_bytes) {
+      hipLaunchKernelGGL(round_kernel<E>, dim3(blocks_for(g.Cout)), dim3(256), 0, st, gb32,
+                         (E *)bp->grad_bias, (long)g.Cout);
+      check();
+    }
   }
   return rc;
 }

@@ -36,17 +36,27 @@ __global__ __launch_bounds__(256) void round_kernel(const float *__restrict__ sr
     dst[i] = from_f32<E>(src[i]);
 }
 
-// grad_bias[co] = sum over images and pixels of grad_output[:, co] (one block per channel).
+// Pixels of one image a block of bwd_bias_kernel sums.
+constexpr int kBiasRun = 8192;
+
+// grad_bias[co] = sum over images and pixels of grad_output[:, co]: block (co, s)
+// sums every `splits`-th run of kBiasRun pixels of channel co and adds its share
+// to the fp32 sum with one atomic.
 template <typename E>
 __global__ __launch_bounds__(256) void bwd_bias_kernel(Geom g, const E *__restrict__ gout,
-                                                       E *__restrict__ gbias) {
+                                                       float *__restrict__ gbias32, int runs_per_image,
+                                                       int splits) {
   __shared__ float part[256];
   const int co = blockIdx.x;
   const long plane = (long)g.Ho * g.Wo;
+  const long work = (long)g.N * runs_per_image;
   float s = 0.0f;
-  for (int n = 0; n < g.N; ++n) {
+  for (long wi = blockIdx.y; wi < work; wi += splits) {
+    const int n = (int)(wi / runs_per_image);
+    const long p0 = (wi - (long)n * runs_per_image) * kBiasRun;
+    const long p1 = min(plane, p0 + kBiasRun);
     const E *row = gout + ((long)n * g.Cout + co) * plane;
-    for (long p = threadIdx.x; p < plane; p += 256) s += to_f32(row[p]);
+    for (long p = p0 + threadIdx.x; p < p1; p += 256) s += to_f32(row[p]);
   }
   part[threadIdx.x] = s;
   __syncthreads();
@@ -54,7 +64,7 @@ __global__ __launch_bounds__(256) void bwd_bias_kernel(Geom g, const E *__restri
     if ((int)threadIdx.x < w) part[threadIdx.x] += part[threadIdx.x + w];
     __syncthreads();
   }
-  if (threadIdx.x == 0) gbias[co] = from_f32<E>(part[0]);
+  if (threadIdx.x == 0) unsafeAtomicAdd(gbias32 + co, part[0]);
 }
 
 // Channels whose column gradient a thread of bwd_data_kernel holds at a time.

@@ -244,7 +244,26 @@ struct BwdScatterArgs {
   int WH, WW;      // window size in input pixels
   int R;           // margin of the window around the tile's undeformed footprint
   int n0;          // first image of the pass
+  // A deformable group's channels are shared among `parts` workgroups per tile
+  // (blockIdx.y), so that the launch has several times more workgroups than the
+  // chip has room for and its last round is short; with parts > 1 each writes its
+  // share of the offset / mask sums as floats to poff / pmask ([part][layout of
+  // grad_offset / grad_mask]), which combine_parts_kernel adds up.
+  int parts;
+  float *poff, *pmask;
+  long off_total, mask_total;  // elements of grad_offset / grad_mask
 };
+
+// out[i] = sum over parts of part[p][i], rounded once.
+template <typename E>
+__global__ __launch_bounds__(256) void combine_parts_kernel(const float *__restrict__ part, E *__restrict__ out,
+                                                            long total, int parts) {
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+    float s = 0.0f;
+    for (int p = 0; p < parts; ++p) s += part[(long)p * total + i];
+    out[i] = from_f32<E>(s);
+  }
+}
 
 // The window is kept in double precision: LDS double-precision atomic adds run
 // several times faster than single-precision ones on this hardware (measured:
@@ -287,7 +306,9 @@ __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
 #pragma unroll
   for (int t = 0; t < kBwdTapsMax; ++t) acc_m[t] = acc_y[t] = acc_x[t] = 0.0f;
 
-  const int c_begin = dgi * g.ch_per_dg, c_end = c_begin + g.ch_per_dg;
+  const int part = blockIdx.y;
+  const int ch_per_part = g.ch_per_dg / a.parts;
+  const int c_begin = dgi * g.ch_per_dg + part * ch_per_part, c_end = c_begin + ch_per_part;
   for (int c0 = c_begin; c0 < c_end; c0 += kScChunk) {
     if (data) {
       __syncthreads();  // the previous chunk's flush is done
@@ -391,14 +412,28 @@ __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
     }
   }
   if (valid && data) {
-    E *goff = (E *)a.goff, *gmask = (E *)a.gmask;
     const long ob = ((long)n * g.DG + dgi) * 2 * g.taps;
+    const long mb = ((long)n * g.DG + dgi) * g.taps;
+    if (a.parts == 1) {
+      E *goff = (E *)a.goff, *gmask = (E *)a.gmask;
 #pragma unroll
-    for (int tap = 0; tap < kBwdTapsMax; ++tap) {
-      if (tap < g.taps) {
-        goff[(ob + 2 * tap) * plane_out + pix] = from_f32<E>(acc_y[tap]);
-        goff[(ob + 2 * tap + 1) * plane_out + pix] = from_f32<E>(acc_x[tap]);
-        if (gmask) gmask[(((long)n * g.DG + dgi) * g.taps + tap) * plane_out + pix] = from_f32<E>(acc_m[tap]);
+      for (int tap = 0; tap < kBwdTapsMax; ++tap) {
+        if (tap < g.taps) {
+          goff[(ob + 2 * tap) * plane_out + pix] = from_f32<E>(acc_y[tap]);
+          goff[(ob + 2 * tap + 1) * plane_out + pix] = from_f32<E>(acc_x[tap]);
+          if (gmask) gmask[(mb + tap) * plane_out + pix] = from_f32<E>(acc_m[tap]);
+        }
+      }
+    } else {
+      float *poff = a.poff + (long)part * a.off_total;
+      float *pmask = a.gmask ? a.pmask + (long)part * a.mask_total : nullptr;
+#pragma unroll
+      for (int tap = 0; tap < kBwdTapsMax; ++tap) {
+        if (tap < g.taps) {
+          poff[(ob + 2 * tap) * plane_out + pix] = acc_y[tap];
+          poff[(ob + 2 * tap + 1) * plane_out + pix] = acc_x[tap];
+          if (pmask) pmask[(mb + tap) * plane_out + pix] = acc_m[tap];
+        }
       }
     }
   }
