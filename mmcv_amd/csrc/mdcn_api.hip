@@ -478,6 +478,7 @@ struct BwdPlan {
   bool gemm;       // data gradients
   bool wgemm;      // grad_weight from stored columns
   int sR, sWH, sWW;  // window of the scatter kernel
+  int sCH;         // channels per pass over that window (kScChunk or kScChunkSmall)
   int n_chunk;     // images per pass
   int M_pad;       // rows of the transposed weight matrix per group
   long P_pad;      // row pitch of the columns matrix
@@ -511,7 +512,18 @@ void make_bwd_plan(const mdcn_bwd_params *bp, const Geom &g, BwdPlan *pl) {
   // matrix-core paths: channels in whole 128-byte slabs, 32-channel blocks per tap
   const int KC = (int)(128 / es);
   const size_t d_img = (size_t)g.taps * g.Cin * plane_out * es;
-  pl->sR = window_margin(g, kScTH, kScTW, kBwdWindowBytes / (8 * kScChunk), &pl->sWH, &pl->sWW);
+  pl->sCH = kScChunk;
+  pl->sR = window_margin(g, kScTH, kScTW, kScWindowBytes / (8 * kScChunk), &pl->sWH, &pl->sWW);
+  if (pl->sR < 2) {  // fewer channels at a time buy a wider window
+    int wh, ww;
+    const int r = window_margin(g, kScTH, kScTW, kScWindowBytes / (8 * kScChunkSmall), &wh, &ww);
+    if (r > pl->sR) {
+      pl->sCH = kScChunkSmall;
+      pl->sR = r;
+      pl->sWH = wh;
+      pl->sWW = ww;
+    }
+  }
   const long s_tiles = (long)g.N * g.DG * ((g.Ho + kScTH - 1) / kScTH) * ((g.Wo + kScTW - 1) / kScTW);
   const bool mfma_ok = g.Cin % KC == 0 && g.cout_g % KC == 0 && g.cin_g % 32 == 0 &&
                        g.ch_per_dg % kScChunk == 0 && pl->sR >= 1 && (s_tiles >= 512 || forced) &&
@@ -660,7 +672,10 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
       sa.off_total = off_total;
       sa.mask_total = mask_total;
       const long sblocks = (long)nb * g.DG * sa.tiles_y * sa.tiles_x;
-      hipLaunchKernelGGL(bwd_scatter_kernel<E>, dim3((unsigned)sblocks, (unsigned)sa.parts), dim3(256), 0, st, sa);
+      if (pl.sCH == kScChunk)
+        hipLaunchKernelGGL((bwd_scatter_kernel<E, kScChunk>), dim3((unsigned)sblocks, (unsigned)sa.parts), dim3(256), 0, st, sa);
+      else
+        hipLaunchKernelGGL((bwd_scatter_kernel<E, kScChunkSmall>), dim3((unsigned)sblocks, (unsigned)sa.parts), dim3(256), 0, st, sa);
       check();
       if (wgemm) {
         WGradArgs wa;

@@ -174,55 +174,45 @@ __global__ __launch_bounds__(256, 2) void bwd_colgrad_kernel(ColGradArgs a) {
   }
 }
 
-// Channels per pass of the scatter kernel over its LDS window.
+// Channels per pass of the scatter kernel over its LDS window: 8, or 4 for
+// geometries (stride 2, dilation) whose window would not fit otherwise.
 constexpr int kScChunk = 8;
+constexpr int kScChunkSmall = 4;
+// Bytes of the scatter kernel's window (two workgroups per CU).
+constexpr int kScWindowBytes = 60 * 1024;
 
-// kScChunk consecutive channels (16 or 32 bytes) as floats.
-template <typename E>
+// CH consecutive channels (8 to 32 bytes) as floats.
+template <typename E, int CH>
 struct VecCh {
-  static constexpr int NV = kScChunk * (int)sizeof(E) / 16;  // 16-byte loads
-  uint4 raw[NV];
+  static constexpr int NW = CH * (int)sizeof(E) / 4;  // 32-bit words
+  uint32_t raw[NW];
   __device__ __forceinline__ void load(const E *p) {
+    if constexpr (NW % 4 == 0) {
 #pragma unroll
-    for (int i = 0; i < NV; ++i) raw[i] = ((const uint4 *)p)[i];
+      for (int i = 0; i < NW / 4; ++i) {
+        const uint4 v = ((const uint4 *)p)[i];
+        raw[4 * i] = v.x;
+        raw[4 * i + 1] = v.y;
+        raw[4 * i + 2] = v.z;
+        raw[4 * i + 3] = v.w;
+      }
+    } else {
+      static_assert(NW == 2, "8 bytes");
+      const uint2 v = *(const uint2 *)p;
+      raw[0] = v.x;
+      raw[1] = v.y;
+    }
   }
-  __device__ __forceinline__ void unpack(float (&out)[kScChunk]) const;
+  __device__ __forceinline__ void unpack(float (&out)[CH]) const {
+    if constexpr (sizeof(E) == 4) {
+#pragma unroll
+      for (int i = 0; i < CH; ++i) out[i] = __uint_as_float(raw[i]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < NW; ++i) ElemTraits<E>::unpack2(raw[i], out[2 * i], out[2 * i + 1]);
+    }
+  }
 };
-template <>
-__device__ __forceinline__ void VecCh<float>::unpack(float (&out)[kScChunk]) const {
-#pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    out[4 * i] = __uint_as_float(raw[i].x);
-    out[4 * i + 1] = __uint_as_float(raw[i].y);
-    out[4 * i + 2] = __uint_as_float(raw[i].z);
-    out[4 * i + 3] = __uint_as_float(raw[i].w);
-  }
-}
-template <>
-__device__ __forceinline__ void VecCh<bf16_t>::unpack(float (&out)[kScChunk]) const {
-#pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    const uint32_t w[4] = {raw[i].x, raw[i].y, raw[i].z, raw[i].w};
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      out[8 * i + 2 * j] = __uint_as_float(w[j] << 16);
-      out[8 * i + 2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
-    }
-  }
-}
-template <>
-__device__ __forceinline__ void VecCh<f16_t>::unpack(float (&out)[kScChunk]) const {
-#pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    const uint32_t w[4] = {raw[i].x, raw[i].y, raw[i].z, raw[i].w};
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const f16x2 p = __builtin_bit_cast(f16x2, w[j]);
-      out[8 * i + 2 * j] = (float)p.x;
-      out[8 * i + 2 * j + 1] = (float)p.y;
-    }
-  }
-}
 
 // Output-pixel tile of the scatter kernel: 8 rows x 32 columns, one thread per
 // pixel (rows of 32 keep the loads of d and the stores of the columns in 64-byte
@@ -268,15 +258,15 @@ __global__ __launch_bounds__(256) void combine_parts_kernel(const float *__restr
 // The window is kept in double precision: LDS double-precision atomic adds run
 // several times faster than single-precision ones on this hardware (measured:
 // 26 against 170 clocks per wavefront instruction per CU), so the window holds
-// kScChunk channels of 8 bytes where an fp32 window would hold 16 of 4.
+// CH channels of 8 bytes where an fp32 window would hold twice as many of 4.
 // With a.col the kernel also stores the forward's columns (mask * bilinear
 // sample, rounded to E as the reference's columns tensor is) for the
 // weight-gradient product; with a.D == null that is all it does.
-template <typename E>
+template <typename E, int CH>
 __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
   constexpr int KC = 128 / (int)sizeof(E);
   static_assert(kScTH * kScTW == 256, "one thread per pixel of the tile");
-  __shared__ double win[kBwdWindowBytes / 8];
+  __shared__ double win[kScWindowBytes / 8];
   const Geom &g = a.g;
   const long plane_out = (long)g.Ho * g.Wo;
   const long plane_in = (long)g.H * g.W;
@@ -309,10 +299,10 @@ __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
   const int part = blockIdx.y;
   const int ch_per_part = g.ch_per_dg / a.parts;
   const int c_begin = dgi * g.ch_per_dg + part * ch_per_part, c_end = c_begin + ch_per_part;
-  for (int c0 = c_begin; c0 < c_end; c0 += kScChunk) {
+  for (int c0 = c_begin; c0 < c_end; c0 += CH) {
     if (data) {
       __syncthreads();  // the previous chunk's flush is done
-      for (int i = tid; i < win_px * kScChunk; i += 256) win[i] = 0.0;
+      for (int i = tid; i < win_px * CH; i += 256) win[i] = 0.0;
       __syncthreads();
     }
     const E *dbase = (const E *)a.D + (((long)nl * (g.Cin / 16) + (c0 >> 4)) * g.taps) * plane_out * 16 + pix * 16 +
@@ -341,12 +331,12 @@ __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
           const bool ok10 = y1 <= g.H - 1 && x0 >= 0, ok11 = y1 <= g.H - 1 && x1 <= g.W - 1;
           // corners outside the image read the copy's zero border
           const E *xp = xbase + ((long)(y0 + 1) * g.Wp + (x0 + 1)) * KC;
-          VecCh<E> r00, r01, r10, r11;
+          VecCh<E, CH> r00, r01, r10, r11;
           r00.load(xp);
           r01.load(xp + KC);
           r10.load(xp + (long)g.Wp * KC);
           r11.load(xp + (long)(g.Wp + 1) * KC);
-          float v00[kScChunk], v01[kScChunk], v10[kScChunk], v11[kScChunk];
+          float v00[CH], v01[CH], v10[CH], v11[CH];
           r00.unpack(v00);
           r01.unpack(v01);
           r10.unpack(v10);
@@ -354,14 +344,14 @@ __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
           const float w00 = hy * hx, w01 = hy * lx, w10 = ly * hx, w11 = ly * lx;
           if (a.col) {
 #pragma unroll
-            for (int cc = 0; cc < kScChunk; ++cc)
+            for (int cc = 0; cc < CH; ++cc)
               crow[(long)cc * a.P_pad] =
                   from_f32<E>(m * (w00 * v00[cc] + w01 * v01[cc] + w10 * v10[cc] + w11 * v11[cc]));
           }
           if (data) {
-            VecCh<E> rd;
+            VecCh<E, CH> rd;
             rd.load(dbase + (long)tap * plane_out * 16);
-            float d[kScChunk];
+            float d[CH];
             rd.unpack(d);
             const int ry = y0 - wy0, rx = x0 - wx0;
             const bool in_win = ry >= 0 && ry + 1 < a.WH && rx >= 0 && rx + 1 < a.WW;
@@ -369,7 +359,7 @@ __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
             const long o00 = (long)y0 * g.W + x0, o01 = o00 + 1, o10 = o00 + g.W, o11 = o10 + 1;
             float am = 0.0f, ay = 0.0f, ax = 0.0f;
 #pragma unroll
-            for (int cc = 0; cc < kScChunk; ++cc) {
+            for (int cc = 0; cc < CH; ++cc) {
               const float dc = d[cc];
               am += dc * (w00 * v00[cc] + w01 * v01[cc] + w10 * v10[cc] + w11 * v11[cc]);
               ay += dc * (hx * (v10[cc] - v00[cc]) + lx * (v11[cc] - v01[cc]));
@@ -395,13 +385,13 @@ __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
           }
         } else if (valid && a.col) {  // a position outside the sampling range: a column of zeros
 #pragma unroll
-          for (int cc = 0; cc < kScChunk; ++cc) crow[(long)cc * a.P_pad] = from_f32<E>(0.0f);
+          for (int cc = 0; cc < CH; ++cc) crow[(long)cc * a.P_pad] = from_f32<E>(0.0f);
         }
       }
     }
     if (data) {
       __syncthreads();  // every add into the window has landed
-      for (int i = tid; i < win_px * kScChunk; i += 256) {
+      for (int i = tid; i < win_px * CH; i += 256) {
         const float v = (float)win[i];
         if (v != 0.0f) {
           const int cc = i / win_px, q = i - cc * win_px;

@@ -131,6 +131,11 @@ struct ElemTraits<bf16_t> : Half16Traits<bf16_t> {
     p.y = (bf16_t)hi;
     return __builtin_bit_cast(uint32_t, p);
   }
+  // the two channels of a 32-bit word as floats
+  static __device__ __forceinline__ void unpack2(uint32_t w, float &lo, float &hi) {
+    lo = __uint_as_float(w << 16);
+    hi = __uint_as_float(w & 0xffff0000u);
+  }
   // (the builtin, not inline assembly: the compiler must see the DOT instruction
   // to insert the wait states its result needs before another VALU reads it)
   static __device__ __forceinline__ float dot2(uint32_t d, uint32_t w, float c) {
@@ -151,6 +156,11 @@ struct ElemTraits<f16_t> : Half16Traits<f16_t> {
     p.x = (f16_t)lo;
     p.y = (f16_t)hi;
     return __builtin_bit_cast(uint32_t, p);
+  }
+  static __device__ __forceinline__ void unpack2(uint32_t w, float &lo, float &hi) {
+    const f16x2 p = __builtin_bit_cast(f16x2, w);
+    lo = (float)p.x;
+    hi = (float)p.y;
   }
   static __device__ __forceinline__ float dot2(uint32_t d, uint32_t w, float c) {
     return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, d), __builtin_bit_cast(f16x2, w), c, false);

@@ -113,6 +113,8 @@ TILED_CASES = [
     ('c64', dict(N=2, Cin=64, Cout=64, H=20, W=19, sigma=2.0)),
     ('c128_g2_dg2', dict(N=1, Cin=128, Cout=128, H=18, W=21, groups=2, deform_groups=2, sigma=2.5)),
     ('c64_co192', dict(N=2, Cin=64, Cout=192, H=23, W=17, sigma=1.5)),
+    ('c64_co128_s2', dict(N=2, Cin=64, Cout=128, H=23, W=37, stride=2, sigma=1.5)),
+    ('c128_s2_dil2_dg2', dict(N=1, Cin=128, Cout=64, H=30, W=21, stride=2, padding=2, dilation=2, deform_groups=2, sigma=2.5)),
     ('c64_dil2_dg4', dict(N=1, Cin=64, Cout=64, H=17, W=17, padding=2, dilation=2, deform_groups=4, sigma=3.0)),
     ('c192_k1x3', dict(N=1, Cin=192, Cout=64, H=9, W=33, k=(1, 3), padding=(0, 1), sigma=1.0)),
     ('c96_f32_only', dict(N=1, Cin=96, Cout=32, H=16, W=16, sigma=6.0)),
