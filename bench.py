@@ -264,6 +264,25 @@ def main():
     cl_ms = e0.elapsed_time(e1) / a.steps
     log(f'channels-last input: step {cl_ms:.4f} ms')
 
+    # the layer's backward (all five gradients) through the same extension, for reference beside
+    # the headline forward figure; not part of `value`
+    gy = torch.randn(N, Cout, Ho, Wo, device='cuda').to(dtype)
+    g_in, g_w, g_b = torch.empty_like(x), torch.empty_like(w), torch.empty_like(b)
+    g_off, g_msk = torch.empty_like(off), torch.empty_like(msk)
+    step_bwd = lambda: ext_module.modulated_deform_conv_backward(
+        x, w, b, empty, off, msk, empty, g_in, g_w, g_b, g_off, g_msk, gy, **kwargs)
+    bsteps = max(3, a.steps // 5)
+    for _ in range(2):
+        step_bwd()
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(bsteps):
+        step_bwd()
+    e1.record()
+    torch.cuda.synchronize()
+    bwd_ms = e0.elapsed_time(e1) / bsteps
+    log(f'backward: step {bwd_ms:.4f} ms')
+
     value = flops / (ms_per_step * 1e-3) / 1e12
     achieved = flops / (main_ms * 1e-3) / 1e12
     peak = PEAK_TFLOPS[dname]
@@ -295,6 +314,9 @@ def main():
         'hbm_GBs_algorithmic': round(alg_bytes / (ms_per_step * 1e-3) / 1e9, 1),
         'channels_last_input': {'ms_per_step': round(cl_ms, 4),
                                 'TFLOPs': round(flops / (cl_ms * 1e-3) / 1e12, 2)},
+        'backward': {'ms_per_step': round(bwd_ms, 4), 'steps': bsteps,
+                     'TFLOPs': round(2.0 * flops / (bwd_ms * 1e-3) / 1e12, 2),
+                     'what': 'grad input/offset/mask/weight/bias; two products of the forward size'},
         'roofline': {
             'bound': 'mfma',
             'kernel': f'fused_kernel<{dname}>',

@@ -526,7 +526,7 @@ void make_bwd_plan(const mdcn_bwd_params *bp, const Geom &g, BwdPlan *pl) {
   }
   const long s_tiles = (long)g.N * g.DG * ((g.Ho + kScTH - 1) / kScTH) * ((g.Wo + kScTW - 1) / kScTW);
   const bool mfma_ok = g.Cin % KC == 0 && g.cout_g % KC == 0 && g.cin_g % 32 == 0 &&
-                       g.ch_per_dg % kScChunk == 0 && pl->sR >= 1 && (s_tiles >= 512 || forced) &&
+                       g.ch_per_dg % kScChunk == 0 && pl->sR >= 1 && (s_tiles >= 64 || forced) &&
                        d_img <= kBwdColGradCap && plane_out <= ((size_t)1 << 30);
   if (mfma_ok) {
     pl->gemm = bp->grad_input != nullptr;
