@@ -94,6 +94,17 @@ typedef struct mdcn_params {
 /* ABI version of the loaded library (== MDCN_ABI_VERSION it was built with). */
 int mdcn_abi_version(void);
 
+/* Large batches are processed in passes of whole images: the forward's input
+ * copy is addressed with 32-bit byte offsets (at most 0xF0000000 bytes per
+ * pass), the backward keeps at most 1.5 GiB of column gradient (and as much of
+ * columns) at a time.  This lowers the two limits for the whole process (0
+ * restores a default; values above the defaults are clipped): a knob for memory
+ * constrained callers and for tests of the pass loops.  Not thread safe against
+ * concurrent calls into the library; workspace sizes must be queried again
+ * after a change.  (No counterpart in the reference, whose im2col_step plays
+ * this role for DCNv1.) */
+void mdcn_set_pass_limits(uint64_t forward_bytes, uint64_t backward_bytes);
+
 /* Static text for a status code. */
 const char *mdcn_status_string(int status);
 

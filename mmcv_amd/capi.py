@@ -13,7 +13,7 @@ MDCN_F32, MDCN_F16, MDCN_BF16 = 0, 1, 2
 PATH_AUTO, PATH_FUSED, PATH_DIRECT = 0, 1, 2
 MDCN_OK = 0
 
-EXPORTS = ('mdcn_abi_version', 'mdcn_status_string', 'mdcn_output_size',
+EXPORTS = ('mdcn_abi_version', 'mdcn_set_pass_limits', 'mdcn_status_string', 'mdcn_output_size',
            'mdcn_fused_eligible', 'mdcn_workspace_bytes', 'mdcn_forward',
            'mdcn_forward_timed', 'mdcn_pack_workspace_bytes', 'mdcn_pack_forward',
            'mdcn_pack_forward_timed', 'mdcn_backward_workspace_bytes', 'mdcn_backward')
@@ -52,6 +52,8 @@ def load():
         P = ctypes.POINTER(MdcnParams)
         lib.mdcn_abi_version.restype = ctypes.c_int
         lib.mdcn_abi_version.argtypes = []
+        lib.mdcn_set_pass_limits.restype = None
+        lib.mdcn_set_pass_limits.argtypes = [ctypes.c_uint64, ctypes.c_uint64]
         lib.mdcn_status_string.restype = ctypes.c_char_p
         lib.mdcn_status_string.argtypes = [ctypes.c_int]
         lib.mdcn_output_size.restype = ctypes.c_int

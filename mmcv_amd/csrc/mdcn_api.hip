@@ -23,6 +23,11 @@ constexpr size_t kAlign = 256;
 constexpr size_t kMaxLds = 160 * 1024;
 // Device byte offsets into the channels-last copy are 32-bit.
 constexpr uint64_t kMaxXtBytes = 0xF0000000ull;
+// Column gradient (and columns) held in memory per pass of the backward's matrix-core paths.
+constexpr uint64_t kBwdColGradCap = (uint64_t)3 << 29;  // 1.5 GiB each
+// Per-pass limits in force (mdcn_set_pass_limits lowers them; process wide).
+uint64_t g_fwd_pass_bytes = kMaxXtBytes;
+uint64_t g_bwd_pass_bytes = kBwdColGradCap;
 
 inline size_t align_up(size_t v) { return (v + kAlign - 1) / kAlign * kAlign; }
 
@@ -132,7 +137,7 @@ int make_plan(const mdcn_params *p, const Geom &g, Plan *pl) {
   pl->n_ctiles = (g.cout_g + pl->CT - 1) / pl->CT;
   pl->slabs = g.cin_g / pl->KC;
   const uint64_t img = (uint64_t)g.Hp * g.Wp * g.Cin * es;
-  pl->n_chunk = (int)std::min<uint64_t>((uint64_t)g.N, std::max<uint64_t>(1, kMaxXtBytes / img));
+  pl->n_chunk = (int)std::min<uint64_t>((uint64_t)g.N, std::max<uint64_t>(1, g_fwd_pass_bytes / img));
   pl->xt_bytes = p->input_nhwc ? 0 : align_up((size_t)img * pl->n_chunk);
   pl->wp_bytes = align_up((size_t)g.G * pl->n_ctiles * pl->slabs * g.taps * pl->CT * pl->KC * es);
   return MDCN_OK;
@@ -453,9 +458,6 @@ int run(const mdcn_params *p, void *stream, float *ms, const mdcn_pack_params *p
   }
 }
 
-// Column gradient (and columns) held in memory per pass of the matrix-core paths.
-constexpr size_t kBwdColGradCap = (size_t)3 << 29;  // 1.5 GiB each
-
 // Largest margin R (up to 8) for which the LDS window of a th x tw output-pixel
 // tile fits max_px pixels; -1 if even R = 0 does not.
 int window_margin(const Geom &g, int th, int tw, long max_px, int *WH, int *WW) {
@@ -534,7 +536,7 @@ void make_bwd_plan(const mdcn_bwd_params *bp, const Geom &g, BwdPlan *pl) {
     pl->wgemm = bp->grad_weight != nullptr && plane_out % (16 / es) == 0;
   }
   if (pl->gemm || pl->wgemm) {
-    pl->n_chunk = (int)std::min<size_t>((size_t)g.N, kBwdColGradCap / d_img);
+    pl->n_chunk = (int)std::min<uint64_t>((uint64_t)g.N, std::max<uint64_t>(1, g_bwd_pass_bytes / d_img));
     pl->xt_bytes = align_up((size_t)g.N * (g.Cin / KC) * g.Hp * g.Wp * 128);
   }
   if (pl->gemm) {
@@ -817,6 +819,11 @@ int check_bwd(const mdcn_bwd_params *bp, Geom *g, bool need_ptrs) {
 extern "C" {
 
 int mdcn_abi_version(void) { return MDCN_ABI_VERSION; }
+
+void mdcn_set_pass_limits(uint64_t forward_bytes, uint64_t backward_bytes) {
+  g_fwd_pass_bytes = forward_bytes ? std::min<uint64_t>(forward_bytes, kMaxXtBytes) : kMaxXtBytes;
+  g_bwd_pass_bytes = backward_bytes ? std::min<uint64_t>(backward_bytes, kBwdColGradCap) : kBwdColGradCap;
+}
 
 const char *mdcn_status_string(int status) {
   switch (status) {
