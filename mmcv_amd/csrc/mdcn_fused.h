@@ -19,17 +19,20 @@
 //     bilinear weights (positions and weights in fp32).  Per K step, each lane
 //     gathers for two pixels 2 x 16 bytes of channels at each of the four corners
 //     (16 x global_load_dwordx4, issued kGatherAhead steps ahead, held in
-//     registers), blends them (v_dot2 on the raw bf16 pairs, mixed-precision FMA
-//     for fp16, FMA for fp32) and writes 4 x 16 bytes of the sample tile.  They
-//     also start the direct-to-LDS copy of the weight tile kWeightAhead steps
-//     ahead.
+//     registers), blends them (16-bit types: horizontal corners paired with
+//     v_perm_b32, one v_dot2 per two products; fp32: FMA) and writes 4 x 16
+//     bytes of the sample tile.
 //   waves 0..3  CONSUMERS.  2 x 2 over the tile (64 pixels x CT/2 channels
 //     each): read sample and weight fragments from LDS, run MFMA
 //     (32x32x16 bf16/f16, 32x32x2 fp32) into fp32 accumulators; at the end of
 //     the tile add the bias, round once, transpose through LDS and store
-//     16 bytes per lane along W of the NCHW output.
+//     16 bytes per lane along W of the NCHW output.  They also issue the
+//     direct-to-LDS copy of the weight tile kWeightAhead steps ahead.
 // One workgroup barrier per K step keeps the two roles in step; the sample
 // tile is double buffered, the weight tiles sit in a ring of kWeightSlots.
+// Where the epilogue's staging fits one ring slot (16-bit types, CT = 256) the
+// producers start the next tile (table, gathers, first sample tile) while the
+// consumers store the current one.
 //
 // LDS tiles have 128-byte rows (one pixel resp. one output channel, KC elements
 // of K); the 16-byte chunks of a row are permuted (swz) so that both the
@@ -315,6 +318,11 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
   constexpr int WDMA = CT / 32;      // 1 KiB direct-to-LDS copies per consumer wave and K step
   constexpr int TPT = (TMAX + kTapGroups - 1) / kTapGroups;  // table entries per producer lane
   static_assert(kWeightAhead * WDMA < 64, "vmcnt holds 6 bits");
+  // Epilogue overlap: when the consumers' four staging areas fit the ring slot
+  // that no copy targets before the first K step of a tile, the epilogue leaves
+  // the sample tiles alone, and the producers build the next tile's table and
+  // first samples while the consumers store the current one.
+  constexpr bool OVL = 4 * 32 * stage_row_bytes<E>() <= CT * kRowB && kWeightAhead + 1 < kWeightSlots;
 
   __shared__ uint4 Xs[2][PT * kRowChunks];                // sample tiles
   __shared__ uint4 Ws[kWeightSlots][CT * kRowChunks];     // weight tiles
@@ -343,8 +351,9 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
   const int wgs_per_xcd = (int)(gridDim.x >> 3);
   const int chunk = (total_tiles + 7) >> 3;
   const int tile_end = min((xcd + 1) * chunk, total_tiles);
+  bool first_tile = true;
 
-  for (int tile = xcd * chunk + wg_in_xcd; tile < tile_end; tile += wgs_per_xcd) {
+  for (int tile = xcd * chunk + wg_in_xcd; tile < tile_end; tile += wgs_per_xcd, first_tile = false) {
     int L = tile;
     const int ctile = L % a.n_ctiles;
     L /= a.n_ctiles;
@@ -522,8 +531,8 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
       // know that a wave keeps its role) and would otherwise guard the consumers'
       // registers with vmcnt waits that also wait for their in-flight weight copies.
       __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), other counters untouched
-      MDCN_BARRIER_LDS();   // E0: the tiles become the consumers' staging area
-      MDCN_BARRIER_LDS();   // E1: epilogue done, tiles and table may be rewritten
+      MDCN_BARRIER_LDS();   // E0: the K loop is over for everybody
+      if (!OVL) MDCN_BARRIER_LDS();   // E1: epilogue done, tiles and table may be rewritten
     } else {
       // =================== CONSUMER ===================
       const int wave_p = wave & 1;   // which 64 pixels
@@ -586,7 +595,7 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
       // vmcnt waits below also cover them)
 #pragma unroll
       for (int j = 0; j <= kWeightAhead; ++j) issue_weights(j);
-      MDCN_BARRIER_LDS();  // B0
+      if (!OVL || first_tile) MDCN_BARRIER_LDS();  // B0 (with OVL: passed before the previous tile's epilogue)
 #pragma unroll
       for (int v = 0; v <= kGatherAhead; ++v) mirror_issue();
       MDCN_BARRIER(kWeightAhead * WDMA);  // B1: W[0] landed
@@ -617,6 +626,9 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
         MDCN_BARRIER(kWeightAhead * WDMA);  // end of step ks: W[ks+1] landed
       }
       MDCN_BARRIER(0);  // E0: copies issued past the end have landed; tiles become staging
+      // B0 of the next tile, taken early: the producers need nothing from the
+      // consumers for its table, gathers and first sample tile
+      if (OVL && tile + wgs_per_xcd < tile_end) MDCN_BARRIER_LDS();
 
       // ---- epilogue: bias, round once, transpose through LDS, NCHW store ----
       // Accumulator block (A = samples, B = weights): register r of lane l holds
@@ -624,8 +636,9 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
       constexpr int RB = stage_row_bytes<E>();
       constexpr int CHUNK_PX = 16 / ES;           // pixels per 16-byte chunk
       constexpr int CHUNKS = 64 / CHUNK_PX;       // chunks per staged row
-      unsigned char *stage = (wave < 2 ? (unsigned char *)&Xs[0][0] : (unsigned char *)&Ws[0][0]) +
-                             (size_t)(wave & 1) * 32 * RB;
+      unsigned char *stage =
+          OVL ? (unsigned char *)&Ws[kWeightSlots - 1][0] + (size_t)wave * 32 * RB
+              : (wave < 2 ? (unsigned char *)&Xs[0][0] : (unsigned char *)&Ws[0][0]) + (size_t)(wave & 1) * 32 * RB;
       E *out = (E *)a.out;
       const int pw0 = p0 + wave_p * 64;           // first pixel of this wave
       const bool vec_ok = a.out_vec_ok != 0;      // 16-byte chunks never straddle images, aligned
@@ -674,7 +687,7 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       }
-      MDCN_BARRIER_LDS();  // E1
+      if (!OVL) MDCN_BARRIER_LDS();  // E1
     }
   }
 }
