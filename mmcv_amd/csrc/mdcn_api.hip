@@ -6,6 +6,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <type_traits>
 
 #include "mdcn_common.h"
 #include "mdcn_direct.h"
@@ -480,15 +481,16 @@ struct BwdPlan {
   bool gemm;       // data gradients
   bool wgemm;      // grad_weight from stored columns
   int sR, sWH, sWW;  // window of the scatter kernel
-  int sCH;         // channels per pass over that window (kScChunk or kScChunkSmall)
+  int sCH;         // channels per pass over that window
   int n_chunk;     // images per pass
   int M_pad;       // rows of the transposed weight matrix per group
   long P_pad;      // row pitch of the columns matrix
   int parts;       // workgroups of the scatter kernel per tile (shares of the channels)
   size_t xt_bytes, gt_bytes, wt_bytes, d_bytes, col_bytes, part_bytes;
   size_t gb_bytes;  // fp32 sum of grad_bias (16-bit tensors)
+  size_t mx_bytes;  // the two maxima that scale the fixed-point window (16-bit tensors)
   size_t total() const {
-    return gin_bytes + gw_bytes + gb_bytes + xt_bytes + gt_bytes + wt_bytes + d_bytes + col_bytes + part_bytes;
+    return gin_bytes + gw_bytes + gb_bytes + mx_bytes + xt_bytes + gt_bytes + wt_bytes + d_bytes + col_bytes + part_bytes;
   }
 };
 
@@ -498,6 +500,7 @@ void make_bwd_plan(const mdcn_bwd_params *bp, const Geom &g, BwdPlan *pl) {
   pl->gin_bytes = (staged && bp->grad_input) ? align_up((size_t)g.N * g.Cin * g.H * g.W * 4) : 0;
   pl->gw_bytes = (staged && bp->grad_weight) ? align_up((size_t)g.Cout * g.cin_g * g.taps * 4) : 0;
   pl->gb_bytes = (staged && bp->grad_bias) ? align_up((size_t)g.Cout * 4) : 0;
+  pl->mx_bytes = 0;
   pl->tiled = pl->gemm = pl->wgemm = false;
   pl->xt_bytes = pl->gt_bytes = pl->wt_bytes = pl->d_bytes = pl->col_bytes = pl->part_bytes = 0;
   pl->parts = 1;
@@ -514,13 +517,15 @@ void make_bwd_plan(const mdcn_bwd_params *bp, const Geom &g, BwdPlan *pl) {
   // matrix-core paths: channels in whole 128-byte slabs, 32-channel blocks per tap
   const int KC = (int)(128 / es);
   const size_t d_img = (size_t)g.taps * g.Cin * plane_out * es;
-  pl->sCH = kScChunk;
-  pl->sR = window_margin(g, kScTH, kScTW, kScWindowBytes / (8 * kScChunk), &pl->sWH, &pl->sWW);
-  if (pl->sR < 2) {  // fewer channels at a time buy a wider window
+  // channels per pass: 16 / 8 of 32-bit fixed point (16-bit tensors), 8 / 4 doubles (fp32)
+  const int ch_big = es == 2 ? 16 : 8;
+  pl->sCH = ch_big;
+  pl->sR = window_margin(g, kScTH, kScTW, kScWindowPx, &pl->sWH, &pl->sWW);
+  if (pl->sR < 2 || g.ch_per_dg % ch_big) {  // fewer channels at a time buy a wider window
     int wh, ww;
-    const int r = window_margin(g, kScTH, kScTW, kScWindowBytes / (8 * kScChunkSmall), &wh, &ww);
-    if (r > pl->sR) {
-      pl->sCH = kScChunkSmall;
+    const int r = window_margin(g, kScTH, kScTW, 2 * kScWindowPx, &wh, &ww);
+    if (r > pl->sR || g.ch_per_dg % ch_big) {
+      pl->sCH = ch_big / 2;
       pl->sR = r;
       pl->sWH = wh;
       pl->sWW = ww;
@@ -528,7 +533,7 @@ void make_bwd_plan(const mdcn_bwd_params *bp, const Geom &g, BwdPlan *pl) {
   }
   const long s_tiles = (long)g.N * g.DG * ((g.Ho + kScTH - 1) / kScTH) * ((g.Wo + kScTW - 1) / kScTW);
   const bool mfma_ok = g.Cin % KC == 0 && g.cout_g % KC == 0 && g.cin_g % 32 == 0 &&
-                       g.ch_per_dg % kScChunk == 0 && pl->sR >= 1 && (s_tiles >= 64 || forced) &&
+                       g.ch_per_dg % pl->sCH == 0 && pl->sR >= 1 && (s_tiles >= 64 || forced) &&
                        d_img <= kBwdColGradCap && plane_out <= ((size_t)1 << 30);
   if (mfma_ok) {
     pl->gemm = bp->grad_input != nullptr;
@@ -545,8 +550,9 @@ void make_bwd_plan(const mdcn_bwd_params *bp, const Geom &g, BwdPlan *pl) {
     pl->wt_bytes = align_up((size_t)g.G * pl->M_pad * g.cout_g * es);
     pl->d_bytes = align_up(d_img * pl->n_chunk);
     // enough workgroups for eight rounds or so of the chip's 2 x CUs slots
-    while (pl->parts < 8 && s_tiles * pl->parts < 4096 && g.ch_per_dg % (2 * pl->parts * kScChunk) == 0)
+    while (pl->parts < 8 && s_tiles * pl->parts < 4096 && g.ch_per_dg % (2 * pl->parts * pl->sCH) == 0)
       pl->parts *= 2;
+    if (staged) pl->mx_bytes = kAlign;
     if (pl->parts > 1) pl->part_bytes = align_up((size_t)pl->parts * g.N * g.DG * 3 * g.taps * plane_out * 4);
   }
   if (pl->wgemm) {
@@ -578,7 +584,8 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
   float *gin32 = pl.gin_bytes ? (float *)ws : (float *)bp->grad_input;
   float *gw32 = pl.gw_bytes ? (float *)(ws + pl.gin_bytes) : (float *)bp->grad_weight;
   float *gb32 = pl.gb_bytes ? (float *)(ws + pl.gin_bytes + pl.gw_bytes) : (float *)bp->grad_bias;
-  unsigned char *xt = ws + pl.gin_bytes + pl.gw_bytes + pl.gb_bytes;
+  uint32_t *maxima = (uint32_t *)(ws + pl.gin_bytes + pl.gw_bytes + pl.gb_bytes);  // [0] |d|, [1] |mask|
+  unsigned char *xt = ws + pl.gin_bytes + pl.gw_bytes + pl.gb_bytes + pl.mx_bytes;
   unsigned char *gT = xt + pl.xt_bytes;
   unsigned char *wT = gT + pl.gt_bytes;
   unsigned char *D = wT + pl.wt_bytes;
@@ -617,6 +624,16 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
       hipLaunchKernelGGL((relayout_kernel<E, false>), dim3((unsigned)((long)g.N * (g.Cout / KC) * o_pchunks)),
                          dim3(256), 0, st, gg, (const E *)bp->grad_output, (E *)gT, o_pchunks, o_words_ok);
       check();
+      if (pl.mx_bytes) {
+        hipLaunchKernelGGL(fill_zero_kernel<uint32_t>, dim3(1), dim3(256), 0, st, maxima, 2L);
+        check();
+        if (p->mask) {
+          const long n_mask = (long)g.N * g.DG * g.taps * plane_out;
+          hipLaunchKernelGGL(absmax_kernel<E>, dim3(std::min(blocks_for(n_mask / 8), 1024)), dim3(256), 0, st,
+                             (const E *)p->mask, n_mask, maxima + 1);
+          check();
+        }
+      }
       const long wtotal = (long)g.G * pl.M_pad * g.cout_g;
       hipLaunchKernelGGL(pack_weight_t_kernel<E>, dim3(blocks_for(wtotal)), dim3(256), 0, st, g,
                          (const E *)p->weight, (E *)wT, pl.M_pad, wtotal);
@@ -648,6 +665,7 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
         ca.Cout = g.Cout;
         ca.kslabs = g.cout_g / KC;
         ca.n0 = n0;
+        ca.dmax = pl.mx_bytes ? maxima : nullptr;
         const long cblocks = (long)nb * g.G * ca.px_tiles * ca.m_tiles;
         hipLaunchKernelGGL(bwd_colgrad_kernel<E>, dim3((unsigned)cblocks), dim3(256), 0, st, ca);
         check();
@@ -673,11 +691,21 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
       sa.pmask = pmask;
       sa.off_total = off_total;
       sa.mask_total = mask_total;
+      sa.dmax = maxima;
+      sa.mmax = p->mask ? maxima + 1 : nullptr;
       const long sblocks = (long)nb * g.DG * sa.tiles_y * sa.tiles_x;
-      if (pl.sCH == kScChunk)
-        hipLaunchKernelGGL((bwd_scatter_kernel<E, kScChunk>), dim3((unsigned)sblocks, (unsigned)sa.parts), dim3(256), 0, st, sa);
-      else
-        hipLaunchKernelGGL((bwd_scatter_kernel<E, kScChunkSmall>), dim3((unsigned)sblocks, (unsigned)sa.parts), dim3(256), 0, st, sa);
+      {
+        // 16-bit tensors: 32-bit fixed-point window (needs the maxima the data path computes;
+        // a columns-only call adds nothing to the window); fp32 tensors: doubles
+        constexpr bool k16 = sizeof(E) == 2;
+        using WT = typename std::conditional<k16, int32_t, double>::type;
+        constexpr int CHB = k16 ? 16 : 8;
+        const dim3 sgrid((unsigned)sblocks, (unsigned)sa.parts);
+        if (pl.sCH == CHB)
+          hipLaunchKernelGGL((bwd_scatter_kernel<E, CHB, WT>), sgrid, dim3(256), 0, st, sa);
+        else
+          hipLaunchKernelGGL((bwd_scatter_kernel<E, CHB / 2, WT>), sgrid, dim3(256), 0, st, sa);
+      }
       check();
       if (wgemm) {
         WGradArgs wa;

@@ -56,6 +56,7 @@ struct ColGradArgs {
   int cin_g, cout_g, taps, G, Cin, Cout;
   int kslabs;      // cout_g / KC
   int n0;          // first image of the pass
+  uint32_t *dmax;  // bit pattern of the largest |d| stored so far (a float >= 0), or null
 };
 
 // Workgroup = 128 rows of wT (one group) x 128 pixels of one image, reduction
@@ -153,6 +154,20 @@ __global__ __launch_bounds__(256, 2) void bwd_colgrad_kernel(ColGradArgs a) {
   // register r of lane l: A row (r/4)*8 + (l/32)*4 + r%4 of the block, B row l%32
   E *D = (E *)a.D;
   const int chunks = a.Cin / 16;
+  if (a.dmax) {  // (every accumulator counts: rows and pixels past the end repeat real ones or are zero)
+    float mx = 0.0f;
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, fabsf(acc[mb][nb][r]));
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    // (non-negative floats order like their bits; the plain read first keeps all but the few
+    // waves that raise the maximum from queueing on one address)
+    if (lane == 0 && __float_as_uint(mx) > __builtin_nontemporal_load(a.dmax)) atomicMax(a.dmax, __float_as_uint(mx));
+  }
 #pragma unroll
   for (int mb = 0; mb < 2; ++mb) {
     const int m0 = mt * kCgTile + wm * 64 + mb * 32;  // a block = one tap, 32 consecutive channels
@@ -174,12 +189,27 @@ __global__ __launch_bounds__(256, 2) void bwd_colgrad_kernel(ColGradArgs a) {
   }
 }
 
-// Channels per pass of the scatter kernel over its LDS window: 8, or 4 for
-// geometries (stride 2, dilation) whose window would not fit otherwise.
-constexpr int kScChunk = 8;
-constexpr int kScChunkSmall = 4;
-// Bytes of the scatter kernel's window (two workgroups per CU).
+// Bytes of the scatter kernel's window (two workgroups per CU).  It holds CH
+// channels of a WH x WW pixel neighbourhood of the tile; kScWindowPx pixels fit
+// with the larger channel count of a type (16-bit tensors: 16 channels of 32-bit
+// fixed point; fp32 tensors: 8 channels of doubles), twice as many -- stride 2,
+// dilation -- with the smaller one.
 constexpr int kScWindowBytes = 60 * 1024;
+constexpr int kScWindowPx = kScWindowBytes / 64;
+// Contributions one window entry can receive at most: every (pixel, tap) of the
+// tile touches an entry at most once per channel.
+constexpr int kScMaxAdds = 256 * 9;
+
+// largest |x| of a tensor, as the bit pattern of a non-negative float
+template <typename E>
+__global__ __launch_bounds__(256) void absmax_kernel(const E *__restrict__ x, long n, uint32_t *out) {
+  float mx = 0.0f;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
+    mx = fmaxf(mx, fabsf(to_f32(x[i])));
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+  if ((threadIdx.x & 63) == 0 && __float_as_uint(mx) > __builtin_nontemporal_load(out)) atomicMax(out, __float_as_uint(mx));
+}
 
 // CH consecutive channels (8 to 32 bytes) as floats.
 template <typename E, int CH>
@@ -242,6 +272,8 @@ struct BwdScatterArgs {
   int parts;
   float *poff, *pmask;
   long off_total, mask_total;  // elements of grad_offset / grad_mask
+  // fixed-point window (16-bit tensors): largest |d| and largest |mask| (null: 1)
+  const uint32_t *dmax, *mmax;
 };
 
 // out[i] = sum over parts of part[p][i], rounded once.
@@ -255,18 +287,34 @@ __global__ __launch_bounds__(256) void combine_parts_kernel(const float *__restr
   }
 }
 
-// The window is kept in double precision: LDS double-precision atomic adds run
-// several times faster than single-precision ones on this hardware (measured:
-// 26 against 170 clocks per wavefront instruction per CU), so the window holds
-// CH channels of 8 bytes where an fp32 window would hold twice as many of 4.
+// The window is not fp32: LDS single-precision atomic adds are slow on this
+// hardware (measured per wavefront instruction per CU: ds_add_f32 170 clocks,
+// ds_add_f64 26, ds_add_u32 11, whatever the addresses).  fp32 tensors use a
+// double-precision window (WT = double).  16-bit tensors use 32-bit fixed point
+// (WT = int32_t): with B = max|d| * max|mask| bounding every contribution and at
+// most kScMaxAdds contributions per entry, the scale 2^k <= 2^30 / (B * kScMaxAdds)
+// cannot overflow, and one contribution is rounded to B * 2^-19 at worst -- two
+// thousand times finer than the bf16/fp16 rounding of the result.  Integer sums
+// are exact, so the window part of grad_input does not depend on the order of
+// the adds.
 // With a.col the kernel also stores the forward's columns (mask * bilinear
 // sample, rounded to E as the reference's columns tensor is) for the
 // weight-gradient product; with a.D == null that is all it does.
-template <typename E, int CH>
+template <typename E, int CH, typename WT>
 __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
   constexpr int KC = 128 / (int)sizeof(E);
+  constexpr bool kFixed = sizeof(WT) == 4;
   static_assert(kScTH * kScTW == 256, "one thread per pixel of the tile");
-  __shared__ double win[kScWindowBytes / 8];
+  static_assert(kScTH * kScTW * kBwdTapsMax <= kScMaxAdds, "bound on the adds per window entry");
+  __shared__ WT win[kScWindowBytes / sizeof(WT)];
+  float fx_scale = 1.0f, fx_inv = 1.0f;
+  if (kFixed && a.D != nullptr) {
+    const float bound = __uint_as_float(*a.dmax) * (a.mmax ? __uint_as_float(*a.mmax) : 1.0f) * (float)kScMaxAdds;
+    // largest power of two not above 2^30 / bound (any scale will do when everything is zero)
+    const int e = (bound > 0.0f && bound < 3.0e38f) ? 29 - ilogbf(bound) : 0;
+    fx_scale = ldexpf(1.0f, max(-120, min(120, e)));
+    fx_inv = 1.0f / fx_scale;
+  }
   const Geom &g = a.g;
   const long plane_out = (long)g.Ho * g.Wo;
   const long plane_in = (long)g.H * g.W;
@@ -302,7 +350,7 @@ __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
   for (int c0 = c_begin; c0 < c_end; c0 += CH) {
     if (data) {
       __syncthreads();  // the previous chunk's flush is done
-      for (int i = tid; i < win_px * CH; i += 256) win[i] = 0.0;
+      for (int i = tid; i < win_px * CH; i += 256) win[i] = (WT)0;
       __syncthreads();
     }
     const E *dbase = (const E *)a.D + (((long)nl * (g.Cin / 16) + (c0 >> 4)) * g.taps) * plane_out * 16 + pix * 16 +
@@ -366,11 +414,19 @@ __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
               ax += dc * (hy * (v01[cc] - v00[cc]) + ly * (v11[cc] - v10[cc]));
               const float t = dc * m;
               if (in_win) {
-                double *wp = win + cc * win_px + wbase;
-                if (ok00) atomicAdd(wp, (double)(w00 * t));
-                if (ok01) atomicAdd(wp + 1, (double)(w01 * t));
-                if (ok10) atomicAdd(wp + a.WW, (double)(w10 * t));
-                if (ok11) atomicAdd(wp + a.WW + 1, (double)(w11 * t));
+                WT *wp = win + cc * win_px + wbase;
+                if constexpr (kFixed) {
+                  const float ts = t * fx_scale;
+                  if (ok00) atomicAdd(wp, __float2int_rn(w00 * ts));
+                  if (ok01) atomicAdd(wp + 1, __float2int_rn(w01 * ts));
+                  if (ok10) atomicAdd(wp + a.WW, __float2int_rn(w10 * ts));
+                  if (ok11) atomicAdd(wp + a.WW + 1, __float2int_rn(w11 * ts));
+                } else {
+                  if (ok00) atomicAdd(wp, (WT)(w00 * t));
+                  if (ok01) atomicAdd(wp + 1, (WT)(w01 * t));
+                  if (ok10) atomicAdd(wp + a.WW, (WT)(w10 * t));
+                  if (ok11) atomicAdd(wp + a.WW + 1, (WT)(w11 * t));
+                }
               } else {
                 float *gi = a.gin32 + ((long)n * g.Cin + c0 + cc) * plane_in;
                 if (ok00) unsafeAtomicAdd(gi + o00, w00 * t);
@@ -392,7 +448,7 @@ __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
     if (data) {
       __syncthreads();  // every add into the window has landed
       for (int i = tid; i < win_px * CH; i += 256) {
-        const float v = (float)win[i];
+        const float v = kFixed ? (float)win[i] * fx_inv : (float)win[i];
         if (v != 0.0f) {
           const int cc = i / win_px, q = i - cc * win_px;
           const int y = wy0 + q / a.WW, x = wx0 + q % a.WW;  // in the image: only valid corners were added
