@@ -156,8 +156,8 @@ def run_cfg5(a):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
-    ap.add_argument('--steps', type=int, default=50)
-    ap.add_argument('--warmup', type=int, default=10)
+    ap.add_argument('--steps', type=int, default=200)
+    ap.add_argument('--warmup', type=int, default=20)
     ap.add_argument('--workload', default='cfg4', choices=sorted(WORKLOADS) + ['cfg5'])
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     ap.add_argument('--copy-probe', action='store_true',
@@ -264,6 +264,52 @@ def main():
     cl_ms = e0.elapsed_time(e1) / a.steps
     log(f'channels-last input: step {cl_ms:.4f} ms')
 
+    # per-call distribution (one event pair per call), rotating buffers (four sets of input /
+    # offset / mask / output, 1.05 GB: no call finds its operands in the 256 MB last-level cache)
+    # and the bare C-ABI call (workspace allocated once, ctypes) beside the headline figure
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(a.steps)]
+    for s0, s1 in evs:
+        s0.record()
+        step()
+        s1.record()
+    torch.cuda.synchronize()
+    per_call = sorted(s0.elapsed_time(s1) for s0, s1 in evs)
+    sets = [(x, off, msk, out)] + [(torch.randn_like(x), off.clone(), msk.clone(), torch.empty_like(out))
+                                   for _ in range(3)]
+    step_rot = lambda i: ext_module.modulated_deform_conv_forward(
+        sets[i % 4][0], w, b, empty, sets[i % 4][1], sets[i % 4][2], sets[i % 4][3], empty, **kwargs)
+    for i in range(4):
+        step_rot(i)
+    torch.cuda.synchronize()
+    e0.record()
+    for i in range(a.steps):
+        step_rot(i)
+    e1.record()
+    torch.cuda.synchronize()
+    rot_ms = e0.elapsed_time(e1) / a.steps
+    del sets
+    import ctypes
+    from mmcv_amd import capi
+    lib = capi.load()
+    cp = capi.make_params({'f32': 0, 'f16': 1, 'bf16': 2}[dname], N, Cin, H, W, Cout, kh, kw, (sh, sw), (ph, pw),
+                          (dh, dw), case['groups'], case['deform_groups'])
+    cp.input, cp.offset, cp.mask, cp.weight, cp.bias, cp.output = (t.data_ptr() for t in (x, off, msk, w, b, out))
+    cws = torch.empty(lib.mdcn_workspace_bytes(ctypes.byref(cp)), dtype=torch.uint8, device='cuda')
+    cp.workspace, cp.workspace_bytes = cws.data_ptr(), cws.numel()
+    cstream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for _ in range(3):
+        assert lib.mdcn_forward(ctypes.byref(cp), cstream) == 0
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(a.steps):
+        lib.mdcn_forward(ctypes.byref(cp), cstream)
+    e1.record()
+    torch.cuda.synchronize()
+    cabi_ms = e0.elapsed_time(e1) / a.steps
+    del cws
+    log(f'per call: median {per_call[len(per_call) // 2]:.4f} min {per_call[0]:.4f} ms; rotating buffers '
+        f'{rot_ms:.4f} ms; bare C ABI {cabi_ms:.4f} ms')
+
     # the layer's backward (all five gradients) through the same extension, for reference beside
     # the headline forward figure; not part of `value`
     gy = torch.randn(N, Cout, Ho, Wo, device='cuda').to(dtype)
@@ -314,6 +360,9 @@ def main():
         'hbm_GBs_algorithmic': round(alg_bytes / (ms_per_step * 1e-3) / 1e9, 1),
         'channels_last_input': {'ms_per_step': round(cl_ms, 4),
                                 'TFLOPs': round(flops / (cl_ms * 1e-3) / 1e12, 2)},
+        'per_call_ms': {'median': round(per_call[len(per_call) // 2], 4), 'min': round(per_call[0], 4)},
+        'rotating_buffers': {'sets': 4, 'ms_per_step': round(rot_ms, 4)},
+        'c_abi_call': {'entry': 'mdcn_forward', 'ms_per_step': round(cabi_ms, 4)},
         'backward': {'ms_per_step': round(bwd_ms, 4), 'steps': bsteps,
                      'TFLOPs': round(2.0 * flops / (bwd_ms * 1e-3) / 1e12, 2),
                      'what': 'grad input/offset/mask/weight/bias; two products of the forward size'},
