@@ -666,8 +666,8 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
         ca.kslabs = g.cout_g / KC;
         ca.n0 = n0;
         ca.dmax = pl.mx_bytes ? maxima : nullptr;
-        const long cblocks = (long)nb * g.G * ca.px_tiles * ca.m_tiles;
-        hipLaunchKernelGGL(bwd_colgrad_kernel<E>, dim3((unsigned)cblocks), dim3(256), 0, st, ca);
+        ca.total = (long)nb * g.G * ca.px_tiles * ca.m_tiles;
+        hipLaunchKernelGGL(bwd_colgrad_kernel<E>, dim3((unsigned)((ca.total + 7) / 8 * 8)), dim3(256), 0, st, ca);
         check();
       }
       BwdScatterArgs sa;
@@ -729,7 +729,8 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
         const long tiles = (long)g.G * wa.co_tiles * wa.m_tiles;
         const long work = (long)nb * wa.ksteps;
         wa.splits = (int)std::max<long>(1, std::min<long>(std::min<long>(work, 65535), (4L * num_cus() + tiles - 1) / tiles));
-        hipLaunchKernelGGL(bwd_wgrad_kernel<E>, dim3((unsigned)tiles, (unsigned)wa.splits), dim3(256), 0, st, wa);
+        wa.total = tiles * wa.splits;
+        hipLaunchKernelGGL(bwd_wgrad_kernel<E>, dim3((unsigned)((wa.total + 7) / 8 * 8)), dim3(256), 0, st, wa);
         check();
       }
     }

@@ -25,6 +25,19 @@ namespace mdcn {
 // Rows of either operand per workgroup tile of the column-gradient product.
 constexpr int kCgTile = 128;
 
+// Work index of a workgroup of a 1-D launch of 8 * ceil(total / 8) workgroups, or
+// -1 for the few that have none.  Consecutive workgroup ids sit on different
+// XCDs (each with its own L2); this hands every XCD one contiguous run of work
+// indices, so that neighbours in the work order -- made to share an operand tile
+// -- run on the same XCD at about the same time and fetch that tile from HBM
+// once instead of once per XCD.
+__device__ __forceinline__ long xcd_work_index(long total) {
+  const long chunk = (total + 7) >> 3;
+  const long xcd = blockIdx.x & 7, i = blockIdx.x >> 3;
+  const long L = xcd * chunk + i;
+  return (i < chunk && L < total) ? L : -1;
+}
+
 // weight[Cout][cin_g][taps] -> wT[G][M_pad][cout_g], row m = tap * cin_g + c,
 // zero rows from taps * cin_g up to M_pad (a multiple of kCgTile).
 template <typename E>
@@ -56,6 +69,7 @@ struct ColGradArgs {
   int cin_g, cout_g, taps, G, Cin, Cout;
   int kslabs;      // cout_g / KC
   int n0;          // first image of the pass
+  long total;      // workgroups with work: images of the pass x G x px_tiles x m_tiles
   uint32_t *dmax;  // bit pattern of the largest |d| stored so far (a float >= 0), or null
 };
 
@@ -77,13 +91,15 @@ __global__ __launch_bounds__(256, 2) void bwd_colgrad_kernel(ColGradArgs a) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int frow = lane & 31, fhalf = lane >> 5;
   const int wm = wave & 1, wn = wave >> 1;
-  int b = blockIdx.x;
-  const int mt = b % a.m_tiles;
+  // (the row tiles of one pixel tile are neighbours: they share the grad_output tile)
+  long b = xcd_work_index(a.total);
+  if (b < 0) return;
+  const int mt = (int)(b % a.m_tiles);
   b /= a.m_tiles;
-  const int pt = b % a.px_tiles;
+  const int pt = (int)(b % a.px_tiles);
   b /= a.px_tiles;
-  const int grp = b % a.G;
-  const int nl = b / a.G;
+  const int grp = (int)(b % a.G);
+  const int nl = (int)(b / a.G);
   const int n = a.n0 + nl;
 
   // this lane's share of the copies: 4 of the 16 one-KiB blocks (8 rows) of each tile
@@ -508,6 +524,7 @@ struct WGradArgs {
   int cin_g, cout_g, taps, G, Cin, Cout;
   int co_tiles, m_tiles;
   int splits;        // workgroups sharing the (image, K step) range of one tile
+  long total;        // workgroups with work: G x co_tiles x m_tiles x splits
 };
 
 // grad_weight[co, (c, tap)] += sum over the pass's images and pixels of
@@ -531,12 +548,16 @@ __global__ __launch_bounds__(256, 2) void bwd_wgrad_kernel(WGradArgs a) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int frow = lane & 31, fhalf = lane >> 5;
   const int wm = wave & 1, wn = wave >> 1;
-  int b = blockIdx.x;
-  const int mt = b % a.m_tiles;
+  // (all tiles of one share of the K range are neighbours: those of a row of
+  // tiles share the grad_output tile, those of a column the columns tile)
+  long b = xcd_work_index(a.total);
+  if (b < 0) return;
+  const int ct = (int)(b % a.co_tiles);
+  b /= a.co_tiles;
+  const int mt = (int)(b % a.m_tiles);
   b /= a.m_tiles;
-  const int ct = b % a.co_tiles;
-  const int grp = b / a.co_tiles;
-  const int split = blockIdx.y;
+  const int grp = (int)(b % a.G);
+  const int split = (int)(b / a.G);
 
   // this lane's rows and 16-byte chunk of the copies
   long a_row[4], b_row[4];
