@@ -188,9 +188,9 @@ int mdcn_pack_forward_timed(const mdcn_pack_params *p, void *hip_stream, float m
  * offset, grad_mask like mask (must be NULL when conv.mask is), grad_weight like
  * weight, grad_bias (Cout).  grad_input and grad_offset/grad_mask are produced
  * together: pass all of them or none.  Sums are formed in fp32 and rounded once.
- * The scatter into grad_input and the pixel reduction of grad_weight use
- * floating-point atomics, so results vary in the last bits from run to run, as
- * the reference's CUDA kernels' do.
+ * The scatter into grad_input (and, for shapes off the matrix-core path, the
+ * pixel reduction of grad_weight) uses floating-point atomics, so results vary
+ * in the last bits from run to run, as the reference's CUDA kernels' do.
  */
 typedef struct mdcn_bwd_params {
   mdcn_params conv;

@@ -483,14 +483,18 @@ struct BwdPlan {
   int sR, sWH, sWW;  // window of the scatter kernel
   int sCH;         // channels per pass over that window
   int n_chunk;     // images per pass
+  int cg_tile;     // tile of the column-gradient product (kCgTile or kCgTileBig)
   int M_pad;       // rows of the transposed weight matrix per group
   long P_pad;      // row pitch of the columns matrix
   int parts;       // workgroups of the scatter kernel per tile (shares of the channels)
   size_t xt_bytes, gt_bytes, wt_bytes, d_bytes, col_bytes, part_bytes;
+  int w_tile, w_splits;  // weight-gradient product: tile, shares of the K range
+  size_t wpart_bytes;    // ... and their partial sums
   size_t gb_bytes;  // fp32 sum of grad_bias (16-bit tensors)
   size_t mx_bytes;  // the two maxima that scale the fixed-point window (16-bit tensors)
   size_t total() const {
-    return gin_bytes + gw_bytes + gb_bytes + mx_bytes + xt_bytes + gt_bytes + wt_bytes + d_bytes + col_bytes + part_bytes;
+    return gin_bytes + gw_bytes + gb_bytes + mx_bytes + xt_bytes + gt_bytes + wt_bytes + d_bytes + col_bytes + part_bytes +
+           wpart_bytes;
   }
 };
 
@@ -502,10 +506,13 @@ void make_bwd_plan(const mdcn_bwd_params *bp, const Geom &g, BwdPlan *pl) {
   pl->gb_bytes = (staged && bp->grad_bias) ? align_up((size_t)g.Cout * 4) : 0;
   pl->mx_bytes = 0;
   pl->tiled = pl->gemm = pl->wgemm = false;
-  pl->xt_bytes = pl->gt_bytes = pl->wt_bytes = pl->d_bytes = pl->col_bytes = pl->part_bytes = 0;
+  pl->xt_bytes = pl->gt_bytes = pl->wt_bytes = pl->d_bytes = pl->col_bytes = pl->part_bytes = pl->wpart_bytes = 0;
+  pl->w_tile = kCgTile;
+  pl->w_splits = 1;
   pl->parts = 1;
   pl->n_chunk = g.N;
   pl->M_pad = 0;
+  pl->cg_tile = kCgTile;
   pl->P_pad = 0;
   pl->R = pl->sR = -1;
   pl->WH = pl->WW = pl->sWH = pl->sWW = 0;
@@ -545,7 +552,8 @@ void make_bwd_plan(const mdcn_bwd_params *bp, const Geom &g, BwdPlan *pl) {
     pl->xt_bytes = align_up((size_t)g.N * (g.Cin / KC) * g.Hp * g.Wp * 128);
   }
   if (pl->gemm) {
-    pl->M_pad = (g.taps * g.cin_g + kCgTile - 1) / kCgTile * kCgTile;
+    pl->cg_tile = (g.taps * g.cin_g >= kCgTileBig && plane_out >= (size_t)kCgTileBig) ? kCgTileBig : kCgTile;
+    pl->M_pad = (g.taps * g.cin_g + pl->cg_tile - 1) / pl->cg_tile * pl->cg_tile;
     pl->gt_bytes = align_up((size_t)g.N * (g.Cout / KC) * plane_out * 128);
     pl->wt_bytes = align_up((size_t)g.G * pl->M_pad * g.cout_g * es);
     pl->d_bytes = align_up(d_img * pl->n_chunk);
@@ -559,6 +567,14 @@ void make_bwd_plan(const mdcn_bwd_params *bp, const Geom &g, BwdPlan *pl) {
     const long kpx = 128 / (long)es;  // pixels per K step
     pl->P_pad = ((long)plane_out + kpx - 1) / kpx * kpx;
     pl->col_bytes = align_up((size_t)pl->n_chunk * g.taps * g.Cin * pl->P_pad * es);
+    const int M = g.taps * g.cin_g;
+    pl->w_tile = (g.cout_g >= 192 && M >= kCgTileBig) ? kCgTileBig : kCgTile;
+    const long tiles = (long)g.G * ((g.cout_g + pl->w_tile - 1) / pl->w_tile) * ((M + pl->w_tile - 1) / pl->w_tile);
+    // one round of workgroups (256-tiles: one per CU, 128-tiles: two), shares of at least 8 K steps
+    const long slots = pl->w_tile == kCgTileBig ? 256 : 512;
+    const long work = (long)pl->n_chunk * (pl->P_pad / kpx);
+    pl->w_splits = (int)std::max<long>(1, std::min<long>(std::min<long>(work / 8, 64), slots / tiles));
+    pl->wpart_bytes = align_up((size_t)pl->w_splits * g.Cout * M * 4);
   }
   if (bp->grad_input && !pl->gemm) {
     // (small problems keep the per-tap kernel: it has taps x more workgroups)
@@ -593,6 +609,7 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
   const long off_total = (long)g.N * g.DG * 2 * g.taps * plane_out, mask_total = off_total / 2;
   float *poff = (float *)(col + pl.col_bytes);
   float *pmask = poff + (long)pl.parts * off_total;
+  float *wpart = (float *)(col + pl.col_bytes + pl.part_bytes);
   // the weight-gradient product copies grad_output rows 16 bytes at a time
   const bool wgemm = pl.wgemm && ((uintptr_t)bp->grad_output % 16) == 0;
   const bool gemm = pl.gemm;
@@ -653,8 +670,8 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
         ca.gT = gT;
         ca.D = D;
         ca.P = (int)plane_out;
-        ca.px_tiles = (int)((plane_out + kCgTile - 1) / kCgTile);
-        ca.m_tiles = pl.M_pad / kCgTile;
+        ca.px_tiles = (int)((plane_out + pl.cg_tile - 1) / pl.cg_tile);
+        ca.m_tiles = pl.M_pad / pl.cg_tile;
         ca.M = g.taps * g.cin_g;
         ca.M_pad = pl.M_pad;
         ca.cin_g = g.cin_g;
@@ -667,7 +684,12 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
         ca.n0 = n0;
         ca.dmax = pl.mx_bytes ? maxima : nullptr;
         ca.total = (long)nb * g.G * ca.px_tiles * ca.m_tiles;
-        hipLaunchKernelGGL(bwd_colgrad_kernel<E>, dim3((unsigned)((ca.total + 7) / 8 * 8)), dim3(256), 0, st, ca);
+        if (pl.cg_tile == kCgTileBig)
+          hipLaunchKernelGGL((bwd_colgrad_kernel<E, kCgTileBig>), dim3((unsigned)((ca.total + 7) / 8 * 8)),
+                             dim3(2 * kCgTileBig), 0, st, ca);
+        else
+          hipLaunchKernelGGL((bwd_colgrad_kernel<E, kCgTile>), dim3((unsigned)((ca.total + 7) / 8 * 8)),
+                             dim3(2 * kCgTile), 0, st, ca);
         check();
       }
       BwdScatterArgs sa;
@@ -711,7 +733,7 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
         WGradArgs wa;
         wa.gout = bp->grad_output;
         wa.col = col;
-        wa.gw32 = gw32;
+        wa.part = wpart;
         wa.P = (int)plane_out;
         wa.P_pad = pl.P_pad;
         wa.ksteps = (int)(pl.P_pad / KC);
@@ -724,13 +746,21 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
         wa.G = g.G;
         wa.Cin = g.Cin;
         wa.Cout = g.Cout;
-        wa.co_tiles = (g.cout_g + kCgTile - 1) / kCgTile;
-        wa.m_tiles = (wa.M + kCgTile - 1) / kCgTile;
+        const int wtile = pl.w_tile;
+        wa.co_tiles = (g.cout_g + wtile - 1) / wtile;
+        wa.m_tiles = (wa.M + wtile - 1) / wtile;
         const long tiles = (long)g.G * wa.co_tiles * wa.m_tiles;
-        const long work = (long)nb * wa.ksteps;
-        wa.splits = (int)std::max<long>(1, std::min<long>(std::min<long>(work, 65535), (4L * num_cus() + tiles - 1) / tiles));
+        wa.splits = pl.w_splits;
         wa.total = tiles * wa.splits;
-        hipLaunchKernelGGL(bwd_wgrad_kernel<E>, dim3((unsigned)((wa.total + 7) / 8 * 8)), dim3(256), 0, st, wa);
+        if (wtile == kCgTileBig)
+          hipLaunchKernelGGL((bwd_wgrad_kernel<E, kCgTileBig>), dim3((unsigned)((wa.total + 7) / 8 * 8)),
+                             dim3(2 * kCgTileBig), 0, st, wa);
+        else
+          hipLaunchKernelGGL((bwd_wgrad_kernel<E, kCgTile>), dim3((unsigned)((wa.total + 7) / 8 * 8)),
+                             dim3(2 * kCgTile), 0, st, wa);
+        check();
+        hipLaunchKernelGGL(wgrad_reduce_kernel, dim3(blocks_for(n_w)), dim3(256), 0, st, wpart, gw32, wa.splits,
+                           g.cin_g, g.taps, n_w);
         check();
       }
     }

@@ -22,8 +22,13 @@
 
 namespace mdcn {
 
-// Rows of either operand per workgroup tile of the column-gradient product.
+// Rows of either operand per workgroup tile of the two products: 256 (8
+// wavefronts, each 128 x 64) where both operands have that many rows, else 128
+// (4 wavefronts, each 64 x 64).  Per K step a 256-tile moves 64 KB for 2 048 MFMA
+// clocks, a 128-tile 32 KB for 512: with two K steps in flight the small tile is
+// bound by the latency of its copies, the large one is not.
 constexpr int kCgTile = 128;
+constexpr int kCgTileBig = 256;
 
 // Work index of a workgroup of a 1-D launch of 8 * ceil(total / 8) workgroups, or
 // -1 for the few that have none.  Consecutive workgroup ids sit on different
@@ -73,21 +78,23 @@ struct ColGradArgs {
   uint32_t *dmax;  // bit pattern of the largest |d| stored so far (a float >= 0), or null
 };
 
-// Workgroup = 128 rows of wT (one group) x 128 pixels of one image, reduction
-// over the group's output channels in slabs of 128 bytes; 4 waves as 2 x 2, each
-// 2 x 2 MFMA blocks of 32 x 32.  Both operand tiles of a slab go to LDS with
+// Workgroup = TILE rows of wT (one group) x TILE pixels of one image, reduction
+// over the group's output channels in slabs of 128 bytes; TILE / 32 waves as
+// 2 x TILE / 64, each TILE / 64 x 2 MFMA blocks of 32 x 32.  Both operand tiles of a slab go to LDS with
 // 16-byte direct-to-LDS copies (rows of 128 bytes, the 16-byte chunks of a row
 // swizzled by the row number on the source side, so that fragment reads are
 // conflict free), double buffered.  A rows = (tap, channel), B rows = pixels:
 // a lane ends up with 4 x 4 consecutive channels of one pixel, which is what the
 // d layout wants (8- or 16-byte stores).
-template <typename E>
-__global__ __launch_bounds__(256, 2) void bwd_colgrad_kernel(ColGradArgs a) {
+template <typename E, int TILE>
+__global__ __launch_bounds__(TILE * 2, TILE == 128 ? 2 : 1) void bwd_colgrad_kernel(ColGradArgs a) {
   using TR = ElemTraits<E>;
   constexpr int ES = (int)sizeof(E);
   constexpr int KC = 128 / ES;
-  __shared__ uint4 As[2][kCgTile * 8];
-  __shared__ uint4 Bs[2][kCgTile * 8];
+  constexpr int MB = TILE / 64;            // 32-row blocks of A per wave
+  constexpr uint32_t kBuf = TILE * 128u;   // bytes of one operand tile
+  __shared__ uint4 As[2][TILE * 8];
+  __shared__ uint4 Bs[2][TILE * 8];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int frow = lane & 31, fhalf = lane >> 5;
   const int wm = wave & 1, wn = wave >> 1;
@@ -109,9 +116,9 @@ __global__ __launch_bounds__(256, 2) void bwd_colgrad_kernel(ColGradArgs a) {
     const int row = (wave * 4 + c) * 8 + (lane >> 3);
     const int ch = (lane & 7) ^ (row & 7);
     a_src[c] = (const unsigned char *)a.wT +
-               ((long)grp * a.M_pad + (long)mt * kCgTile + row) * a.cout_g * ES + ch * 16;
+               ((long)grp * a.M_pad + (long)mt * TILE + row) * a.cout_g * ES + ch * 16;
     // rows past the image repeat its last pixel; they are never stored
-    const int px = min(pt * kCgTile + row, a.P - 1);
+    const int px = min(pt * TILE + row, a.P - 1);
     b_src[c] = (const unsigned char *)a.gT +
                (((long)n * (a.Cout / KC) + (long)grp * a.kslabs) * a.P + px) * 128 + ch * 16;
   }
@@ -123,14 +130,14 @@ __global__ __launch_bounds__(256, 2) void bwd_colgrad_kernel(ColGradArgs a) {
   auto issue = [&](int ks, int buf) {
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
-      copy16_global_to_lds(a_src[c] + (long)ks * 128, lds_a + (uint32_t)buf * 16384u + (uint32_t)c * 1024u);
-      copy16_global_to_lds(b_src[c] + (long)ks * b_step, lds_b + (uint32_t)buf * 16384u + (uint32_t)c * 1024u);
+      copy16_global_to_lds(a_src[c] + (long)ks * 128, lds_a + (uint32_t)buf * kBuf + (uint32_t)c * 1024u);
+      copy16_global_to_lds(b_src[c] + (long)ks * b_step, lds_b + (uint32_t)buf * kBuf + (uint32_t)c * 1024u);
     }
   };
 
-  f32x16 acc[2][2];
+  f32x16 acc[MB][2];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < MB; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -148,10 +155,10 @@ __global__ __launch_bounds__(256, 2) void bwd_colgrad_kernel(ColGradArgs a) {
     __syncthreads();
 #pragma unroll
     for (int ksub = 0; ksub < 4; ++ksub) {
-      uint4 af[2], bf[2];
+      uint4 af[MB], bf[2];
 #pragma unroll
-      for (int mb = 0; mb < 2; ++mb) {
-        const int row = wm * 64 + mb * 32 + frow;
+      for (int mb = 0; mb < MB; ++mb) {
+        const int row = wm * (TILE / 2) + mb * 32 + frow;
         af[mb] = As[buf][row * 8 + ((ksub * 2 + fhalf) ^ (row & 7))];
       }
 #pragma unroll
@@ -160,7 +167,7 @@ __global__ __launch_bounds__(256, 2) void bwd_colgrad_kernel(ColGradArgs a) {
         bf[nb] = Bs[buf][row * 8 + ((ksub * 2 + fhalf) ^ (row & 7))];
       }
 #pragma unroll
-      for (int mb = 0; mb < 2; ++mb)
+      for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
         for (int nb = 0; nb < 2; ++nb) TR::mma(acc[mb][nb], af[mb], bf[nb]);
     }
@@ -173,7 +180,7 @@ __global__ __launch_bounds__(256, 2) void bwd_colgrad_kernel(ColGradArgs a) {
   if (a.dmax) {  // (every accumulator counts: rows and pixels past the end repeat real ones or are zero)
     float mx = 0.0f;
 #pragma unroll
-    for (int mb = 0; mb < 2; ++mb)
+    for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
       for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
@@ -185,14 +192,14 @@ __global__ __launch_bounds__(256, 2) void bwd_colgrad_kernel(ColGradArgs a) {
     if (lane == 0 && __float_as_uint(mx) > __builtin_nontemporal_load(a.dmax)) atomicMax(a.dmax, __float_as_uint(mx));
   }
 #pragma unroll
-  for (int mb = 0; mb < 2; ++mb) {
-    const int m0 = mt * kCgTile + wm * 64 + mb * 32;  // a block = one tap, 32 consecutive channels
+  for (int mb = 0; mb < MB; ++mb) {
+    const int m0 = mt * TILE + wm * (TILE / 2) + mb * 32;  // a block = one tap, 32 consecutive channels
     if (m0 >= a.M) continue;
     const int tap = m0 / a.cin_g;
     const int cb = grp * a.cin_g + (m0 - tap * a.cin_g);
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb) {
-      const int px = pt * kCgTile + wn * 64 + nb * 32 + frow;
+      const int px = pt * TILE + wn * 64 + nb * 32 + frow;
       if (px >= a.P) continue;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
@@ -515,7 +522,7 @@ __global__ __launch_bounds__(256) void zero_col_pad_kernel(E *col, long rows, in
 struct WGradArgs {
   const void *gout;  // [N][Cout][P]
   const void *col;   // [images of the pass][G][taps][cin_g][P_pad]
-  float *gw32;       // (Cout, cin_g, kh, kw) fp32, zero before the first pass
+  float *part;       // partial sums [split][G][cout_g][M], every element written
   int P;
   long P_pad;
   int ksteps;        // P_pad / (pixels per 128 bytes)
@@ -536,15 +543,19 @@ struct WGradArgs {
 // in bwd_colgrad_kernel (grad_output is read in place: its rows are pixel
 // contiguous).  Runs of pixels past the end of an image read the row's last
 // 16 bytes again; the zero padding of col cancels them.  Rows past the group's
-// channels repeat its last row and are dropped at the end.  Partial sums leave
-// through fp32 atomics.
-template <typename E>
-__global__ __launch_bounds__(256, 2) void bwd_wgrad_kernel(WGradArgs a) {
+// channels repeat its last row and are dropped at the end.  Each share of the K
+// range stores its partial tile (plain stores, rows of M contiguous);
+// wgrad_reduce_kernel adds the shares up in a fixed order, so grad_weight does
+// not vary from run to run.
+template <typename E, int TILE>
+__global__ __launch_bounds__(TILE * 2, TILE == 128 ? 2 : 1) void bwd_wgrad_kernel(WGradArgs a) {
   using TR = ElemTraits<E>;
   constexpr int ES = (int)sizeof(E);
   constexpr int PXC = 16 / ES;  // pixels per 16-byte chunk
-  __shared__ uint4 As[2][kCgTile * 8];
-  __shared__ uint4 Bs[2][kCgTile * 8];
+  constexpr int MB = TILE / 64;
+  constexpr uint32_t kBuf = TILE * 128u;
+  __shared__ uint4 As[2][TILE * 8];
+  __shared__ uint4 Bs[2][TILE * 8];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int frow = lane & 31, fhalf = lane >> 5;
   const int wm = wave & 1, wn = wave >> 1;
@@ -566,8 +577,8 @@ __global__ __launch_bounds__(256, 2) void bwd_wgrad_kernel(WGradArgs a) {
   for (int c = 0; c < 4; ++c) {
     const int row = (wave * 4 + c) * 8 + (lane >> 3);
     chunk[c] = (lane & 7) ^ (row & 7);
-    const int co = min(ct * kCgTile + row, a.cout_g - 1);
-    const int m = min(mt * kCgTile + row, a.M - 1);
+    const int co = min(ct * TILE + row, a.cout_g - 1);
+    const int m = min(mt * TILE + row, a.M - 1);
     a_row[c] = ((long)grp * a.cout_g + co) * a.P;            // + n * Cout * P
     b_row[c] = ((long)grp * a.M + m) * a.P_pad;              // + nl * taps * Cin * P_pad
   }
@@ -585,14 +596,14 @@ __global__ __launch_bounds__(256, 2) void bwd_wgrad_kernel(WGradArgs a) {
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
       const int px = p0 + chunk[c] * PXC;
-      copy16_global_to_lds(ga + a_row[c] + min(px, last_chunk_px), lds_a + (uint32_t)buf * 16384u + (uint32_t)c * 1024u);
-      copy16_global_to_lds(cb + b_row[c] + px, lds_b + (uint32_t)buf * 16384u + (uint32_t)c * 1024u);
+      copy16_global_to_lds(ga + a_row[c] + min(px, last_chunk_px), lds_a + (uint32_t)buf * kBuf + (uint32_t)c * 1024u);
+      copy16_global_to_lds(cb + b_row[c] + px, lds_b + (uint32_t)buf * kBuf + (uint32_t)c * 1024u);
     }
   };
 
-  f32x16 acc[2][2];
+  f32x16 acc[MB][2];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < MB; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -615,10 +626,10 @@ __global__ __launch_bounds__(256, 2) void bwd_wgrad_kernel(WGradArgs a) {
       __syncthreads();
 #pragma unroll
       for (int ksub = 0; ksub < 4; ++ksub) {
-        uint4 af[2], bf[2];
+        uint4 af[MB], bf[2];
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb) {
-          const int row = wm * 64 + mb * 32 + frow;
+        for (int mb = 0; mb < MB; ++mb) {
+          const int row = wm * (TILE / 2) + mb * 32 + frow;
           af[mb] = As[buf][row * 8 + ((ksub * 2 + fhalf) ^ (row & 7))];
         }
 #pragma unroll
@@ -627,7 +638,7 @@ __global__ __launch_bounds__(256, 2) void bwd_wgrad_kernel(WGradArgs a) {
           bf[nb] = Bs[buf][row * 8 + ((ksub * 2 + fhalf) ^ (row & 7))];
         }
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb)
+        for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
           for (int nb = 0; nb < 2; ++nb) TR::mma(acc[mb][nb], af[mb], bf[nb]);
       }
@@ -636,21 +647,33 @@ __global__ __launch_bounds__(256, 2) void bwd_wgrad_kernel(WGradArgs a) {
   }
 
   // register r of lane l: A row (output channel) (r/4)*8 + (l/32)*4 + r%4 of the block, B row (column row) l%32
-  const int k_g = a.cin_g * a.taps;
+  float *part = a.part + ((long)split * a.G + grp) * a.cout_g * a.M;
 #pragma unroll
-  for (int mb = 0; mb < 2; ++mb)
+  for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb) {
-      const int m = mt * kCgTile + wn * 64 + nb * 32 + frow;
+      const int m = mt * TILE + wn * 64 + nb * 32 + frow;
       if (m >= a.M) continue;
-      const int tap = m / a.cin_g, cl = m - tap * a.cin_g;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int co = ct * kCgTile + wm * 64 + mb * 32 + (r >> 2) * 8 + fhalf * 4 + (r & 3);
-        if (co < a.cout_g)
-          unsafeAtomicAdd(a.gw32 + ((long)grp * a.cout_g + co) * k_g + (long)cl * a.taps + tap, acc[mb][nb][r]);
+        const int co = ct * TILE + wm * (TILE / 2) + mb * 32 + (r >> 2) * 8 + fhalf * 4 + (r & 3);
+        if (co < a.cout_g) part[(long)co * a.M + m] = acc[mb][nb][r];
       }
     }
+}
+
+// gw32[(grp, co), (c, tap)] += sum over the shares of part[share][grp][co][m = tap * cin_g + c].
+__global__ __launch_bounds__(256) void wgrad_reduce_kernel(const float *__restrict__ part, float *__restrict__ gw32,
+                                                           int splits, int cin_g, int taps, long n_w) {
+  const int M = cin_g * taps;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n_w; i += (long)gridDim.x * blockDim.x) {
+    const long row = i / M;  // (grp, co)
+    const int m = (int)(i - row * M);
+    float sum = 0.0f;
+    for (int sp = 0; sp < splits; ++sp) sum += part[(long)sp * n_w + i];
+    const int tap = m / cin_g, cl = m - tap * cin_g;
+    gw32[row * M + (long)cl * taps + tap] += sum;
+  }
 }
 
 }  // namespace mdcn
