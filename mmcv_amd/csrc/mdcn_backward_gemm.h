@@ -216,7 +216,8 @@ __global__ __launch_bounds__(TILE * 2, TILE == 128 ? 2 : 1) void bwd_colgrad_ker
 // channels of a WH x WW pixel neighbourhood of the tile; kScWindowPx pixels fit
 // with the larger channel count of a type (16-bit tensors: 16 channels of 32-bit
 // fixed point; fp32 tensors: 8 channels of doubles), twice as many -- stride 2,
-// dilation -- with the smaller one.
+// dilation -- with the smaller one.  (A 48 KB window with 8 channels and three
+// workgroups per CU was slower: the passes over the window double.)
 constexpr int kScWindowBytes = 60 * 1024;
 constexpr int kScWindowPx = kScWindowBytes / 64;
 // Contributions one window entry can receive at most: every (pixel, tap) of the
@@ -366,6 +367,16 @@ __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
   float acc_m[kBwdTapsMax], acc_y[kBwdTapsMax], acc_x[kBwdTapsMax];
 #pragma unroll
   for (int t = 0; t < kBwdTapsMax; ++t) acc_m[t] = acc_y[t] = acc_x[t] = 0.0f;
+  // this pixel's offsets and mask, fetched once: every channel pass needs them before it can
+  // address its corners, and a load there would also wait for the pass's older stores
+  E t_dy[kBwdTapsMax], t_dx[kBwdTapsMax], t_m[kBwdTapsMax];
+#pragma unroll
+  for (int t = 0; t < kBwdTapsMax; ++t) {
+    const int tc = min(t, g.taps - 1);
+    t_dy[t] = off[(long)(2 * tc) * a.om.off_ch];
+    t_dx[t] = off[(long)(2 * tc + 1) * a.om.off_ch];
+    t_m[t] = msk[(long)tc * a.om.msk_ch];
+  }
 
   const int part = blockIdx.y;
   const int ch_per_part = g.ch_per_dg / a.parts;
@@ -386,9 +397,12 @@ __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
     for (int tap = 0; tap < kBwdTapsMax; ++tap) {
       if (tap < g.taps) {
         const int ti = tap / g.kw, tj = tap - ti * g.kw;
-        const float dy = to_f32(off[(long)(2 * tap) * a.om.off_ch]);
-        const float dx = to_f32(off[(long)(2 * tap + 1) * a.om.off_ch]);
-        const float m = mask_value<E>(msk[(long)tap * a.om.msk_ch], a.om.logit);
+        float dy = to_f32(t_dy[tap]);
+        float dx = to_f32(t_dx[tap]);
+        // (opaque to the optimiser: it would otherwise move the position arithmetic of all taps
+        // out of the channel loop and spill what that keeps alive)
+        asm volatile("" : "+v"(dy), "+v"(dx));
+        const float m = mask_value<E>(t_m[tap], a.om.logit);
         const float py = (float)(ho * g.sh - g.ph + ti * g.dh) + dy;
         const float px = (float)(wo * g.sw - g.pw + tj * g.dw) + dx;
         const bool inside =
