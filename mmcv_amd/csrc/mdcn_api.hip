@@ -490,11 +490,12 @@ struct BwdPlan {
   size_t xt_bytes, gt_bytes, wt_bytes, d_bytes, col_bytes, part_bytes;
   int w_tile, w_splits;  // weight-gradient product: tile, shares of the K range
   size_t wpart_bytes;    // ... and their partial sums
+  size_t gpad_bytes;     // grad_output with padded rows, when its own rows cannot be copied 16 bytes at a time
   size_t gb_bytes;  // fp32 sum of grad_bias (16-bit tensors)
   size_t mx_bytes;  // the two maxima that scale the fixed-point window (16-bit tensors)
   size_t total() const {
     return gin_bytes + gw_bytes + gb_bytes + mx_bytes + xt_bytes + gt_bytes + wt_bytes + d_bytes + col_bytes + part_bytes +
-           wpart_bytes;
+           wpart_bytes + gpad_bytes;
   }
 };
 
@@ -509,6 +510,7 @@ void make_bwd_plan(const mdcn_bwd_params *bp, const Geom &g, BwdPlan *pl) {
   pl->xt_bytes = pl->gt_bytes = pl->wt_bytes = pl->d_bytes = pl->col_bytes = pl->part_bytes = pl->wpart_bytes = 0;
   pl->w_tile = kCgTile;
   pl->w_splits = 1;
+  pl->gpad_bytes = 0;
   pl->parts = 1;
   pl->n_chunk = g.N;
   pl->M_pad = 0;
@@ -544,8 +546,7 @@ void make_bwd_plan(const mdcn_bwd_params *bp, const Geom &g, BwdPlan *pl) {
                        d_img <= kBwdColGradCap && plane_out <= ((size_t)1 << 30);
   if (mfma_ok) {
     pl->gemm = bp->grad_input != nullptr;
-    // (grad_output rows are copied to LDS 16 bytes at a time)
-    pl->wgemm = bp->grad_weight != nullptr && plane_out % (16 / es) == 0;
+    pl->wgemm = bp->grad_weight != nullptr;
   }
   if (pl->gemm || pl->wgemm) {
     pl->n_chunk = (int)std::min<uint64_t>((uint64_t)g.N, std::max<uint64_t>(1, g_bwd_pass_bytes / d_img));
@@ -575,6 +576,9 @@ void make_bwd_plan(const mdcn_bwd_params *bp, const Geom &g, BwdPlan *pl) {
     const long work = (long)pl->n_chunk * (pl->P_pad / kpx);
     pl->w_splits = (int)std::max<long>(1, std::min<long>(std::min<long>(work / 8, 64), slots / tiles));
     pl->wpart_bytes = align_up((size_t)pl->w_splits * g.Cout * M * 4);
+    // grad_output rows go to LDS 16 bytes at a time: in place when they start aligned
+    if (plane_out % (16 / es) != 0 || ((uintptr_t)bp->grad_output % 16) != 0)
+      pl->gpad_bytes = align_up((size_t)g.N * g.Cout * pl->P_pad * es);
   }
   if (bp->grad_input && !pl->gemm) {
     // (small problems keep the per-tap kernel: it has taps x more workgroups)
@@ -610,8 +614,8 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
   float *poff = (float *)(col + pl.col_bytes);
   float *pmask = poff + (long)pl.parts * off_total;
   float *wpart = (float *)(col + pl.col_bytes + pl.part_bytes);
-  // the weight-gradient product copies grad_output rows 16 bytes at a time
-  const bool wgemm = pl.wgemm && ((uintptr_t)bp->grad_output % 16) == 0;
+  const bool wgemm = pl.wgemm;
+  unsigned char *gpad = (unsigned char *)wpart + pl.wpart_bytes;
   const bool gemm = pl.gemm;
 
   if (bp->grad_input) {
@@ -654,6 +658,12 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
       const long wtotal = (long)g.G * pl.M_pad * g.cout_g;
       hipLaunchKernelGGL(pack_weight_t_kernel<E>, dim3(blocks_for(wtotal)), dim3(256), 0, st, g,
                          (const E *)p->weight, (E *)wT, pl.M_pad, wtotal);
+      check();
+    }
+    if (wgemm && pl.gpad_bytes) {
+      const long rows = (long)g.N * g.Cout;
+      hipLaunchKernelGGL(pad_rows_kernel<E>, dim3(blocks_for(rows * pl.P_pad)), dim3(256), 0, st,
+                         (const E *)bp->grad_output, (E *)gpad, rows, (int)plane_out, pl.P_pad);
       check();
     }
     if (wgemm && pl.P_pad > plane_out) {
@@ -731,7 +741,8 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
       check();
       if (wgemm) {
         WGradArgs wa;
-        wa.gout = bp->grad_output;
+        wa.gout = pl.gpad_bytes ? (const void *)gpad : bp->grad_output;
+        wa.a_pitch = pl.gpad_bytes ? pl.P_pad : plane_out;
         wa.col = col;
         wa.part = wpart;
         wa.P = (int)plane_out;

@@ -533,8 +533,22 @@ __global__ __launch_bounds__(256) void zero_col_pad_kernel(E *col, long rows, in
   }
 }
 
+// dst[row][0 .. P_pad) = src[row][0 .. P), zeros behind: grad_output with rows that start 16-byte
+// aligned, for images whose pixel count is not a multiple of the copy granule.
+template <typename E>
+__global__ __launch_bounds__(256) void pad_rows_kernel(const E *__restrict__ src, E *__restrict__ dst, long rows,
+                                                       int P, long P_pad) {
+  const long total = rows * P_pad;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+    const long r = i / P_pad;
+    const long p = i - r * P_pad;
+    dst[i] = p < P ? src[r * P + p] : from_f32<E>(0.0f);
+  }
+}
+
 struct WGradArgs {
-  const void *gout;  // [N][Cout][P]
+  const void *gout;  // [N][Cout][a_pitch]: grad_output in place (a_pitch = P) or its padded copy (P_pad)
+  long a_pitch;
   const void *col;   // [images of the pass][G][taps][cin_g][P_pad]
   float *part;       // partial sums [split][G][cout_g][M], every element written
   int P;
@@ -593,7 +607,7 @@ __global__ __launch_bounds__(TILE * 2, TILE == 128 ? 2 : 1) void bwd_wgrad_kerne
     chunk[c] = (lane & 7) ^ (row & 7);
     const int co = min(ct * TILE + row, a.cout_g - 1);
     const int m = min(mt * TILE + row, a.M - 1);
-    a_row[c] = ((long)grp * a.cout_g + co) * a.P;            // + n * Cout * P
+    a_row[c] = ((long)grp * a.cout_g + co) * a.a_pitch;      // + n * Cout * a_pitch
     b_row[c] = ((long)grp * a.M + m) * a.P_pad;              // + nl * taps * Cin * P_pad
   }
   const uint32_t lds_a = (uint32_t)(uintptr_t)(lptr_t)(&As[0][0]) +
@@ -601,11 +615,11 @@ __global__ __launch_bounds__(TILE * 2, TILE == 128 ? 2 : 1) void bwd_wgrad_kerne
   const uint32_t lds_b = (uint32_t)(uintptr_t)(lptr_t)(&Bs[0][0]) +
                          (uint32_t)__builtin_amdgcn_readfirstlane(wave) * 4096u;
   const E *gout = (const E *)a.gout, *col = (const E *)a.col;
-  const int last_chunk_px = a.P - PXC;  // (P is a multiple of PXC)
+  const int last_chunk_px = (int)a.a_pitch - PXC;  // (the pitch is a multiple of PXC)
   auto issue = [&](long wi, int buf) {
     const int nl = (int)(wi / a.ksteps);
     const int p0 = (int)(wi - (long)nl * a.ksteps) * (8 * PXC);
-    const E *ga = gout + (long)(a.n0 + nl) * a.Cout * a.P;
+    const E *ga = gout + (long)(a.n0 + nl) * a.Cout * a.a_pitch;
     const E *cb = col + (long)nl * a.taps * a.Cin * a.P_pad;
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
