@@ -35,6 +35,9 @@ SMALL = {
     'far_offsets': dict(N=1, Cin=64, Cout=32, H=10, W=10, sigma=8.0),
     'cout256': dict(N=1, Cin=64, Cout=256, H=14, W=14),
     'cout512': dict(N=1, Cin=64, Cout=512, H=9, W=9),
+    'cout384_dg2': dict(N=2, Cin=128, Cout=384, H=9, W=11, deform_groups=2),
+    'cout640_s2': dict(N=1, Cin=64, Cout=640, H=13, W=15, stride=2),
+    'cout1024_g2': dict(N=1, Cin=128, Cout=1024, H=8, W=10, groups=2),
     'pad0': dict(N=1, Cin=64, Cout=32, H=9, W=9, padding=0),
     'asym': dict(N=1, Cin=64, Cout=32, H=17, W=12, stride=(2, 1), padding=(0, 2), dilation=(1, 2)),
     'odd_plane': dict(N=3, Cin=64, Cout=64, H=7, W=9),
