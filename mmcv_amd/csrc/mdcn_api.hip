@@ -650,7 +650,7 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
         check();
         if (p->mask) {
           const long n_mask = (long)g.N * g.DG * g.taps * plane_out;
-          hipLaunchKernelGGL(absmax_kernel<E>, dim3(std::min(blocks_for(n_mask / 8), 1024)), dim3(256), 0, st,
+          hipLaunchKernelGGL(absmax_kernel<E>, dim3(std::min(blocks_for(n_mask / 8), 256)), dim3(256), 0, st,
                              (const E *)p->mask, n_mask, maxima + 1);
           check();
         }

@@ -56,7 +56,19 @@ __global__ __launch_bounds__(256) void bwd_bias_kernel(Geom g, const E *__restri
     const long p0 = (wi - (long)n * runs_per_image) * kBiasRun;
     const long p1 = min(plane, p0 + kBiasRun);
     const E *row = gout + ((long)n * g.Cout + co) * plane;
-    for (long p = p0 + threadIdx.x; p < p1; p += 256) s += to_f32(row[p]);
+    constexpr int EPV = 16 / (int)sizeof(E);  // elements per 16-byte load
+    if (plane % EPV == 0 && ((uintptr_t)gout % 16) == 0) {  // (runs start at multiples of kBiasRun)
+      const long nv = (p1 - p0) / EPV;
+      for (long v = threadIdx.x; v < nv; v += 256) {
+        const uint4 q = *(const uint4 *)(row + p0 + v * EPV);
+        const E *e = (const E *)&q;
+#pragma unroll
+        for (int i = 0; i < EPV; ++i) s += to_f32(e[i]);
+      }
+      for (long p = p0 + nv * EPV + threadIdx.x; p < p1; p += 256) s += to_f32(row[p]);
+    } else {
+      for (long p = p0 + threadIdx.x; p < p1; p += 256) s += to_f32(row[p]);
+    }
   }
   part[threadIdx.x] = s;
   __syncthreads();

@@ -228,11 +228,23 @@ constexpr int kScMaxAdds = 256 * 9;
 template <typename E>
 __global__ __launch_bounds__(256) void absmax_kernel(const E *__restrict__ x, long n, uint32_t *out) {
   float mx = 0.0f;
-  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
+  constexpr int EPV = 16 / (int)sizeof(E);  // elements per 16-byte load
+  const long nv = (((uintptr_t)x % 16) == 0) ? n / EPV : 0;
+  for (long v = (long)blockIdx.x * blockDim.x + threadIdx.x; v < nv; v += (long)gridDim.x * blockDim.x) {
+    const uint4 q = ((const uint4 *)x)[v];
+    const E *e = (const E *)&q;
+#pragma unroll
+    for (int i = 0; i < EPV; ++i) mx = fmaxf(mx, fabsf(to_f32(e[i])));
+  }
+  for (long i = nv * EPV + (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
     mx = fmaxf(mx, fabsf(to_f32(x[i])));
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
-  if ((threadIdx.x & 63) == 0 && __float_as_uint(mx) > __builtin_nontemporal_load(out)) atomicMax(out, __float_as_uint(mx));
+  __shared__ float wmax[4];
+  if ((threadIdx.x & 63) == 0) wmax[threadIdx.x >> 6] = mx;
+  __syncthreads();
+  if (threadIdx.x == 0)  // one atomic per workgroup: they all queue on one address
+    atomicMax(out, __float_as_uint(fmaxf(fmaxf(wmax[0], wmax[1]), fmaxf(wmax[2], wmax[3]))));
 }
 
 // CH consecutive channels (8 to 32 bytes) as floats.
