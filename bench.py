@@ -307,6 +307,19 @@ def main():
     torch.cuda.synchronize()
     cabi_ms = e0.elapsed_time(e1) / a.steps
     del cws
+    # what the matrix cores of this box sustain (back-to-back MFMAs on every CU, random and zero
+    # operands): context for the published peak the roofline fraction is taken against
+    sustained = None
+    if dname in ('bf16', 'f16'):
+        scratch = torch.empty(16384, dtype=torch.uint8, device='cuda')
+        tf = ctypes.c_float()
+        sustained = {}
+        for key, zero in (('random_operands', 0), ('zero_operands', 1)):
+            rc = lib.mdcn_mfma_probe(2 if dname == 'bf16' else 1, 2, zero, ctypes.c_void_p(scratch.data_ptr()), cstream,
+                                     ctypes.byref(tf))
+            assert rc == 0, capi.status_string(rc)
+            sustained[key] = round(tf.value, 1)
+        log(f'sustained MFMA rate: {sustained}')
     log(f'per call: median {per_call[len(per_call) // 2]:.4f} min {per_call[0]:.4f} ms; rotating buffers '
         f'{rot_ms:.4f} ms; bare C ABI {cabi_ms:.4f} ms')
 
@@ -377,6 +390,10 @@ def main():
             # WRITE_SIZE, scaled by a copy kernel (profiles/fused_kernel_bf16_cfg4.md)
             'traffic': 378.3e6 if a.workload == 'cfg4' else None,
         },
+        # measured on this box, same run: TFLOP/s of back-to-back 32x32x16 MFMAs on all CUs; the kernel's
+        # share of what the matrix cores sustain on non-trivial operands
+        'mfma_sustained_TFLOPs': sustained,
+        'frac_of_sustained': (round(achieved / sustained['random_operands'], 4) if sustained else None),
     }
     if not a.no_cpu:
         log('timing the CPU baseline ...')

@@ -132,6 +132,16 @@ int mdcn_forward(const mdcn_params *p, void *hip_stream);
  * Stages a path does not run report 0.  For measurement only. */
 int mdcn_forward_timed(const mdcn_params *p, void *hip_stream, float ms[4]);
 
+/* Measures what the matrix cores of the current device sustain: every CU runs
+ * `waves_per_simd` (1 or 2) wavefronts of back-to-back 32x32x16 MFMAs (dtype
+ * MDCN_BF16 or MDCN_F16) on pseudo-random operands, or on zeros with `zero_data`
+ * != 0 (the clock, and with it the rate, depends on how much the operands
+ * toggle).  Launches on `hip_stream`, waits for it and stores TFLOP/s in
+ * *tflops.  Uses `scratch`, at least 16 KiB of device memory.  For
+ * measurement only: the bench reports it beside the published peak.  (No
+ * counterpart in the reference.) */
+int mdcn_mfma_probe(int dtype, int waves_per_simd, int zero_data, void *scratch, void *hip_stream, float *tflops);
+
 /*
  * The deformable convolution together with the step in front of it in
  * ModulatedDeformConv2dPack.forward (mmcv/ops/modulated_deform_conv.py:327-335):

@@ -15,7 +15,7 @@ MDCN_OK = 0
 
 EXPORTS = ('mdcn_abi_version', 'mdcn_set_pass_limits', 'mdcn_status_string', 'mdcn_output_size',
            'mdcn_fused_eligible', 'mdcn_workspace_bytes', 'mdcn_forward',
-           'mdcn_forward_timed', 'mdcn_pack_workspace_bytes', 'mdcn_pack_forward',
+           'mdcn_forward_timed', 'mdcn_mfma_probe', 'mdcn_pack_workspace_bytes', 'mdcn_pack_forward',
            'mdcn_pack_forward_timed', 'mdcn_backward_workspace_bytes', 'mdcn_backward')
 
 
@@ -68,6 +68,9 @@ def load():
         lib.mdcn_forward_timed.restype = ctypes.c_int
         lib.mdcn_forward_timed.argtypes = [P, ctypes.c_void_p,
                                            ctypes.POINTER(ctypes.c_float)]
+        lib.mdcn_mfma_probe.restype = ctypes.c_int
+        lib.mdcn_mfma_probe.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p,
+                                        ctypes.POINTER(ctypes.c_float)]
         PP = ctypes.POINTER(MdcnPackParams)
         lib.mdcn_pack_workspace_bytes.restype = ctypes.c_size_t
         lib.mdcn_pack_workspace_bytes.argtypes = [PP]

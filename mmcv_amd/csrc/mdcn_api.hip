@@ -936,6 +936,50 @@ int mdcn_forward(const mdcn_params *p, void *hip_stream) {
   return run(p, hip_stream, nullptr);
 }
 
+int mdcn_mfma_probe(int dtype, int waves_per_simd, int zero_data, void *scratch, void *hip_stream, float *tflops) {
+  if (!scratch || !tflops) return MDCN_ERR_NULL;
+  if (dtype != MDCN_BF16 && dtype != MDCN_F16) return MDCN_ERR_DTYPE;
+  if (waves_per_simd < 1 || waves_per_simd > 2) return MDCN_ERR_SHAPE;
+  hipStream_t st = (hipStream_t)hip_stream;
+  // operands: 4096 words of two 16-bit values of magnitude 0.5 .. 2 with random signs and
+  // mantissas (finite in both formats)
+  uint32_t host[4096];
+  uint32_t rng = 12345u;
+  auto next = [&]() { rng = rng * 1664525u + 1013904223u; return rng >> 8; };
+  const uint32_t base = dtype == MDCN_BF16 ? 0x3f00u : 0x3800u;
+  for (int i = 0; i < 4096; ++i) {
+    const uint32_t lo = base + (next() & 0xffu) + ((next() & 1u) << 15);
+    const uint32_t hi = base + (next() & 0xffu) + ((next() & 1u) << 15);
+    host[i] = lo | (hi << 16);
+  }
+  if (hipMemcpyAsync(scratch, host, sizeof(host), hipMemcpyHostToDevice, st) != hipSuccess) return MDCN_ERR_LAUNCH;
+  if (hipStreamSynchronize(st) != hipSuccess) return MDCN_ERR_LAUNCH;
+  const int blocks = num_cus() * waves_per_simd, iters = 20000;
+  hipEvent_t e0, e1;
+  if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) return MDCN_ERR_LAUNCH;
+  auto launch = [&](int n) {
+    if (dtype == MDCN_BF16)
+      hipLaunchKernelGGL(mfma_probe_kernel<bf16_t>, dim3(blocks), dim3(256), 0, st, (const uint4 *)scratch,
+                         (float *)scratch, n, zero_data);
+    else
+      hipLaunchKernelGGL(mfma_probe_kernel<f16_t>, dim3(blocks), dim3(256), 0, st, (const uint4 *)scratch,
+                         (float *)scratch, n, zero_data);
+  };
+  launch(2000);  // warm up (clocks)
+  hipEventRecord(e0, st);
+  launch(iters);
+  hipEventRecord(e1, st);
+  int rc = MDCN_OK;
+  float ms = 0.0f;
+  if (hipEventSynchronize(e1) != hipSuccess || hipEventElapsedTime(&ms, e0, e1) != hipSuccess ||
+      hipGetLastError() != hipSuccess || ms <= 0.0f)
+    rc = MDCN_ERR_LAUNCH;
+  hipEventDestroy(e0);
+  hipEventDestroy(e1);
+  if (rc == MDCN_OK) *tflops = (float)((double)blocks * 4 * iters * 8 * 32768.0 / ms / 1e9);
+  return rc;
+}
+
 int mdcn_forward_timed(const mdcn_params *p, void *hip_stream, float ms[4]) {
   if (!ms) return MDCN_ERR_NULL;
   return run(p, hip_stream, ms);
