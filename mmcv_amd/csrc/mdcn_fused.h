@@ -172,6 +172,34 @@ struct ElemTraits<f16_t> : Half16Traits<f16_t> {
     c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
                                                __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
   }
+  // fp16 has packed arithmetic (bf16 on this chip has not): the table keeps every
+  // corner weight twice in one word, and a word of two channels takes one
+  // v_pk_mul_f16 and three v_pk_fma_f16 -- four instructions where the dot-product
+  // form needs nine.  The blend then rounds to fp16 after every corner instead of
+  // once (three more roundings of 2^-11 relative, far inside the fp16 bar).
+  static __device__ __forceinline__ void table_weights(const TapSample &s, uint32_t (&tw)[4]) {
+    tw[0] = pack2(s.w00, s.w00);
+    tw[1] = pack2(s.w01, s.w01);
+    tw[2] = pack2(s.w10, s.w10);
+    tw[3] = pack2(s.w11, s.w11);
+  }
+  static __device__ __forceinline__ uint4 blend(const uint4 &v0, const uint4 &v1, const uint4 &v2,
+                                                const uint4 &v3, const uint4 &w) {
+    const uint32_t c0[4] = {v0.x, v0.y, v0.z, v0.w}, c1[4] = {v1.x, v1.y, v1.z, v1.w};
+    const uint32_t c2[4] = {v2.x, v2.y, v2.z, v2.w}, c3[4] = {v3.x, v3.y, v3.z, v3.w};
+    const f16x2 w0 = __builtin_bit_cast(f16x2, w.x), w1 = __builtin_bit_cast(f16x2, w.y);
+    const f16x2 w2 = __builtin_bit_cast(f16x2, w.z), w3 = __builtin_bit_cast(f16x2, w.w);
+    uint32_t o[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      f16x2 acc = __builtin_bit_cast(f16x2, c0[j]) * w0;
+      acc = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, c1[j]), w1, acc);
+      acc = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, c2[j]), w2, acc);
+      acc = __builtin_elementwise_fma(__builtin_bit_cast(f16x2, c3[j]), w3, acc);
+      o[j] = __builtin_bit_cast(uint32_t, acc);
+    }
+    return make_uint4(o[0], o[1], o[2], o[3]);
+  }
 };
 
 // ---- fp32 --------------------------------------------------------------------
