@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define MDCN_ABI_VERSION 2
+#define MDCN_ABI_VERSION 3
 
 /* Element type of every tensor of a call (the Python wrapper unifies them to
  * offset's dtype, mmcv/ops/modulated_deform_conv.py:136-139). */
@@ -47,7 +47,8 @@ enum mdcn_status {
   MDCN_ERR_WORKSPACE = -4,  /* workspace missing, misaligned or smaller than mdcn_workspace_bytes() */
   MDCN_ERR_PATH = -5,       /* MDCN_PATH_FUSED asked for a shape it does not cover */
   MDCN_ERR_TOO_LARGE = -6,  /* one padded image exceeds the 32-bit byte offsets used on the device */
-  MDCN_ERR_LAUNCH = -7      /* HIP reported a launch error */
+  MDCN_ERR_LAUNCH = -7,     /* HIP reported a launch error */
+  MDCN_ERR_SCRATCH_LIMIT = -8 /* mdcn_forward_noalloc(): the call needs more than MDCN_NOALLOC_SCRATCH_BYTES */
 };
 
 /*
@@ -125,6 +126,22 @@ size_t mdcn_workspace_bytes(const mdcn_params *p);
  * modulated_deform_conv_forward_fallthrough for device tensors
  * (mmcv/ops/csrc/pytorch/modulated_deform_conv.cpp:62-138). */
 int mdcn_forward(const mdcn_params *p, void *hip_stream);
+
+/* mdcn_forward() for callers that cannot allocate device memory and have no
+ * workspace to pass: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  (No counterpart in the reference, which
+ * allocates its columns buffer inside the op.)  `workspace` and
+ * `workspace_bytes` of *p are ignored: the input copy and the packed weights go
+ * to a buffer of MDCN_NOALLOC_SCRATCH_BYTES that is part of the library's
+ * device image (each device the library runs on holds one until the process
+ * ends).  Calls whose mdcn_workspace_bytes() exceeds that size return
+ * MDCN_ERR_SCRATCH_LIMIT and enqueue nothing.  The call allocates and frees
+ * nothing, on the host or on the device.  All calls on one device share the
+ * buffer: calls that overlap in time on one device (different streams or
+ * threads) race; calls on one stream are ordered by the stream.  Nothing in the
+ * buffer has to survive between calls: each call rewrites every byte it reads. */
+#define MDCN_NOALLOC_SCRATCH_BYTES (64u << 20)
+int mdcn_forward_noalloc(const mdcn_params *p, void *hip_stream);
 
 /* Same work as mdcn_forward(), with HIP events recorded on `hip_stream` around
  * each stage; waits for the stream and reports milliseconds per stage:

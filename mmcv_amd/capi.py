@@ -12,9 +12,10 @@ LIB_PATH = os.path.join(_HERE, 'lib', 'libmdcn_hip.so')
 MDCN_F32, MDCN_F16, MDCN_BF16 = 0, 1, 2
 PATH_AUTO, PATH_FUSED, PATH_DIRECT = 0, 1, 2
 MDCN_OK = 0
+NOALLOC_SCRATCH_BYTES = 64 << 20
 
 EXPORTS = ('mdcn_abi_version', 'mdcn_set_pass_limits', 'mdcn_status_string', 'mdcn_output_size',
-           'mdcn_fused_eligible', 'mdcn_workspace_bytes', 'mdcn_forward',
+           'mdcn_fused_eligible', 'mdcn_workspace_bytes', 'mdcn_forward', 'mdcn_forward_noalloc',
            'mdcn_forward_timed', 'mdcn_mfma_probe', 'mdcn_pack_workspace_bytes', 'mdcn_pack_forward',
            'mdcn_pack_forward_timed', 'mdcn_backward_workspace_bytes', 'mdcn_backward')
 
@@ -65,6 +66,8 @@ def load():
         lib.mdcn_workspace_bytes.argtypes = [P]
         lib.mdcn_forward.restype = ctypes.c_int
         lib.mdcn_forward.argtypes = [P, ctypes.c_void_p]
+        lib.mdcn_forward_noalloc.restype = ctypes.c_int
+        lib.mdcn_forward_noalloc.argtypes = [P, ctypes.c_void_p]
         lib.mdcn_forward_timed.restype = ctypes.c_int
         lib.mdcn_forward_timed.argtypes = [P, ctypes.c_void_p,
                                            ctypes.POINTER(ctypes.c_float)]

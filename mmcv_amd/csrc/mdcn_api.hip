@@ -6,6 +6,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <mutex>
 #include <type_traits>
 
 #include "mdcn_common.h"
@@ -31,6 +32,29 @@ uint64_t g_fwd_pass_bytes = kMaxXtBytes;
 uint64_t g_bwd_pass_bytes = kBwdColGradCap;
 
 inline size_t align_up(size_t v) { return (v + kAlign - 1) / kAlign * kAlign; }
+
+// Scratch of mdcn_forward_noalloc(): the input copy and the packed weights of one
+// call, held by every device the library runs on until the process ends.  Host
+// code never uses the array's name as an address: scratch_of_current_device()
+// asks the runtime where the current device keeps its copy.
+static __device__ __align__(256) unsigned char scratch[MDCN_NOALLOC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices] = {nullptr};
+
+int scratch_of_current_device(void **out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return MDCN_ERR_LAUNCH;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void *ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return MDCN_ERR_LAUNCH;
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return MDCN_OK;
+}
 
 inline size_t elem_size(int dtype) { return dtype == MDCN_F32 ? 4 : 2; }
 
@@ -905,6 +929,7 @@ const char *mdcn_status_string(int status) {
     case MDCN_ERR_PATH: return "shape not covered by the fused path";
     case MDCN_ERR_TOO_LARGE: return "tensor too large for 32-bit device offsets";
     case MDCN_ERR_LAUNCH: return "HIP launch error";
+    case MDCN_ERR_SCRATCH_LIMIT: return "call needs more scratch than the library's built-in buffer holds";
     default: return "unknown status";
   }
 }
@@ -934,6 +959,23 @@ size_t mdcn_workspace_bytes(const mdcn_params *p) {
 
 int mdcn_forward(const mdcn_params *p, void *hip_stream) {
   return run(p, hip_stream, nullptr);
+}
+
+int mdcn_forward_noalloc(const mdcn_params *p, void *hip_stream) {
+  Geom g;
+  int rc = check_params(p, &g, true);
+  if (rc != MDCN_OK) return rc;
+  Plan pl;
+  rc = make_plan(p, g, &pl);
+  if (rc != MDCN_OK) return rc;
+  if (pl.xt_bytes + pl.wp_bytes > (size_t)MDCN_NOALLOC_SCRATCH_BYTES) return MDCN_ERR_SCRATCH_LIMIT;
+  void *ptr = nullptr;
+  rc = scratch_of_current_device(&ptr);
+  if (rc != MDCN_OK) return rc;
+  mdcn_params q = *p;
+  q.workspace = ptr;
+  q.workspace_bytes = (size_t)MDCN_NOALLOC_SCRATCH_BYTES;
+  return run(&q, hip_stream, nullptr);
 }
 
 int mdcn_mfma_probe(int dtype, int waves_per_simd, int zero_data, void *scratch, void *hip_stream, float *tflops) {
