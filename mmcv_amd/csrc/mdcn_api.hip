@@ -6,6 +6,8 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <cstdlib>
+#include <cstdio>
 #include <mutex>
 #include <type_traits>
 
@@ -14,6 +16,7 @@
 #include "mdcn_backward.h"
 #include "mdcn_backward_gemm.h"
 #include "mdcn_fused.h"
+#include "mdcn_fused2.h"
 #include "mdcn_oconv.h"
 #include "mdcn_prepass.h"
 
@@ -247,10 +250,24 @@ hipError_t launch_fused_ct(const FusedArgs &fa, bool unbordered, hipStream_t st)
   return hipGetLastError();
 }
 
+// 256-channel tiles: the eight-wave kernel of mdcn_fused2.h
+template <typename E>
+hipError_t launch_fused2(const FusedArgs &fa, bool unbordered, hipStream_t st) {
+  const int total_wg = fa.n_ptiles * fa.n_ctiles * fa.g.G;
+  const int per_xcd = std::max(1, std::min((total_wg + 7) / 8, num_cus() / 8));
+  if (unbordered)
+    hipLaunchKernelGGL((fused2_kernel<E, kTapsSmall, true>), dim3(per_xcd * 8), dim3(kF2Threads), 0, st, fa);
+  else
+    hipLaunchKernelGGL((fused2_kernel<E, kTapsSmall, false>), dim3(per_xcd * 8), dim3(kF2Threads), 0, st, fa);
+  return hipGetLastError();
+}
+
 template <typename E, int CT>
 hipError_t launch_fused_tm(const FusedArgs &fa, bool ub, hipStream_t st) {
   const bool small = fa.g.taps <= kTapsSmall;
   if constexpr (CT == 256) {  // (pick_ct never pairs the 256-wide tile with the large table)
+    static const bool v1 = getenv("MDCN_FUSED_V1") != nullptr;
+    if (!v1 && fa.g.DG == 1) return launch_fused2<E>(fa, ub, st);
     return fa.g.DG > 1 ? launch_fused_ct<E, CT, kTapsSmall, true>(fa, ub, st)
                        : launch_fused_ct<E, CT, kTapsSmall, false>(fa, ub, st);
   } else {
@@ -432,6 +449,25 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
         fa.om = dense_view((const E *)p->offset + (size_t)n0 * g.DG * 2 * g.taps * plane_out,
                            p->mask ? (const E *)p->mask + (size_t)n0 * g.DG * g.taps * plane_out : nullptr, g);
       }
+      fa.prof = nullptr;
+#if defined(MDCN_F2_PROFILE) && MDCN_F2_PROFILE
+      {  // profiling build: phase sums land behind the packed weights (the workspace is over-allocated by the harness)
+        static void *prof_buf = nullptr;
+        if (!prof_buf) (void)hipMalloc(&prof_buf, 4096);
+        fa.prof = prof_buf;
+        static bool once = (atexit([]() {
+          long long h[128];
+          if (hipMemcpy(h, prof_buf, sizeof(h), hipMemcpyDeviceToHost) == hipSuccess)
+            for (int b = 0; b < 2; ++b)
+              for (int w = 0; w < 8; ++w) {
+                printf("prof block %d wave %d:", b, w);
+                for (int i = 0; i < 8; ++i) printf(" %lld", h[(b * 8 + w) * 8 + i]);
+                printf("\n");
+              }
+        }), true);
+        (void)once;
+      }
+#endif
       fa.bias = p->bias;
       fa.out = (E *)p->output + (size_t)n0 * g.Cout * plane_out;
       fa.total_px = (long)gc.N * plane_out;

@@ -71,9 +71,31 @@ struct FusedArgs {
   uint32_t px_bytes;   // bytes between horizontally adjacent pixels: kRowB (copy) or Cin * sizeof(E)
   uint32_t slab_bytes; // bytes between channel slabs of one pixel: plane_px * kRowB (copy) or kRowB
   uint32_t img_bytes;  // bytes between images
+  void *prof;          // per-phase clock sums of a profiling build, else unused
 };
 
 typedef __attribute__((address_space(3))) void *lptr_t;
+
+// Byte offset, inside one image of the input copy, of the upper left corner of
+// a sample's 2 x 2 block (slab 0).
+// Zero-bordered copy: +1 in both coordinates (y0, x0 >= -1 when the position is
+// inside).  A position outside (-1,H) x (-1,W) adds nothing in the reference
+// (mmcv/ops/csrc/pytorch/cpu/modulated_deform_conv.cpp:160-164): its block is
+// put on padded pixels (0, Wp-1), (1, 0), (1, Wp-1), (2, 0) -- four border
+// pixels that follow one another in memory the way a block's corners do -- so
+// that the four loads return stored zeros whatever the image holds.
+// Channels-last input read in place: the block is moved into the image and the
+// weights of the corners that were outside become zero (clamp_to_image; call
+// before the weights are taken from `s`).
+template <bool UNBORDERED>
+__device__ __forceinline__ uint32_t corner_offset(TapSample &s, const Geom &g, const FusedArgs &a) {
+  if (UNBORDERED) {
+    clamp_to_image(s, g.H, g.W);
+    return (uint32_t)s.y0 * a.row_bytes + (uint32_t)s.x0 * a.px_bytes;
+  }
+  return s.inside ? (uint32_t)(s.y0 + 1) * a.row_bytes + (uint32_t)(s.x0 + 1) * (uint32_t)kRowB
+                  : (uint32_t)(g.Wp - 1) * (uint32_t)kRowB;
+}
 
 template <typename E>
 struct ElemTraits;
@@ -438,15 +460,7 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
                 make_tap_sample(tb_ho * g.sh - g.ph + ti * g.dh, tb_wo * g.sw - g.pw + tj * g.dw,
                                 to_f32(rdy[i]), to_f32(rdx[i]), mask_value<E>(rm[i], a.om.logit), g.H, g.W);
             // byte offset of the upper left corner, slab 0 of image tb_n
-            uint32_t pix;
-            if (UNBORDERED) {
-              clamp_to_image(sm, g.H, g.W);
-              pix = (uint32_t)tb_n * a.img_bytes + (uint32_t)sm.y0 * a.row_bytes + (uint32_t)sm.x0 * a.px_bytes;
-            } else {
-              // +1: coordinates in the zero-bordered copy (y0, x0 >= -1 when inside,
-              // 0 with zero weights otherwise)
-              pix = (uint32_t)tb_n * a.img_bytes + (uint32_t)(sm.y0 + 1) * a.row_bytes + (uint32_t)(sm.x0 + 1) * kRowB;
-            }
+            uint32_t pix = (uint32_t)tb_n * a.img_bytes + corner_offset<UNBORDERED>(sm, g, a);
             uint32_t tw[4];
             TR::table_weights(sm, tw);
             if (!tb_valid) {
