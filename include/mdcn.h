@@ -36,7 +36,11 @@ enum mdcn_dtype { MDCN_F32 = 0, MDCN_F16 = 1, MDCN_BF16 = 2 };
 enum mdcn_path {
   MDCN_PATH_AUTO = 0,   /* fused MFMA kernel when the shape allows, else direct */
   MDCN_PATH_FUSED = 1,  /* fused implicit-GEMM MFMA kernel; error if not eligible */
-  MDCN_PATH_DIRECT = 2  /* one thread per output element; any shape */
+  MDCN_PATH_DIRECT = 2, /* one thread per output element; any shape */
+  MDCN_PATH_FUSED_SPLIT = 3 /* forward only: as MDCN_PATH_FUSED, but always the fused kernel with specialised
+                               producer / consumer wavefronts (what fp32 tensors, several deformable groups and
+                               tiles narrower than 256 channels run anyway), never the eight-wave streaming
+                               kernel that 16-bit 256-channel tiles get by default; for comparisons and tests */
 };
 
 enum mdcn_status {

@@ -13,13 +13,16 @@
 #include <string>
 #include <vector>
 
+#include <atomic>
+
 #include "mdcn.h"
 
 namespace {
 
 using at::Tensor;
 
-int g_path = MDCN_PATH_AUTO;
+// device path of every op of this module (set_path); read once per call
+std::atomic<int> g_path{MDCN_PATH_AUTO};
 
 std::string device_str(const at::Device &d) {
   std::string s = c10::DeviceTypeName(d.type(), /*lower_case=*/true);
@@ -84,7 +87,7 @@ void prepare(Prepared &pr, const Tensor &input, const Tensor &weight,
   mdcn_params &p = pr.p;
   p = mdcn_params{};
   p.dtype = mdcn_dtype_of(input);
-  p.path = g_path;
+  p.path = g_path.load();
   p.N = (int)batch; p.Cin = (int)channels; p.H = (int)height; p.W = (int)width;
   p.Cout = (int)channels_out; p.kh = kernel_h; p.kw = kernel_w;
   p.sh = stride_h; p.sw = stride_w; p.ph = pad_h; p.pw = pad_w;
@@ -120,7 +123,7 @@ void prepare(Prepared &pr, const Tensor &input, const Tensor &weight,
   if (!input.is_contiguous() && input.is_contiguous(at::MemoryFormat::ChannelsLast)) {
     p.input = input.data_ptr();
     p.input_nhwc = 1;
-    if (!mdcn_fused_eligible(&p) || g_path == MDCN_PATH_DIRECT) {
+    if (!mdcn_fused_eligible(&p) || p.path == MDCN_PATH_DIRECT) {
       p.input = nullptr;
       p.input_nhwc = 0;
     }
@@ -219,7 +222,7 @@ std::vector<double> modulated_deform_conv_pack_forward(
   mdcn_pack_params pp{};
   mdcn_params &p = pp.conv;
   p.dtype = mdcn_dtype_of(input);
-  p.path = g_path;
+  p.path = g_path.load();
   p.N = (int)batch; p.Cin = (int)channels; p.H = (int)input.size(2); p.W = (int)input.size(3);
   p.Cout = (int)channels_out; p.kh = kernel_h; p.kw = kernel_w;
   p.sh = stride_h; p.sw = stride_w; p.ph = pad_h; p.pw = pad_w;
@@ -331,7 +334,7 @@ void deform_conv_forward(Tensor input, Tensor weight, Tensor offset, Tensor outp
   }
   mdcn_params p{};
   p.dtype = mdcn_dtype_of(input);
-  p.path = g_path;
+  p.path = g_path.load();
   p.N = (int)batch; p.Cin = (int)planes; p.H = (int)input.size(2); p.W = (int)input.size(3);
   p.Cout = (int)weight.size(0); p.kh = kH; p.kw = kW;
   p.sh = dH; p.sw = dW; p.ph = padH; p.pw = padW; p.dh = dilationH; p.dw = dilationW;
@@ -403,6 +406,7 @@ void run_backward(const char *op, const Tensor &input, const Tensor &weight, con
   p.Cout = (int)weight.size(0); p.kh = kernel_h; p.kw = kernel_w;
   p.sh = stride_h; p.sw = stride_w; p.ph = pad_h; p.pw = pad_w; p.dh = dilation_h; p.dw = dilation_w;
   p.groups = group; p.dgroups = deformable_group;
+  p.path = g_path.load();
   int32_t Ho = 0, Wo = 0;
   int rc = mdcn_output_size(&p, &Ho, &Wo);
   TORCH_CHECK(rc == MDCN_OK, op, ": ", mdcn_status_string(rc));
@@ -562,9 +566,11 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("dilation_h"), py::arg("dilation_w"), py::arg("group"),
         py::arg("deformable_group"), py::arg("with_bias"));
   m.def("set_path", [](int path) {
-          TORCH_CHECK(path >= MDCN_PATH_AUTO && path <= MDCN_PATH_DIRECT, "path must be 0 (auto), 1 (fused) or 2 (direct)");
-          g_path = path;
-        }, "choose the device path: 0 auto, 1 fused MFMA kernel, 2 direct kernel", py::arg("path"));
-  m.def("get_path", []() { return g_path; });
+          TORCH_CHECK(path >= MDCN_PATH_AUTO && path <= MDCN_PATH_FUSED_SPLIT,
+                      "path must be 0 (auto), 1 (fused), 2 (direct) or 3 (fused, specialised-wave kernel only)");
+          g_path.store(path);
+        }, "choose the device path of forward and backward: 0 auto, 1 fused / matrix-core kernels, 2 direct kernels, "
+           "3 fused with the specialised-wave forward kernel", py::arg("path"));
+  m.def("get_path", []() { return g_path.load(); });
   m.def("abi_version", []() { return mdcn_abi_version(); });
 }

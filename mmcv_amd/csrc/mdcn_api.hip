@@ -6,7 +6,6 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
-#include <cstdlib>
 #include <cstdio>
 #include <mutex>
 #include <type_traits>
@@ -150,7 +149,7 @@ struct PackExtra {
 
 int make_plan(const mdcn_params *p, const Geom &g, Plan *pl) {
   const bool ok = fused_ok(p, g);
-  if (p->path == MDCN_PATH_FUSED && !ok) return MDCN_ERR_PATH;
+  if ((p->path == MDCN_PATH_FUSED || p->path == MDCN_PATH_FUSED_SPLIT) && !ok) return MDCN_ERR_PATH;
   if (p->input_nhwc && (!ok || p->path == MDCN_PATH_DIRECT)) return MDCN_ERR_PATH;  // in-place reads: fused kernel only
   pl->fused = ok && p->path != MDCN_PATH_DIRECT;
   pl->CT = pl->KC = pl->n_ctiles = pl->slabs = pl->n_chunk = 0;
@@ -188,7 +187,7 @@ int make_pack_plan(const mdcn_pack_params *pp, const Geom &g, Plan *pl) {
   if (pp->offset_weight) {
     if (pl->fused) {
       if (pl->CO_pad > 128) {  // accumulator blocks of the conv_offset kernel
-        if (p->path == MDCN_PATH_FUSED) return MDCN_ERR_PATH;
+        if (p->path == MDCN_PATH_FUSED || p->path == MDCN_PATH_FUSED_SPLIT) return MDCN_ERR_PATH;
         pl->fused = false;
         pl->xt_bytes = pl->wp_bytes = 0;
       } else {
@@ -256,18 +255,20 @@ hipError_t launch_fused2(const FusedArgs &fa, bool unbordered, hipStream_t st) {
   const int total_wg = fa.n_ptiles * fa.n_ctiles * fa.g.G;
   const int per_xcd = std::max(1, std::min((total_wg + 7) / 8, num_cus() / 8));
   if (unbordered)
-    hipLaunchKernelGGL((fused2_kernel<E, kTapsSmall, true>), dim3(per_xcd * 8), dim3(kF2Threads), 0, st, fa);
+    hipLaunchKernelGGL((fused2_kernel<E, true>), dim3(per_xcd * 8), dim3(kF2Threads), 0, st, fa);
   else
-    hipLaunchKernelGGL((fused2_kernel<E, kTapsSmall, false>), dim3(per_xcd * 8), dim3(kF2Threads), 0, st, fa);
+    hipLaunchKernelGGL((fused2_kernel<E, false>), dim3(per_xcd * 8), dim3(kF2Threads), 0, st, fa);
   return hipGetLastError();
 }
 
 template <typename E, int CT>
-hipError_t launch_fused_tm(const FusedArgs &fa, bool ub, hipStream_t st) {
+hipError_t launch_fused_tm(const FusedArgs &fa, bool ub, bool split, hipStream_t st) {
   const bool small = fa.g.taps <= kTapsSmall;
   if constexpr (CT == 256) {  // (pick_ct never pairs the 256-wide tile with the large table)
-    static const bool v1 = getenv("MDCN_FUSED_V1") != nullptr;
-    if (!v1 && fa.g.DG == 1) return launch_fused2<E>(fa, ub, st);
+    if constexpr (sizeof(E) == 2) {
+      const int nk_pad = (fa.slabs * fa.g.taps + kF2Unroll - 1) / kF2Unroll * kF2Unroll;
+      if (!split && fa.g.DG == 1 && nk_pad >= kF2MinSteps) return launch_fused2<E>(fa, ub, st);
+    }
     return fa.g.DG > 1 ? launch_fused_ct<E, CT, kTapsSmall, true>(fa, ub, st)
                        : launch_fused_ct<E, CT, kTapsSmall, false>(fa, ub, st);
   } else {
@@ -280,11 +281,11 @@ hipError_t launch_fused_tm(const FusedArgs &fa, bool ub, hipStream_t st) {
 }
 
 template <typename E>
-hipError_t launch_fused(const FusedArgs &fa, int CT, bool ub, hipStream_t st) {
+hipError_t launch_fused(const FusedArgs &fa, int CT, bool ub, bool split, hipStream_t st) {
   switch (CT) {
-    case 64: return launch_fused_tm<E, 64>(fa, ub, st);
-    case 128: return launch_fused_tm<E, 128>(fa, ub, st);
-    default: return launch_fused_tm<E, 256>(fa, ub, st);
+    case 64: return launch_fused_tm<E, 64>(fa, ub, split, st);
+    case 128: return launch_fused_tm<E, 128>(fa, ub, split, st);
+    default: return launch_fused_tm<E, 256>(fa, ub, split, st);
   }
 }
 
@@ -478,7 +479,7 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
       fa.plane_px = g.Hp * g.Wp;
       fa.out_vec_ok = (plane_out % (long)(16 / es) == 0) && (((uintptr_t)fa.out % 16) == 0);
       tic();
-      if (launch_fused<E>(fa, pl.CT, nhwc, st) != hipSuccess) rc = MDCN_ERR_LAUNCH;
+      if (launch_fused<E>(fa, pl.CT, nhwc, p->path == MDCN_PATH_FUSED_SPLIT, st) != hipSuccess) rc = MDCN_ERR_LAUNCH;
       toc(2);
     }
   }
@@ -578,7 +579,7 @@ void make_bwd_plan(const mdcn_bwd_params *bp, const Geom &g, BwdPlan *pl) {
   pl->P_pad = 0;
   pl->R = pl->sR = -1;
   pl->WH = pl->WW = pl->sWH = pl->sWW = 0;
-  const int path = bp->conv.path;
+  const int path = bp->conv.path == MDCN_PATH_FUSED_SPLIT ? MDCN_PATH_FUSED : bp->conv.path;
   if (path == MDCN_PATH_DIRECT || g.taps > kBwdTapsMax) return;
   const bool forced = path == MDCN_PATH_FUSED;
   const size_t plane_out = (size_t)g.Ho * g.Wo;
@@ -936,7 +937,7 @@ int check_bwd(const mdcn_bwd_params *bp, Geom *g, bool need_ptrs) {
   if (data != (bp->grad_offset != nullptr)) return MDCN_ERR_NULL;
   if (p->mask ? (data != (bp->grad_mask != nullptr)) : (bp->grad_mask != nullptr)) return MDCN_ERR_NULL;
   if ((uint64_t)g->N * g->DG * g->taps > 0x7fffffffull) return MDCN_ERR_TOO_LARGE;
-  if (p->path == MDCN_PATH_FUSED) {  // asked for the tiled kernels: the shape must allow them
+  if (p->path == MDCN_PATH_FUSED || p->path == MDCN_PATH_FUSED_SPLIT) {  // asked for the tiled kernels: the shape must allow them
     BwdPlan pl;
     make_bwd_plan(bp, *g, &pl);
     if ((data && !pl.tiled && !pl.gemm) || (!data && bp->grad_weight && !pl.wgemm)) return MDCN_ERR_PATH;

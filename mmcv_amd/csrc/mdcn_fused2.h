@@ -1,13 +1,13 @@
-// Fused DCNv2 forward for gfx950, 256-channel output tiles: the same implicit
-// GEMM, tile shapes, LDS layouts and input copy as mdcn_fused.h, with another
-// division of labour.
+// Fused DCNv2 forward for gfx950, 16-bit tensors, 256-channel output tiles, one
+// deformable group: the same implicit GEMM, tile shapes, LDS tile layouts and
+// input copy as mdcn_fused.h, with another division of labour.
 //
 // Eight wavefronts, all alike.  Per K step (128 bytes of channels of one tap)
 // every wave
-//   * "produces" 16 of the tile's 128 pixels: waits for the gather it issued two
-//     steps earlier (4 corners x 2 x 16 bytes per lane, held in registers),
+//   * "produces" 16 of the tile's 128 pixels: waits for the gather it issued
+//     three steps earlier (4 corners x 2 x 16 bytes per lane, held in registers),
 //     blends the corners into 2 x 16 bytes of the sample tile, writes them to
-//     LDS and refills the registers with the gather of the step after next;
+//     LDS and refills the registers with the gather of three steps ahead;
 //   * issues its share (4 x 1 KiB) of the direct-to-LDS copy of the weight tile
 //     of the next step;
 //   * "consumes": 16 MFMAs (32x32x16) on its 64 pixel x 64 channel part of the
@@ -15,24 +15,31 @@
 // One workgroup barrier per step.  The two waves that share a SIMD run the two
 // halves in opposite order (waves 0-3: MFMA, produce, barrier; waves 4-7: MFMA,
 // barrier, produce -- the same instruction stream with the barrier at another
-// place), so that the matrix pipe of a SIMD works for one wave while its
-// vector ALU blends for the other.
+// place), so that one wave of a SIMD computes while the other waits for memory.
 //
-// The blend itself runs on the matrix pipe for 16-bit types: one
-// v_mfma_f32_4x4x4 (16 blocks of 4x4x4) takes the four lanes that serve one
-// pixel as one block, the lane's 4 channels as a column of B and
-// (corner weight) x identity as A, so four instructions -- one per corner --
-// accumulate the bilinear sum of 4 channels in fp32 without unpacking the
-// 16-bit values on the vector ALU (which would otherwise be the busiest unit of
-// the kernel).  fp32 tensors blend with FMAs.
+// The produce side streams across the tiles of a workgroup: its three cursors
+// (gather, blend, weight copy) walk one sequence of steps -- tile after tile,
+// each tile's step count padded to a multiple of six so that register sets,
+// sample tiles and ring slots are addressed statically -- and step over a tile
+// boundary three, zero and one step ahead of the consume side, so the memory
+// pipeline never drains between tiles.  The (pixel, tap) table exists twice;
+// the next tile's is built during the second round of the current tile's K
+// loop.  At the end of a tile a wave stores its accumulators straight from
+// registers (the two halves of the wave exchange packed pixel pairs with
+// v_permlane32_swap, after which a lane holds 16 bytes of one channel's row).
 //
 // All vector-memory traffic of the K loop is issued from inline assembly and
-// waited for with explicit counts: a wave has 2 x 8 gather loads and the weight
+// waited for with explicit counts: a wave has 3 x 8 gather loads and the weight
 // copies of up to three steps in flight, and the compiler's own bookkeeping
 // would drain them at every use.  Per wave and K step the order of issue is
 // fixed: kWD weight copies, then 8 gather loads (two groups of four, each group
 // issued right after the blend that frees its registers), which makes the
 // number of younger operations at every wait a constant.
+//
+// Build-time switches for measurements (all 0 in the product): MDCN_F2_ABLATE
+// (bit 0 no gathers, 1 no weight copies, 2 no blend, 3 no MFMA), MDCN_F2_PROFILE
+// (per-phase clock sums of two workgroups), MDCN_F2_BLEND 0 (bf16 blend on the
+// vector ALU instead of the matrix pipe).
 #pragma once
 
 #include "mdcn_fused.h"
@@ -61,8 +68,10 @@ constexpr int kF2VmBar = 2 * kF2GL + kF2WD;
 static_assert(kF2VmBlend < 64 && kF2VmBar < 64, "vmcnt holds 6 bits");
 static_assert(kF2Unroll % kF2Sets == 0 && kF2Unroll % 2 == 0 && kF2Unroll % kF2Slots == 0, "static indices");
 
-constexpr size_t fused2_lds_bytes(int tmax) {
-  return (size_t)2 * kPT * kRowB + (size_t)kF2Slots * kF2CT * kRowB + (size_t)kPT * tmax * 20;
+constexpr int kF2Taps = kTapsSmall;    // table capacity (kh * kw)
+constexpr int kF2MinSteps = 18;        // padded steps per tile the streaming needs (the next table is built in round 2)
+constexpr size_t fused2_lds_bytes() {
+  return (size_t)2 * kPT * kRowB + (size_t)kF2Slots * kF2CT * kRowB + (size_t)2 * kPT * kF2Taps * 12;
 }
 
 // 16 bytes per lane from `base` (two SGPRs) + 32-bit byte offset + immediate
@@ -94,17 +103,29 @@ constexpr size_t fused2_lds_bytes(int tmax) {
 typedef __attribute__((address_space(3))) u32x4 *lds_u32x4_ptr;
 static_assert(kF2WD == 4, "issue_weights spells out four copies");
 
-// Blend of one 16-byte chunk (8 or 4 channels) from the same chunk at the four
-// corners.  prep() turns a table entry into what run() needs, once per step.
+// Blend of one 16-byte chunk (8 channels) from the same chunk at the four
+// corners.  The table keeps the four mask-scaled bilinear weights as two words of
+// E pairs, (w00, w01) and (w10, w11); prep() turns them into what run() needs,
+// once per step.
 template <typename E>
 struct Blend2;
 
-template <typename E>
-struct Blend2Half {
+#ifndef MDCN_F2_BLEND
+#define MDCN_F2_BLEND 1
+#endif
+#if MDCN_F2_BLEND == 1
+// bf16 on the matrix pipe: one v_mfma_f32_4x4x4 (16 blocks of 4x4x4) takes the four
+// lanes that serve one pixel as one block, a lane's 4 channels (two words) as a
+// column of B and (corner weight) x identity as A -- lane q of the block holds row
+// q: the weight at K position q, zeros elsewhere -- so four instructions, one per
+// corner, accumulate the bilinear sum of 4 channels in fp32 without unpacking the
+// 16-bit values on the vector ALU.
+template <>
+struct Blend2<bf16_t> {
   struct Wt { u32x2 a[4]; };
-  // sh, m0, m1 depend on the lane's place q among the four lanes of its pixel:
-  // the corner weight sits at K position q of the lane's row of A, zeros elsewhere
-  static __device__ __forceinline__ Wt prep(const uint4 &tw, uint32_t sh, uint32_t m0, uint32_t m1) {
+  static __device__ __forceinline__ Wt prep(const uint2 &tw, int q) {
+    const uint32_t sh = (uint32_t)(q & 1) * 16u;
+    const uint32_t m0 = q < 2 ? 0xffffffffu : 0u, m1 = ~m0;
     const uint32_t c[4] = {tw.x & 0xffffu, tw.x >> 16, tw.y & 0xffffu, tw.y >> 16};
     Wt w;
 #pragma unroll
@@ -115,55 +136,37 @@ struct Blend2Half {
     }
     return w;
   }
+  static __device__ __forceinline__ f32x4 mma4(const u32x2 &a, const u32x2 &b, const f32x4 &c) {
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, a), __builtin_bit_cast(s16x4, b), c, 0, 0, 0);
+  }
   static __device__ __forceinline__ u32x4 run(const u32x4 (&v)[4], const Wt &w) {
     f32x4 d0 = {0.f, 0.f, 0.f, 0.f}, d1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
       const u32x2 b0 = {v[c].x, v[c].y}, b1 = {v[c].z, v[c].w};
-      d0 = Blend2<E>::mma4(w.a[c], b0, d0);
-      d1 = Blend2<E>::mma4(w.a[c], b1, d1);
+      d0 = mma4(w.a[c], b0, d0);
+      d1 = mma4(w.a[c], b1, d1);
     }
     u32x4 o;
-    o.x = ElemTraits<E>::pack2(d0[0], d0[1]);
-    o.y = ElemTraits<E>::pack2(d0[2], d0[3]);
-    o.z = ElemTraits<E>::pack2(d1[0], d1[1]);
-    o.w = ElemTraits<E>::pack2(d1[2], d1[3]);
+    o.x = ElemTraits<bf16_t>::pack2(d0[0], d0[1]);
+    o.y = ElemTraits<bf16_t>::pack2(d0[2], d0[3]);
+    o.z = ElemTraits<bf16_t>::pack2(d1[0], d1[1]);
+    o.w = ElemTraits<bf16_t>::pack2(d1[2], d1[3]);
     return o;
-  }
-  static __device__ __forceinline__ void table_weights(const TapSample &s, uint32_t (&tw)[4]) {
-    Half16Traits<E>::table_weights(s, tw);  // (w00, w01), (w10, w11) rounded to E
-  }
-};
-
-#ifndef MDCN_F2_BLEND_MFMA
-#define MDCN_F2_BLEND_MFMA 0
-#endif
-#if MDCN_F2_BLEND_MFMA
-template <>
-struct Blend2<bf16_t> : Blend2Half<bf16_t> {
-  static __device__ __forceinline__ f32x4 mma4(const u32x2 &a, const u32x2 &b, const f32x4 &c) {
-    typedef short s16x4 __attribute__((ext_vector_type(4)));
-    return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, a), __builtin_bit_cast(s16x4, b), c, 0, 0, 0);
-  }
-};
-
-template <>
-struct Blend2<f16_t> : Blend2Half<f16_t> {
-  static __device__ __forceinline__ f32x4 mma4(const u32x2 &a, const u32x2 &b, const f32x4 &c) {
-    return __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(f16x4, a), __builtin_bit_cast(f16x4, b), c, 0, 0, 0);
   }
 };
 #else
 // bf16 on the vector ALU: a 32-bit word holds two channels; shifting / masking
 // turns each into an fp32 value exactly, the four corners are summed with fp32
-// FMAs (fp32 weights) and the pair is rounded to bf16 once.
+// FMAs and the pair is rounded to bf16 once.
 template <>
 struct Blend2<bf16_t> {
   struct Wt { float w[4]; };
-  static __device__ __forceinline__ Wt prep(const uint4 &tw, uint32_t, uint32_t, uint32_t) {
+  static __device__ __forceinline__ Wt prep(const uint2 &tw, int) {
     Wt w;
-    w.w[0] = __uint_as_float(tw.x); w.w[1] = __uint_as_float(tw.y);
-    w.w[2] = __uint_as_float(tw.z); w.w[3] = __uint_as_float(tw.w);
+    w.w[0] = __uint_as_float(tw.x << 16); w.w[1] = __uint_as_float(tw.x & 0xffff0000u);
+    w.w[2] = __uint_as_float(tw.y << 16); w.w[3] = __uint_as_float(tw.y & 0xffff0000u);
     return w;
   }
   static __device__ __forceinline__ u32x4 run(const u32x4 (&v)[4], const Wt &w) {
@@ -181,18 +184,21 @@ struct Blend2<bf16_t> {
     }
     return o;
   }
-  static __device__ __forceinline__ void table_weights(const TapSample &s, uint32_t (&tw)[4]) {
-    ElemTraits<float>::table_weights(s, tw);
-  }
 };
+#endif
 
-// fp16 has packed arithmetic: see ElemTraits<f16_t>::blend
+// fp16 has packed arithmetic: every corner weight in both halves of a word, one
+// v_pk_mul_f16 and three v_pk_fma_f16 per two channels (the blend then rounds to
+// fp16 after every corner instead of once).
 template <>
 struct Blend2<f16_t> {
   struct Wt { uint4 w; };
-  static __device__ __forceinline__ Wt prep(const uint4 &tw, uint32_t, uint32_t, uint32_t) {
+  static __device__ __forceinline__ Wt prep(const uint2 &tw, int) {
     Wt w;
-    w.w = tw;
+    w.w.x = (tw.x & 0xffffu) | (tw.x << 16);
+    w.w.y = (tw.x >> 16) | (tw.x & 0xffff0000u);
+    w.w.z = (tw.y & 0xffffu) | (tw.y << 16);
+    w.w.w = (tw.y >> 16) | (tw.y & 0xffff0000u);
     return w;
   }
   static __device__ __forceinline__ u32x4 run(const u32x4 (&v)[4], const Wt &w) {
@@ -200,55 +206,26 @@ struct Blend2<f16_t> {
                                              __builtin_bit_cast(uint4, v[2]), __builtin_bit_cast(uint4, v[3]), w.w);
     return __builtin_bit_cast(u32x4, r);
   }
-  static __device__ __forceinline__ void table_weights(const TapSample &s, uint32_t (&tw)[4]) {
-    ElemTraits<f16_t>::table_weights(s, tw);
-  }
-};
-#endif
-
-template <>
-struct Blend2<float> {
-  struct Wt { float w[4]; };
-  static __device__ __forceinline__ Wt prep(const uint4 &tw, uint32_t, uint32_t, uint32_t) {
-    Wt w;
-    w.w[0] = __uint_as_float(tw.x); w.w[1] = __uint_as_float(tw.y);
-    w.w[2] = __uint_as_float(tw.z); w.w[3] = __uint_as_float(tw.w);
-    return w;
-  }
-  static __device__ __forceinline__ u32x4 run(const u32x4 (&v)[4], const Wt &w) {
-    u32x4 o;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      float acc = w.w[0] * __uint_as_float(v[0][j]);
-      acc = acc + w.w[1] * __uint_as_float(v[1][j]);
-      acc = acc + w.w[2] * __uint_as_float(v[2][j]);
-      acc = acc + w.w[3] * __uint_as_float(v[3][j]);
-      o[j] = __float_as_uint(acc);
-    }
-    return o;
-  }
-  static __device__ __forceinline__ void table_weights(const TapSample &s, uint32_t (&tw)[4]) {
-    ElemTraits<float>::table_weights(s, tw);
-  }
 };
 
-template <typename E, int TMAX, bool UNBORDERED>
+template <typename E, bool UNBORDERED>
 __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
   using TR = ElemTraits<E>;
   using BL = Blend2<E>;
+  static_assert(sizeof(E) == 2, "16-bit element types");
   constexpr int PT = kPT;
   constexpr int CT = kF2CT;
   constexpr int KC = TR::KC;
-  constexpr int ES = (int)sizeof(E);
-  constexpr int NS = kF2Sets;
+  constexpr int TMAX = kF2Taps;
+  constexpr int TBL = PT * TMAX;               // entries of one table
   constexpr int TPT = (TMAX + 3) / 4;          // table entries per lane and build
   constexpr int NB = 2, MB = 2;                // 32 x 32 accumulator blocks per wave: pixels x channels
   constexpr uint32_t kXTile = PT * kRowB, kWTile = CT * kRowB;
 
   __shared__ uint4 Xs[2][PT * kRowChunks];               // sample tiles
   __shared__ uint4 Ws[kF2Slots][CT * kRowChunks];        // weight tiles
-  __shared__ uint32_t tpix[PT * TMAX];                   // (pixel, tap) table, [tap][PT]: corner byte offset
-  __shared__ uint4 tws[PT * TMAX];                       // ... and the blend weights
+  __shared__ uint32_t tpix[2][TBL];                      // (pixel, tap) tables, [tap][PT]: corner byte offset
+  __shared__ uint2 tws[2][TBL];                          // ... and the blend weights
 
   const Geom &g = a.g;
   const int taps = g.taps;
@@ -256,14 +233,12 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
   const int nk_pad = (nk + kF2Unroll - 1) / kF2Unroll * kF2Unroll;
   const int plane_out = g.Ho * g.Wo;
   const int total_px = (int)a.total_px;
-  const int spd = g.ch_per_dg / KC;  // slabs per deformable group
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   // waves 4..7 run the produce half of a step after its barrier (see above)
   const bool late = wave >= 4;
-  const int ahead = late ? 2 : 1;
 
   const uint32_t lds_x = (uint32_t)(uintptr_t)(lptr_t)(&Xs[0][0]);
   const uint32_t lds_w = (uint32_t)(uintptr_t)(lptr_t)(&Ws[0][0]);
@@ -271,8 +246,6 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
   // ---- produce role: lane serves 16-byte chunks q and q + 4 of pixel pl
   const int q = lane & 3;
   const int pl = wave * 16 + (lane >> 2);
-  const uint32_t bsh = (uint32_t)(q & 1) * 16u;
-  const uint32_t bm0 = q < 2 ? 0xffffffffu : 0u, bm1 = ~bm0;
   const uint32_t xw0 = lds_x + (uint32_t)tile_chunk(pl, q) * 16u;       // where its two chunks go in X[0]
   const uint32_t xw1 = lds_x + (uint32_t)tile_chunk(pl, q + 4) * 16u;
   const unsigned char *xt = (const unsigned char *)a.xt;
@@ -292,53 +265,55 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
   const uint32_t wlane = (uint32_t)(wave * kF2WD) * 1024u +
                          (uint32_t)((lane >> 3) * kRowB + (((lane & 7) ^ swz(lane >> 3)) * 16));
 
-  // XCD-aware persistent schedule (as in fused_kernel)
+  // XCD-aware persistent schedule (as in fused_kernel): this workgroup's tiles
+  // are first, first + stride, ... below tile_end
   const int total_tiles = a.n_ptiles * a.n_ctiles * g.G;
   const int xcd = (int)(blockIdx.x & 7);
-  const int wg_in_xcd = (int)(blockIdx.x >> 3);
-  const int wgs_per_xcd = (int)(gridDim.x >> 3);
+  const int stride = (int)(gridDim.x >> 3);
   const int chunk = (total_tiles + 7) >> 3;
+  const int first = xcd * chunk + (int)(blockIdx.x >> 3);
   const int tile_end = min((xcd + 1) * chunk, total_tiles);
+  if (first >= tile_end) return;
+  const int T = (tile_end - first + stride - 1) / stride;
 
-  // ---- state of the tile whose gathers are being issued
-  int ctile = 0, grp = 0, p0 = 0, ch0 = 0, slab0 = 0;
-  int tb_n = 0, tb_ho = 0, tb_wo = 0, tb_rem = 0;
-  bool tb_valid = false;
-  const int tb_pl = tid & (PT - 1);
-  const unsigned char *wp_tile = nullptr;
-  StepCursor cur;   // the next step whose gather is issued
-  StepCursor bcur;  // the next step to blend
-  auto set_tile = [&](int tile) {
-    int L = tile;
+  auto decode = [&](int t, int &ctile, int &grp, int &p0) {
+    int L = first + t * stride;
     ctile = L % a.n_ctiles;
     L /= a.n_ctiles;
     grp = L % g.G;
     p0 = (L / g.G) * PT;
-    ch0 = grp * g.cin_g;
-    slab0 = ch0 / KC;
-    // table: lane serves pixel tid % 128, taps tid / 128 + 4 i
+  };
+  auto weights_of = [&](int t) {
+    int ctile, grp, p0;
+    decode(t, ctile, grp, p0);
+    return (const unsigned char *)a.wp + ((size_t)(grp * a.n_ctiles + ctile) * nk) * (size_t)kWTile;
+  };
+  auto slab0_of = [&](int t) {
+    int ctile, grp, p0;
+    decode(t, ctile, grp, p0);
+    return grp * g.cin_g / KC;
+  };
+
+  // ---- (pixel, tap) table of tile t into buffer t % 2: lane serves pixel tid % 128, taps tid / 128 + 4 i
+  auto build_table = [&](int t) {
+    // (opaque to the optimiser: the per-tap address arithmetic below would otherwise
+    // be computed once per kernel and kept in -- spilled -- registers across the K loop)
+    int tapq = tid >> 7;
+    asm volatile("" : "+v"(tapq));
+    int ctile, grp, p0;
+    decode(t, ctile, grp, p0);
+    const int tb_pl = tid & (PT - 1);
     const int tb_p = p0 + tb_pl;
-    tb_valid = tb_p < total_px;
-    tb_n = tb_ho = tb_wo = tb_rem = 0;
+    const bool tb_valid = tb_p < total_px;
+    int tb_n = 0, tb_ho = 0, tb_wo = 0, tb_rem = 0;
     if (tb_valid) {
       tb_n = tb_p / plane_out;
       tb_rem = tb_p - tb_n * plane_out;
       tb_ho = tb_rem / g.Wo;
       tb_wo = tb_rem - tb_ho * g.Wo;
     }
-    wp_tile = (const unsigned char *)a.wp + ((size_t)(grp * a.n_ctiles + ctile) * nk) * (size_t)kWTile;
-    cur.init(slab0, spd);
-    bcur.init(slab0, spd);
-  };
-  auto build_table = [&](int dgi) {
-    // (opaque to the optimiser: the per-tap address arithmetic below would otherwise
-    // be computed once per kernel and kept in -- spilled -- registers across the K loop)
-    int tapq = tid >> 7;
-    asm volatile("" : "+v"(tapq));
-    const E *off = (const E *)a.om.off + (long)tb_n * a.om.off_n + (long)tb_rem * a.om.off_px +
-                   (long)(dgi * 2 * taps) * a.om.off_ch;
-    const E *msk = (const E *)a.om.msk + (long)tb_n * a.om.msk_n + (long)tb_rem * a.om.msk_px +
-                   (long)(dgi * taps) * a.om.msk_ch;
+    const E *off = (const E *)a.om.off + (long)tb_n * a.om.off_n + (long)tb_rem * a.om.off_px;
+    const E *msk = (const E *)a.om.msk + (long)tb_n * a.om.msk_n + (long)tb_rem * a.om.msk_px;
     E rdy[TPT], rdx[TPT], rm[TPT];
 #pragma unroll
     for (int i = 0; i < TPT; ++i) {
@@ -347,6 +322,8 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
       rdx[i] = off[(long)(2 * tap + 1) * a.om.off_ch];
       rm[i] = msk[(long)tap * a.om.msk_ch];
     }
+    uint32_t *tp = tpix[t & 1];
+    uint2 *tw2 = tws[t & 1];
 #pragma unroll
     for (int i = 0; i < TPT; ++i) {
       const int tap = tapq + 4 * i;
@@ -355,27 +332,52 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
         TapSample sm = make_tap_sample(tb_ho * g.sh - g.ph + ti * g.dh, tb_wo * g.sw - g.pw + tj * g.dw,
                                        to_f32(rdy[i]), to_f32(rdx[i]), mask_value<E>(rm[i], a.om.logit), g.H, g.W);
         const uint32_t pix = tb_valid ? (uint32_t)tb_n * a.img_bytes + corner_offset<UNBORDERED>(sm, g, a) : 0u;
-        uint32_t tw[4];
-        BL::table_weights(sm, tw);
-        if (!tb_valid) tw[0] = tw[1] = tw[2] = tw[3] = 0u;
-        tpix[tap * PT + tb_pl] = pix;
-        tws[tap * PT + tb_pl] = make_uint4(tw[0], tw[1], tw[2], tw[3]);
+        uint2 w2 = make_uint2(TR::pack2(sm.w00, sm.w01), TR::pack2(sm.w10, sm.w11));
+        if (!tb_valid) w2 = make_uint2(0u, 0u);
+        tp[tap * PT + tb_pl] = pix;
+        tw2[tap * PT + tb_pl] = w2;
       }
     }
+    // Retire the loads above with a wait the compiler can see.  Those of taps past
+    // the last one are never read; the compiler would otherwise keep their
+    // registers marked as pending and guard every later write to them -- the
+    // assembly loads of the K loop -- with a full wait.
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), other counters untouched
   };
 
-  // gather registers: sets x two halves of the 128-byte row x four corners
-  u32x4 gs[NS][2][4];
+  // ---- the three cursors of the produce side.  Each walks steps 0 .. nk_pad - 1
+  // of tile 0, 1, ...; steps nk .. nk_pad - 1 repeat the last real step (loads
+  // nobody uses, which keep the wait counts constant).  Past the last tile the
+  // gather and weight cursors stay where they are.
+  int g_t = 0, g_s = 0, g_tap = 0, g_slab = 0, g_slab0 = slab0_of(0);  // gather
+  int b_t = 0, b_s = 0, b_tap = 0;                                     // blend
+  int w_t = 0, w_s = 0;                                                // weight copies
+  const unsigned char *w_ptr = weights_of(0);
 
-  // addresses of the gather cursor's step, then move the cursor on
+  // gather registers: sets x two halves of the 128-byte row x four corners
+  u32x4 gs[kF2Sets][2][4];
+
   uint32_t o_tl, o_tr, o_bl, o_br;
   auto next_addresses = [&]() {
-    const int e = cur.tap * PT + pl;
-    o_tl = tpix[e] + (uint32_t)(slab0 + cur.slab) * a.slab_bytes + (uint32_t)q * 16u;
+    o_tl = tpix[g_t & 1][g_tap * PT + pl] + (uint32_t)(g_slab0 + g_slab) * a.slab_bytes + (uint32_t)q * 16u;
     o_tr = o_tl + pxb;
     o_bl = o_tl + a.row_bytes;
     o_br = o_bl + pxb;
-    cur.advance(nk, taps, spd);
+    ++g_s;
+    if (g_s < nk) {
+      if (++g_tap == taps) {
+        g_tap = 0;
+        ++g_slab;
+      }
+    } else if (g_s == nk_pad) {
+      if (g_t + 1 < T) {
+        ++g_t;
+        g_s = g_tap = g_slab = 0;
+        g_slab0 = slab0_of(g_t);
+      } else {
+        g_s = nk_pad - 1;
+      }
+    }
   };
 #define MDCN_F2_GATHER_HALF(S, H)                     \
   do {                                                \
@@ -392,8 +394,8 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
   } while (0)
 
   int islot = 0;  // ring slot of the next weight tile to issue
-  auto issue_weights = [&](int ks) {
-    const int kk = min(ks, nk - 1);  // past the end: repeat the last tile (never read)
+  auto issue_weights = [&](bool advance) {
+    const int kk = min(w_s, nk - 1);
     const uint32_t voff = (uint32_t)kk * kWTile + wlane;
     const uint32_t voff_odd = voff ^ 32u;
     const uint32_t dst = lds_w + (uint32_t)islot * kWTile + (uint32_t)(wave * kF2WD) * 1024u;
@@ -405,23 +407,33 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
                    "global_load_lds_dwordx4 %1, %3 offset:2048\n\t"
                    "global_load_lds_dwordx4 %2, %3 offset:3072"
                    :
-                   : "s"(dst), "v"(voff), "v"(voff_odd), "s"(wp_tile)
+                   : "s"(dst), "v"(voff), "v"(voff_odd), "s"(w_ptr)
                    : "memory");
     }
+    if (!advance) return;
     islot = (islot == kF2Slots - 1) ? 0 : islot + 1;
+    if (++w_s == nk_pad) {
+      if (w_t + 1 < T) {
+        ++w_t;
+        w_s = 0;
+        w_ptr = weights_of(w_t);
+      } else {
+        w_s = nk_pad - 1;
+      }
+    }
   };
+  static_assert(kF2WD == 4, "issue_weights spells out four copies");
 
-  // One produce block: the weight copies of step j + 1, the blend of step j
-  // (gather set SI) into sample tile j % 2, the gather of step j + NS into the set.
-#define MDCN_F2_BLOCK(J, SI)                                                            \
+  // One produce block: the weight copies of the step after the blend cursor's,
+  // the blend of the cursor's step (gather set SI) into its sample tile, the
+  // gather of three steps ahead into the set.
+#define MDCN_F2_BLOCK(SI)                                                               \
   do {                                                                                  \
-    const int j_ = (J);                                                                 \
-    if (j_ < nk) {                                                                      \
-      issue_weights(j_ + 1);                                                            \
+    if (b_t < T) {                                                                      \
+      issue_weights(true);                                                              \
       next_addresses();                                                                 \
-      const typename BL::Wt w_ = BL::prep(tws[bcur.tap * PT + pl], bsh, bm0, bm1);      \
-      bcur.advance(nk, taps, spd);                                                      \
-      const uint32_t xo_ = (j_ & 1) ? kXTile : 0u;                                      \
+      const typename BL::Wt w_ = BL::prep(tws[b_t & 1][b_tap * PT + pl], q);               \
+      const uint32_t xo_ = (b_s & 1) ? kXTile : 0u;                                     \
       MDCN_VMWAIT4(kF2VmBlend, gs[SI][0][0], gs[SI][0][1], gs[SI][0][2], gs[SI][0][3]); \
       {                                                                                 \
         const u32x4 o_ = (MDCN_F2_ABLATE & 4) ? (gs[SI][0][0] ^ gs[SI][0][1] ^ gs[SI][0][2] ^ gs[SI][0][3]) \
@@ -436,6 +448,13 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
         *(lds_u32x4_ptr)(xw1 + xo_) = o_;                                               \
       }                                                                                 \
       MDCN_F2_GATHER_HALF(gs[SI], 1);                                                   \
+      ++b_s;                                                                            \
+      if (b_s < nk) {                                                                   \
+        if (++b_tap == taps) b_tap = 0;                                                 \
+      } else if (b_s == nk_pad) {                                                       \
+        ++b_t;                                                                          \
+        b_s = b_tap = 0;                                                                \
+      }                                                                                 \
     }                                                                                   \
   } while (0)
 
@@ -471,69 +490,60 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
     }
   };
 
-  // Table and first gathers of a tile.  A wave keeps step j in set j % NS; the
-  // late waves, which run one block ahead, in set (j + NS - 1) % NS, so that both
-  // kinds use the same set at the same place of the K loop.  The issue order
-  // gather, copies, gather, copies, ... is the K loop's, which keeps the counts
-  // of the waits valid from the first block on (the second group of copies
-  // repeats what block 0 issues again: same data, same slot).
-  auto tile_prologue = [&](int tile) {
-    set_tile(tile);
-    __builtin_amdgcn_sched_barrier(0);
-    build_table(ch0 / g.ch_per_dg);
-    MDCN_BARRIER_LDS();  // T0: table visible
-    __builtin_amdgcn_sched_barrier(0);
-    islot = 0;
-    rslot = 0;
-    if (!late) {
-      MDCN_F2_GATHER(0);
-      issue_weights(0);
-      MDCN_F2_GATHER(1);
-      issue_weights(1);
-      islot = 1;
-      MDCN_F2_GATHER(2);
-    } else {
-      MDCN_F2_GATHER(2);
-      issue_weights(0);
-      MDCN_F2_GATHER(0);
-      issue_weights(1);
-      islot = 1;
-      MDCN_F2_GATHER(1);
-    }
-  };
-  static_assert(kF2Sets == 3, "the prologue spells out three sets");
-
 #if MDCN_F2_PROFILE
   long long prof_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
   long long prof_t = clock64();
 #endif
-  int tile = xcd * chunk + wg_in_xcd;
-  if (tile < tile_end) tile_prologue(tile);
-  MDCN_PROF(2);
 
-  while (tile < tile_end) {
-    // the tile whose products are accumulated now (the state above moves on to
-    // the next tile before this one's results are stored)
-    const int c_ctile = ctile, c_grp = grp, c_p0 = p0;
+  // ---- start of the stream: first table, first gathers.  A wave keeps step j of
+  // the stream in set j % 3; the late waves, which run one block ahead, in set
+  // (j + 2) % 3, so that both kinds use the same set at the same place of the K
+  // loop.  The issue order gather, copies, gather, copies, gather is the K
+  // loop's, which keeps the counts of the waits valid from the first block on
+  // (the second group of copies is issued again by the first block: same data,
+  // same slot).
+  // bias of this lane's output channels, fetched together with a tile's table (the
+  // wait that ends the table's loads covers it, so the epilogue never waits on memory)
+  float bv[MB], bv_next[MB];
+  auto load_bias = [&](int t, float (&b)[MB]) {
+    int ctile, grp, p0;
+    decode(t, ctile, grp, p0);
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[nb][mb][r] = 0.0f;
-
-    if (!late) {
-      MDCN_F2_BLOCK(0, 0);
-    } else {
-      MDCN_F2_BLOCK(0, 2);
-      MDCN_F2_BLOCK(1, 0);
+    for (int mb = 0; mb < MB; ++mb) {
+      const int col = ctile * CT + wave_c * 64 + mb * 32 + frow;
+      b[mb] = (a.bias && col < g.cout_g) ? to_f32(((const E *)a.bias)[(long)grp * g.cout_g + col]) : 0.0f;
     }
-    MDCN_PROF(2);
-    MDCN_BARRIER(kF2VmBar);  // X[0] and W[0] complete
-    __builtin_amdgcn_sched_barrier(0);
-    MDCN_PROF(1);
+  };
+  load_bias(0, bv);
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) bv_next[mb] = 0.0f;
+  build_table(0);
+  MDCN_BARRIER_LDS();  // table visible
+  __builtin_amdgcn_sched_barrier(0);
+  if (!late) {
+    MDCN_F2_GATHER(0);
+    issue_weights(true);
+    MDCN_F2_GATHER(1);
+    issue_weights(false);
+    MDCN_F2_GATHER(2);
+    MDCN_F2_BLOCK(0);
+  } else {
+    MDCN_F2_GATHER(2);
+    issue_weights(true);
+    MDCN_F2_GATHER(0);
+    issue_weights(false);
+    MDCN_F2_GATHER(1);
+    MDCN_F2_BLOCK(2);
+    MDCN_F2_BLOCK(0);
+  }
+  static_assert(kF2Sets == 3, "the prologue spells out three sets");
+  MDCN_PROF(2);
+  MDCN_BARRIER(kF2VmBar);  // X[0] and W[0] complete
+  __builtin_amdgcn_sched_barrier(0);
+  MDCN_PROF(1);
 
-    // ---- K loop: kF2Unroll steps per round; step k runs block k + 1 (late waves: k + 2) on set (k + 1) % NS
+  // ---- K loop of a tile: kF2Unroll steps per round; step k runs the produce
+  // block one (late waves: two) steps ahead on set (k + 1) % 3
 #define MDCN_F2_STEP(K, SI)                                   \
   do {                                                        \
     mfma_step(K);                                             \
@@ -542,14 +552,31 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
     if (late) MDCN_BARRIER(kF2VmBar);                         \
     __builtin_amdgcn_sched_barrier(0);                        \
     MDCN_PROF(5);                                             \
-    MDCN_F2_BLOCK((K) + ahead, SI);                           \
+    MDCN_F2_BLOCK(SI);                                        \
     __builtin_amdgcn_sched_barrier(0);                        \
     MDCN_PROF(4);                                             \
     if (!late) MDCN_BARRIER(kF2VmBar);                        \
     __builtin_amdgcn_sched_barrier(0);                        \
     MDCN_PROF(5);                                             \
   } while (0)
+
+  for (int t = 0; t < T; ++t) {
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[nb][mb][r] = 0.0f;
+
     for (int k = 0; k < nk_pad; k += kF2Unroll) {
+      if (k == kF2Unroll && t + 1 < T) {
+        // the next tile's table: its buffer was last read in the previous tile, its
+        // first reader is the gather cursor near the end of this one
+        load_bias(t + 1, bv_next);
+        build_table(t + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        MDCN_PROF(0);
+      }
       MDCN_F2_STEP(k + 0, 1);
       MDCN_F2_STEP(k + 1, 2);
       MDCN_F2_STEP(k + 2, 0);
@@ -557,98 +584,87 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
       MDCN_F2_STEP(k + 4, 2);
       MDCN_F2_STEP(k + 5, 0);
     }
-    // every copy and gather issued past the last step has landed, every wave is
-    // through with the table, the sample tiles and the ring
-    MDCN_VMWAIT4(0, gs[0][0][0], gs[0][1][0], gs[1][0][0], gs[2][1][0]);
-    MDCN_BARRIER(0);  // E0
-    __builtin_amdgcn_sched_barrier(0);
-    MDCN_PROF(5);
-
-    // bias of this lane's output channels
-    float bv[MB];
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-      const int mycol = c_ctile * CT + wave_c * 64 + mb * 32 + frow;
-      bv[mb] = 0.0f;
-      if (a.bias && mycol < g.cout_g) bv[mb] = to_f32(((const E *)a.bias)[c_grp * g.cout_g + mycol]);
-    }
 
     // ---- epilogue: bias, one rounding, NCHW store straight from the accumulators.
     // Accumulator block (A = samples, B = weights): register r of lane l holds
     //   pixel = (r/4)*8 + (l/32)*4 + r%4,  channel = l%32.
-    // 16-bit types: the two halves of the wave exchange packed pixel pairs
-    // (v_permlane32_swap), after which a lane holds 8 consecutive pixels = 16 bytes.
+    // The two halves of the wave exchange packed pixel pairs, after which a lane
+    // holds 8 consecutive pixels = 16 bytes of one channel.
     {
+      int ctile, grp, p0;
+      decode(t, ctile, grp, p0);
       E *out = (E *)a.out;
       const bool vec_ok = a.out_vec_ok != 0;
-      const int pw0 = c_p0 + wave_p * 64;
-      auto store_run = [&](int col, int p, const uint4 &val) {  // 16 bytes: pixels p .. of channel col
-        constexpr int RUN = 16 / ES;
-        if (col >= g.cout_g || p >= total_px) return;
-        const long cbase = (long)c_grp * g.cout_g + col;
-        if (vec_ok && p + RUN <= total_px) {
-          const int n = p / plane_out;
-          const int rem = p - n * plane_out;
-          *(uint4 *)(out + ((long)n * g.Cout + cbase) * plane_out + rem) = val;
+      const int pw0 = p0 + wave_p * 64;
+      // image and pixel-in-image of the wave's first pixel; the runs below step on from there
+      const int n0 = pw0 / plane_out;
+      const int rem0 = pw0 - n0 * plane_out;
+      auto store_run = [&](long cbase, int dp, const u32x4 &val) {  // pixels pw0 + dp .. + 7 of channel cbase
+        const int p = pw0 + dp;
+        if (p >= total_px) return;
+        int n = n0, rem = rem0 + dp;
+        while (rem >= plane_out) {
+          rem -= plane_out;
+          ++n;
+        }
+        E *dst = out + ((long)n * g.Cout + cbase) * plane_out + rem;
+        if (vec_ok && p + 8 <= total_px) {  // (rows of 8 never straddle images then)
+          *(u32x4 *)dst = val;
         } else {
-          const E *ve = (const E *)&val;
-#pragma unroll 1
-          for (int i = 0; i < RUN; ++i) {
-            const int pi = p + i;
-            if (pi < total_px) {
-              const int ni = pi / plane_out;
-              const int ri = pi - ni * plane_out;
-              out[((long)ni * g.Cout + cbase) * plane_out + ri] = ve[i];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            const uint32_t word = val[i >> 1];
+            const uint16_t bits = (uint16_t)((i & 1) ? (word >> 16) : (word & 0xffffu));
+            if (p + i < total_px) {
+              int ni = n, ri = rem + i;
+              while (ri >= plane_out) {
+                ri -= plane_out;
+                ++ni;
+              }
+              *(uint16_t *)(out + ((long)ni * g.Cout + cbase) * plane_out + ri) = bits;
             }
           }
         }
       };
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
-        const int col = c_ctile * CT + wave_c * 64 + mb * 32 + frow;
+        const int col = ctile * CT + wave_c * 64 + mb * 32 + frow;
+        const bool col_ok = col < g.cout_g;
+        const long cbase = (long)grp * g.cout_g + col;
+        const float bvm = bv[mb];
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
           const f32x16 &c = acc[nb][mb];
-          if constexpr (ES == 2) {
 #pragma unroll
-            for (int g2 = 0; g2 < 2; ++g2) {
-              const int ga = 2 * g2, gb = 2 * g2 + 1;
-              const uint32_t a0 = TR::pack2(c[4 * ga + 0] + bv[mb], c[4 * ga + 1] + bv[mb]);
-              const uint32_t a1 = TR::pack2(c[4 * ga + 2] + bv[mb], c[4 * ga + 3] + bv[mb]);
-              const uint32_t b0 = TR::pack2(c[4 * gb + 0] + bv[mb], c[4 * gb + 1] + bv[mb]);
-              const uint32_t b1 = TR::pack2(c[4 * gb + 2] + bv[mb], c[4 * gb + 3] + bv[mb]);
-              // lower half keeps group ga and receives the upper half's part of it; upper half likewise with gb
-              const auto s0 = __builtin_amdgcn_permlane32_swap(a0, b0, false, false);
-              const auto s1 = __builtin_amdgcn_permlane32_swap(a1, b1, false, false);
-              const int p = pw0 + nb * 32 + 8 * (fhalf ? gb : ga);
-              store_run(col, p, make_uint4(s0[0], s1[0], s0[1], s1[1]));
-            }
-          } else {
-#pragma unroll
-            for (int gq = 0; gq < 4; ++gq) {
-              const int p = pw0 + nb * 32 + 8 * gq + 4 * fhalf;
-              store_run(col, p, make_uint4(__float_as_uint(c[4 * gq + 0] + bv[mb]), __float_as_uint(c[4 * gq + 1] + bv[mb]),
-                                           __float_as_uint(c[4 * gq + 2] + bv[mb]), __float_as_uint(c[4 * gq + 3] + bv[mb])));
-            }
+          for (int g2 = 0; g2 < 2; ++g2) {
+            const int ga = 2 * g2, gb = 2 * g2 + 1;
+            const uint32_t a0 = TR::pack2(c[4 * ga + 0] + bvm, c[4 * ga + 1] + bvm);
+            const uint32_t a1 = TR::pack2(c[4 * ga + 2] + bvm, c[4 * ga + 3] + bvm);
+            const uint32_t b0 = TR::pack2(c[4 * gb + 0] + bvm, c[4 * gb + 1] + bvm);
+            const uint32_t b1 = TR::pack2(c[4 * gb + 2] + bvm, c[4 * gb + 3] + bvm);
+            // lower half keeps group ga and receives the upper half's part of it; upper half likewise with gb
+            const auto s0 = __builtin_amdgcn_permlane32_swap(a0, b0, false, false);
+            const auto s1 = __builtin_amdgcn_permlane32_swap(a1, b1, false, false);
+            u32x4 val;
+            val.x = s0[0]; val.y = s1[0]; val.z = s0[1]; val.w = s1[1];
+            if (col_ok) store_run(cbase, nb * 32 + 8 * (fhalf ? gb : ga), val);
           }
         }
       }
     }
-    MDCN_PROF(6);
-    __builtin_amdgcn_sched_barrier(0);  // (keeps the next tile's address arithmetic out of the epilogue's registers)
-    // ---- the next tile's table and first gathers
-    tile += wgs_per_xcd;
-    if (tile < tile_end) tile_prologue(tile);
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) bv[mb] = bv_next[mb];
     __builtin_amdgcn_sched_barrier(0);
-    MDCN_PROF(0);
-
+    MDCN_PROF(6);
   }
+  // copies issued past the last step must have landed before the workgroup gives up its LDS
+  MDCN_VMWAIT4(0, gs[0][0][0], gs[0][1][0], gs[1][0][0], gs[2][1][0]);
 #undef MDCN_F2_STEP
 #undef MDCN_F2_BLOCK
 #undef MDCN_F2_GATHER
 #undef MDCN_F2_GATHER_HALF
 #if MDCN_F2_PROFILE
-  // slots: 0 next tile's table and first gathers, 1 barrier before the K loop, 2 first blocks, 3 MFMA steps,
+  // slots: 0 next tile's table, 1 barrier before the K loop, 2 first blocks, 3 MFMA steps,
   //        4 produce blocks, 5 step barriers, 6 epilogue
   if (a.prof && lane == 0 && (blockIdx.x == 0 || blockIdx.x == 101))
     for (int i = 0; i < 8; ++i) ((long long *)a.prof)[((blockIdx.x ? 1 : 0) * 8 + wave) * 8 + i] = prof_acc[i];

@@ -87,3 +87,56 @@ def test_auto_picks_direct_for_odd_channels():
     x = torch.zeros(1, device='cuda')
     p.input = p.offset = p.mask = p.weight = p.output = x.data_ptr()
     assert lib.mdcn_forward(ctypes.byref(p), None) == -5  # MDCN_ERR_PATH
+
+
+# Shapes that reach the eight-wave streaming kernel (16-bit tensors, more than 128 output channels per group,
+# one deformable group, at least 18 K steps), chosen so that workgroups walk several tiles, tiles end inside
+# an image, images end inside a tile and the padded step count differs from the real one.
+STREAM = {
+    'many_tiles': dict(N=4, Cin=128, Cout=256, H=96, W=96),                 # 288 tiles on 256 workgroups
+    'ragged': dict(N=3, Cin=192, Cout=200, H=61, W=53, sigma=3.0),          # 27 steps padded to 30, odd plane
+    'stride2_groups': dict(N=2, Cin=256, Cout=512, H=37, W=41, stride=2, groups=2),
+    'dilated_far': dict(N=1, Cin=128, Cout=384, H=30, W=34, dilation=2, padding=2, sigma=9.0),
+    'k1x3': dict(N=2, Cin=384, Cout=256, H=20, W=24, k=(1, 3), padding=(0, 1)),
+}
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('name', sorted(STREAM))
+def test_streaming_kernel(name, dtype):
+    """Default fused path (streaming kernel) against the oracle and against the
+    specialised-wave kernel on the same inputs."""
+    print(f'case={name} dtype={dtype}', flush=True)
+    case = make_case(11, **STREAM[name])
+    dev = cast_case(case, dtype, 'cuda')
+    y = capi_forward(dev, path=capi.PATH_FUSED)
+    y_split = capi_forward(dev, path=capi.PATH_FUSED_SPLIT)
+    ref = oracle_forward(cast_case(case, dtype))
+    assert rel_err(y.float().cpu().numpy(), ref) <= TOL[dtype]
+    assert rel_err(y_split.float().cpu().numpy(), ref) <= TOL[dtype]
+    assert rel_err(y.float().cpu().numpy(), y_split.float().cpu().numpy()) <= TOL[dtype]
+
+
+@pytest.mark.parametrize('path', [capi.PATH_FUSED, capi.PATH_FUSED_SPLIT, capi.PATH_DIRECT])
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+def test_outside_taps_never_touch_the_image(path, dtype):
+    """A tap whose position lies outside (-1, H) x (-1, W) adds nothing in the
+    reference (cpu/modulated_deform_conv.cpp:160-164), whatever the image holds:
+    Inf / NaN in the corner pixels must not leak into outputs whose taps that
+    would touch them are all outside."""
+    kw = dict(N=2, Cin=128, Cout=256, H=24, W=28)
+    case = make_case(5, **kw)
+    # every tap of every pixel far outside, except the lower right quarter of the plane, which samples
+    # around its own position (away from the poisoned corner)
+    off = case['offset']
+    off[:] = 1000.0
+    off[:, :, 12:, 14:] = torch.randn(off[:, :, 12:, 14:].shape, generator=torch.Generator().manual_seed(3)) * 0.5
+    case['input'][:, :, 0:2, 0:2] = float('inf')
+    case['input'][:, 1::2, 0, 0] = float('nan')
+    clean = dict(case)
+    clean['input'] = case['input'].clone()
+    clean['input'][:, :, 0:2, 0:2] = 0.0  # nothing in the oracle run may depend on these pixels
+    ref = oracle_forward(cast_case(clean, dtype))
+    y = capi_forward(cast_case(case, dtype, 'cuda'), path=path).float().cpu().numpy()
+    assert np.isfinite(y).all()
+    assert rel_err(y, ref) <= TOL[dtype]
