@@ -15,6 +15,11 @@ per-stage breakdown go to stderr.
   cpu_baseline  the reference's own CPU path (compiled from its sources into
               oracle/_ref) or, when that is absent, the C restatement, timed on
               this host on a bounded number of samples of the same workload
+  parity      max|y - y_ref| / max|y_ref| of the GPU output against the outputs the
+              CPU leg has just computed on the same (rounded) inputs
+  configs     the other benchmark configurations (cfg 1-3, cfg 4 in fp16, the 13
+              layers of cfg 5) with fewer steps: ms, TFLOP/s, fraction of the
+              dtype's matrix peak
 """
 import argparse
 import json
@@ -28,6 +33,10 @@ sys.path.insert(0, os.path.join(ROOT, 'tests'))
 
 PEAK_TFLOPS = {'bf16': 2500.0, 'f16': 2500.0, 'f32': 157.3}
 HBM_PEAK_GBS = 8000.0
+# (workload, dominant kernel) -> (HBM bytes per launch from rocprofv3 counters, the profile they are in)
+TRAFFIC = {
+    ('cfg4', 'fused2_kernel<bf16>'): (None, None),
+}
 
 WORKLOADS = {
     'cfg1': dict(N=1, Cin=64, Cout=64, H=56, W=56, sigma=2.0, dtype='f32'),
@@ -44,7 +53,10 @@ def log(*a):
 
 
 def cpu_baseline(case, flops_per_sample, budget_s=20.0):
-    """Time the CPU path on as many samples of the workload as fit the budget."""
+    """Time the CPU path on as many samples of the workload as fit the budget.
+    `case` holds fp32 CPU tensors (the values the device sees, up-cast).  Returns
+    the record and the CPU output of the samples that were run."""
+    import numpy as np
     import torch
     import oracle
     N = case['input'].shape[0]
@@ -57,16 +69,17 @@ def cpu_baseline(case, flops_per_sample, budget_s=20.0):
         t = {k: case[k][:n] for k in ('input', 'offset', 'mask')}
         t0 = time.perf_counter()
         if use_ref:
-            oracle.reference_forward(t['input'], t['offset'], t['mask'], case['weight'],
-                                     case['bias'], **args(n))
+            y = oracle.reference_forward(t['input'], t['offset'], t['mask'], case['weight'],
+                                         case['bias'], **args(n))
         else:
-            oracle.forward(t['input'].numpy(), t['offset'].numpy(), t['mask'].numpy(),
-                           case['weight'].numpy(), case['bias'].numpy(), **args(n))
-        return time.perf_counter() - t0
+            y = oracle.forward(t['input'].numpy(), t['offset'].numpy(), t['mask'].numpy(),
+                               case['weight'].numpy(), case['bias'].numpy(), **args(n))
+        return time.perf_counter() - t0, y
 
-    t1 = run(1)  # also the warm-up
+    t1, _ = run(1)  # also the warm-up
     n = int(max(1, min(N, budget_s // max(t1, 1e-3))))
-    tn = run(n)
+    tn, y_ref = run(n)
+    y_ref = y_ref.numpy() if hasattr(y_ref, 'numpy') else np.asarray(y_ref)
     threads = torch.get_num_threads() if use_ref else int(os.environ.get('OMP_NUM_THREADS', os.cpu_count()))
     return {
         'value': round(flops_per_sample * n / tn / 1e12, 5),
@@ -77,7 +90,7 @@ def cpu_baseline(case, flops_per_sample, budget_s=20.0):
                    f'({tn / n * 1e3:.0f} ms/sample; im2col stage is single-threaded, '
                    f'GEMM uses {threads} threads)'),
         'ms_per_layer_extrapolated': round(tn / n * N * 1e3, 1),
-    }
+    }, y_ref
 
 
 # cfg 5: DCNv2 ResNet-50 stages c3-c5 at an 800x1344 image scale, batch 16, bf16:
@@ -153,6 +166,45 @@ def run_cfg5(a):
     return rows, tot_dcn, tot_prod, tot_flops, tot_pack
 
 
+def quick_config(name, steps, warmup):
+    """One of the single-layer configurations with few steps: ms per call of the
+    extension op, TFLOP/s and the fraction of the dtype's matrix peak."""
+    import torch
+    from common import make_case, cast_case
+    from mmcv_amd.ops.modulated_deform_conv import ext_module
+    wl = dict(WORKLOADS[name])
+    dname = wl.pop('dtype')
+    dtype = {'bf16': torch.bfloat16, 'f16': torch.float16, 'f32': torch.float32}[dname]
+    case = make_case(20240 + int(name[3]), **wl)
+    dev = cast_case(case, dtype, 'cuda')
+    x, off, msk, w, b = (dev[k] for k in ('input', 'offset', 'mask', 'weight', 'bias'))
+    N, Cin, H, W = x.shape
+    Cout, cin_g, kh, kw = w.shape
+    (sh, sw), (ph, pw), (dh, dw) = case['stride'], case['padding'], case['dilation']
+    Ho = (H + 2 * ph - (dh * (kh - 1) + 1)) // sh + 1
+    Wo = (W + 2 * pw - (dw * (kw - 1) + 1)) // sw + 1
+    out = torch.empty(N, Cout, Ho, Wo, dtype=dtype, device='cuda')
+    empty = x.new_empty(0)
+    kwargs = dict(kernel_h=kh, kernel_w=kw, stride_h=sh, stride_w=sw, pad_h=ph, pad_w=pw,
+                  dilation_h=dh, dilation_w=dw, group=case['groups'],
+                  deformable_group=case['deform_groups'], with_bias=True)
+    fn = lambda: ext_module.modulated_deform_conv_forward(x, w, b, empty, off, msk, out, empty, **kwargs)
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / steps
+    flops = 2.0 * N * Ho * Wo * Cout * cin_g * kh * kw
+    tf = flops / ms / 1e9
+    return {'dtype': dname, 'ms_per_layer': round(ms, 4), 'TFLOPs': round(tf, 2),
+            'pct_matrix_peak': round(100.0 * tf / PEAK_TFLOPS[dname], 2), 'steps': steps, 'warmup': warmup}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -160,6 +212,8 @@ def main():
     ap.add_argument('--warmup', type=int, default=20)
     ap.add_argument('--workload', default='cfg4', choices=sorted(WORKLOADS) + ['cfg5'])
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
+    ap.add_argument('--no-configs', action='store_true',
+                    help='skip the short runs of the other benchmark configurations')
     ap.add_argument('--copy-probe', action='store_true',
                     help='run a plain elementwise copy of known size instead (calibrates the '
                          'FETCH_SIZE / WRITE_SIZE counters) and exit')
@@ -314,10 +368,14 @@ def main():
         scratch = torch.empty(16384, dtype=torch.uint8, device='cuda')
         tf = ctypes.c_float()
         sustained = {}
+        probe = ctypes.CDLL(os.path.join(ROOT, 'mmcv_amd', 'lib', 'libmdcn_probe.so'))
+        probe.mdcn_mfma_probe.restype = ctypes.c_int
+        probe.mdcn_mfma_probe.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+                                          ctypes.c_void_p, ctypes.POINTER(ctypes.c_float)]
         for key, zero in (('random_operands', 0), ('zero_operands', 1)):
-            rc = lib.mdcn_mfma_probe(2 if dname == 'bf16' else 1, 2, zero, ctypes.c_void_p(scratch.data_ptr()), cstream,
-                                     ctypes.byref(tf))
-            assert rc == 0, capi.status_string(rc)
+            rc = probe.mdcn_mfma_probe(2 if dname == 'bf16' else 1, 2, zero, ctypes.c_void_p(scratch.data_ptr()),
+                                       cstream, ctypes.byref(tf))
+            assert rc == 0, f'mdcn_mfma_probe: status {rc}'
             sustained[key] = round(tf.value, 1)
         log(f'sustained MFMA rate: {sustained}')
     log(f'per call: median {per_call[len(per_call) // 2]:.4f} min {per_call[0]:.4f} ms; rotating buffers '
@@ -344,6 +402,9 @@ def main():
 
     value = flops / (ms_per_step * 1e-3) / 1e12
     achieved = flops / (main_ms * 1e-3) / 1e12
+    # the 16-bit 256-channel tiles of cfg 4 run the eight-wave streaming kernel, the rest fused_kernel
+    kernel_name = (f'fused2_kernel<{dname}>' if a.workload.startswith('cfg4') and ext_module.get_path() in (0, 1)
+                   else f'fused_kernel<{dname}>')
     peak = PEAK_TFLOPS[dname]
     rec = {
         'metric': 'DCNv2 fwd TFLOP/s + ms/layer (N=16,C=256,100x152 bf16); % MFMA peak',
@@ -381,23 +442,54 @@ def main():
                      'what': 'grad input/offset/mask/weight/bias; two products of the forward size'},
         'roofline': {
             'bound': 'mfma',
-            'kernel': f'fused_kernel<{dname}>',
+            'kernel': kernel_name,
             'achieved': round(achieved, 2),
             'peak': peak,
             'unit': 'TFLOP/s',
             'frac': round(achieved / peak, 4),
-            # HBM bytes per launch of the fused kernel on cfg4/bf16 from rocprofv3 FETCH_SIZE and
-            # WRITE_SIZE, scaled by a copy kernel (profiles/fused_kernel_bf16_cfg4.md)
-            'traffic': 378.3e6 if a.workload == 'cfg4' else None,
+            # HBM bytes per launch of that kernel from rocprofv3 FETCH_SIZE and WRITE_SIZE, scaled by a
+            # copy kernel of known size: a figure from the named profile, not from this run
+            'traffic': TRAFFIC.get((a.workload, kernel_name), (None, None))[0],
+            'traffic_source': TRAFFIC.get((a.workload, kernel_name), (None, None))[1],
         },
         # measured on this box, same run: TFLOP/s of back-to-back 32x32x16 MFMAs on all CUs; the kernel's
         # share of what the matrix cores sustain on non-trivial operands
         'mfma_sustained_TFLOPs': sustained,
         'frac_of_sustained': (round(achieved / sustained['random_operands'], 4) if sustained else None),
     }
+    if not a.no_configs:
+        others = {}
+        for name in sorted(WORKLOADS):
+            if name != a.workload:
+                others[name] = quick_config(name, max(5, min(a.steps, 50)), max(2, min(a.warmup, 10)))
+                log(name, others[name])
+        a5 = argparse.Namespace(steps=max(5, min(a.steps, 20)), warmup=max(2, min(a.warmup, 5)))
+        rows, tot_dcn, tot_prod, tot_flops, tot_pack = run_cfg5(a5)
+        others['cfg5'] = {'dtype': 'bf16', 'summed_ms': round(tot_dcn, 4),
+                          'TFLOPs': round(tot_flops / tot_dcn / 1e9, 1),
+                          'pct_matrix_peak': round(100.0 * tot_flops / tot_dcn / 1e9 / PEAK_TFLOPS['bf16'], 2),
+                          'summed_ms_pack_fused': round(tot_pack, 4), 'steps': a5.steps, 'warmup': a5.warmup,
+                          'per_layer_ms': {r['layer']: r['dcn_ms'] for r in rows}}
+        rec['configs'] = others
     if not a.no_cpu:
         log('timing the CPU baseline ...')
-        rec['cpu_baseline'] = cpu_baseline(case, flops / N)
+        # the CPU path gets the values the device saw (rounded to the tensor dtype, up-cast), so its
+        # output is the reference for the GPU output of the timed steps
+        seen = dict(case)
+        for k in ('input', 'offset', 'mask', 'weight', 'bias'):
+            seen[k] = dev[k].float().cpu()
+        step()
+        torch.cuda.synchronize()
+        rec['cpu_baseline'], y_ref = cpu_baseline(seen, flops / N)
+        import numpy as np
+        n_ref = y_ref.shape[0]
+        y_gpu = out[:n_ref].float().cpu().numpy()
+        err = float(np.abs(y_gpu - y_ref).max() / np.abs(y_ref).max())
+        tol = 1e-4 if dname == 'f32' else 2e-2
+        rec['parity'] = {'max_abs_err_over_max_abs_ref': float(f'{err:.3e}'), 'tolerance': tol,
+                         'samples_checked': n_ref, 'of': N, 'ok': bool(err <= tol and np.isfinite(y_gpu).all()),
+                         'against': rec['cpu_baseline']['kind'] + ' CPU path on the same rounded inputs'}
+        log('parity', rec['parity'])
     print(json.dumps(rec), flush=True)
 
 

@@ -26,11 +26,19 @@
 extern "C" {
 #endif
 
-#define MDCN_ABI_VERSION 3
+#define MDCN_ABI_VERSION 4
 
 /* Element type of every tensor of a call (the Python wrapper unifies them to
  * offset's dtype, mmcv/ops/modulated_deform_conv.py:136-139). */
-enum mdcn_dtype { MDCN_F32 = 0, MDCN_F16 = 1, MDCN_BF16 = 2 };
+enum mdcn_dtype {
+  MDCN_F32 = 0,
+  MDCN_F16 = 1,
+  MDCN_BF16 = 2,
+  MDCN_F64 = 3 /* double: the reference dispatches its kernels over it as well
+                  (mmcv/ops/csrc/pytorch/cuda/modulated_deform_conv_cuda.cu:16); served by plain
+                  one-thread-per-output kernels that compute in double, forward and backward, never by
+                  the fused path, and not by the pack-level call (MDCN_ERR_DTYPE there) */
+};
 
 /* Which device path runs. */
 enum mdcn_path {
@@ -152,16 +160,6 @@ int mdcn_forward_noalloc(const mdcn_params *p, void *hip_stream);
  *   ms[0] input re-layout, ms[1] weight repack, ms[2] main kernel, ms[3] total.
  * Stages a path does not run report 0.  For measurement only. */
 int mdcn_forward_timed(const mdcn_params *p, void *hip_stream, float ms[4]);
-
-/* Measures what the matrix cores of the current device sustain: every CU runs
- * `waves_per_simd` (1 or 2) wavefronts of back-to-back 32x32x16 MFMAs (dtype
- * MDCN_BF16 or MDCN_F16) on pseudo-random operands, or on zeros with `zero_data`
- * != 0 (the clock, and with it the rate, depends on how much the operands
- * toggle).  Launches on `hip_stream`, waits for it and stores TFLOP/s in
- * *tflops.  Uses `scratch`, at least 16 KiB of device memory.  For
- * measurement only: the bench reports it beside the published peak.  (No
- * counterpart in the reference.) */
-int mdcn_mfma_probe(int dtype, int waves_per_simd, int zero_data, void *scratch, void *hip_stream, float *tflops);
 
 /*
  * The deformable convolution together with the step in front of it in

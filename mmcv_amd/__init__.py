@@ -7,5 +7,8 @@ behind mmcv's own API for that path.
 The device code is hand-written HIP for gfx950 in ``lib/libmdcn_hip.so`` (C ABI:
 ``include/mdcn.h``); ``mmcv_amd._ext`` is the PyTorch-ROCm extension module that
 mmcv's Python op layer binds to.  Build both with ``python -m mmcv_amd.build``.
+``mmcv_amd.patch()`` binds an installed mmcv to it at run time.
 """
-__version__ = '0.1.0'
+__version__ = '0.2.0'
+
+from .patch import patch, unpatch  # noqa: E402,F401

@@ -2,6 +2,7 @@
 
 ``libmdcn_hip.so``  hand-written HIP for gfx950 behind the C ABI of include/mdcn.h
                     (hipcc cross-compiles it without a GPU),
+``libmdcn_probe.so`` the bench's MFMA-rate probe (not part of the product ABI),
 ``_ext*.so``        the PyTorch-ROCm extension module ``mmcv_amd._ext`` (host
                     compiler only) that mmcv's Python op layer binds to.
 
@@ -17,6 +18,7 @@ ROOT = os.path.dirname(PKG)
 CSRC = os.path.join(PKG, 'csrc')
 LIBDIR = os.path.join(PKG, 'lib')
 HIP_LIB = os.path.join(LIBDIR, 'libmdcn_hip.so')
+PROBE_LIB = os.path.join(LIBDIR, 'libmdcn_probe.so')
 EXT_LIB = os.path.join(PKG, '_ext' + sysconfig.get_config_var('EXT_SUFFIX'))
 ROCM = os.environ.get('ROCM_PATH', '/opt/rocm')
 
@@ -41,6 +43,14 @@ def build_hip(extra=()):
     _run([hipcc, *HIPCC_FLAGS, *extra, '-I', os.path.join(ROOT, 'include'),
           '-o', HIP_LIB, os.path.join(CSRC, 'mdcn_api.hip')])
     return HIP_LIB
+
+
+def build_probe():
+    """The bench's MFMA-rate probe: its own library, not part of the product ABI."""
+    hipcc = os.path.join(ROCM, 'bin', 'hipcc')
+    _run([hipcc, *HIPCC_FLAGS, '-I', os.path.join(ROOT, 'include'),
+          '-o', PROBE_LIB, os.path.join(CSRC, 'mdcn_probe.hip')])
+    return PROBE_LIB
 
 
 def build_ext():
@@ -69,6 +79,7 @@ def build_ext():
 
 def build_all():
     build_hip()
+    build_probe()
     build_ext()
 
 

@@ -9,14 +9,14 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, 'lib', 'libmdcn_hip.so')
 
-MDCN_F32, MDCN_F16, MDCN_BF16 = 0, 1, 2
+MDCN_F32, MDCN_F16, MDCN_BF16, MDCN_F64 = 0, 1, 2, 3
 PATH_AUTO, PATH_FUSED, PATH_DIRECT, PATH_FUSED_SPLIT = 0, 1, 2, 3
 MDCN_OK = 0
 NOALLOC_SCRATCH_BYTES = 64 << 20
 
 EXPORTS = ('mdcn_abi_version', 'mdcn_set_pass_limits', 'mdcn_status_string', 'mdcn_output_size',
            'mdcn_fused_eligible', 'mdcn_workspace_bytes', 'mdcn_forward', 'mdcn_forward_noalloc',
-           'mdcn_forward_timed', 'mdcn_mfma_probe', 'mdcn_pack_workspace_bytes', 'mdcn_pack_forward',
+           'mdcn_forward_timed', 'mdcn_pack_workspace_bytes', 'mdcn_pack_forward',
            'mdcn_pack_forward_timed', 'mdcn_backward_workspace_bytes', 'mdcn_backward')
 
 
@@ -71,9 +71,6 @@ def load():
         lib.mdcn_forward_timed.restype = ctypes.c_int
         lib.mdcn_forward_timed.argtypes = [P, ctypes.c_void_p,
                                            ctypes.POINTER(ctypes.c_float)]
-        lib.mdcn_mfma_probe.restype = ctypes.c_int
-        lib.mdcn_mfma_probe.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p,
-                                        ctypes.POINTER(ctypes.c_float)]
         PP = ctypes.POINTER(MdcnPackParams)
         lib.mdcn_pack_workspace_bytes.restype = ctypes.c_size_t
         lib.mdcn_pack_workspace_bytes.argtypes = [PP]

@@ -35,6 +35,7 @@ int mdcn_dtype_of(const Tensor &t) {
     case at::kFloat: return MDCN_F32;
     case at::kHalf: return MDCN_F16;
     case at::kBFloat16: return MDCN_BF16;
+    case at::kDouble: return MDCN_F64;
     default:
       TORCH_CHECK(false, "\"modulated_deform_conv_forward\" not implemented for '",
                   c10::toString(t.scalar_type()), "'");

@@ -12,6 +12,7 @@
 
 #include "mdcn_common.h"
 #include "mdcn_direct.h"
+#include "mdcn_f64.h"
 #include "mdcn_backward.h"
 #include "mdcn_backward_gemm.h"
 #include "mdcn_fused.h"
@@ -58,11 +59,11 @@ int scratch_of_current_device(void **out) {
   return MDCN_OK;
 }
 
-inline size_t elem_size(int dtype) { return dtype == MDCN_F32 ? 4 : 2; }
+inline size_t elem_size(int dtype) { return dtype == MDCN_F64 ? 8 : dtype == MDCN_F32 ? 4 : 2; }
 
 int check_params(const mdcn_params *p, Geom *g, bool need_ptrs, bool need_offsets = true) {
   if (!p) return MDCN_ERR_NULL;
-  if (p->dtype != MDCN_F32 && p->dtype != MDCN_F16 && p->dtype != MDCN_BF16)
+  if (p->dtype != MDCN_F32 && p->dtype != MDCN_F16 && p->dtype != MDCN_BF16 && p->dtype != MDCN_F64)
     return MDCN_ERR_DTYPE;
   if (p->N <= 0 || p->Cin <= 0 || p->H <= 0 || p->W <= 0 || p->Cout <= 0 ||
       p->kh <= 0 || p->kw <= 0 || p->sh <= 0 || p->sw <= 0 || p->ph < 0 ||
@@ -103,6 +104,7 @@ inline int pick_ct(int cout_g, int taps) {
 }
 
 bool fused_ok(const mdcn_params *p, const Geom &g) {
+  if (p->dtype == MDCN_F64) return false;  // double precision: the one-thread-per-output kernels only
   const int KC = slab_channels(p->dtype);
   if (p->input_nhwc && (g.H < 2 || g.W < 2 || ((uintptr_t)p->input % 16) != 0)) return false;
   if (g.cin_g % KC || g.ch_per_dg % KC) return false;
@@ -359,15 +361,22 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
     const bool own_oconv = px && px->offset_weight;
     const int cof = pl.CO_pad / 32;
 
-    // weights: once per call
+    // weights: once per call -- inside the launch that re-lays the first batch chunk when the
+    // input allows the vector re-layout (whole 16-byte runs per channel row), else on their own
+    constexpr int EPV = 16 / (int)sizeof(E);
+    const bool vec_relayout = !p->input_nhwc && ((g.H * g.W) % EPV == 0) && (((uintptr_t)p->input % 16) == 0);
+    const long wtotal = (long)g.G * pl.n_ctiles * pl.slabs * g.taps * pl.CT * pl.KC;
+    bool packed = false;
     {
-      const long total = (long)g.G * pl.n_ctiles * pl.slabs * g.taps * pl.CT * pl.KC;
-      const int grid = (int)std::min<long>((total + 255) / 256, 1L << 16);
       tic();
-      hipLaunchKernelGGL(pack_weight_kernel<E>, dim3(grid), dim3(256), 0, st, g,
-                         (const E *)p->weight, wp, pl.CT, pl.KC, pl.n_ctiles,
-                         pl.slabs, total);
-      if (hipGetLastError() != hipSuccess) rc = MDCN_ERR_LAUNCH;
+      if (!vec_relayout) {
+        const int grid = (int)std::min<long>((wtotal + 255) / 256, 1L << 16);
+        hipLaunchKernelGGL(pack_weight_kernel<E>, dim3(grid), dim3(256), 0, st, g,
+                           (const E *)p->weight, wp, pl.CT, pl.KC, pl.n_ctiles,
+                           pl.slabs, wtotal);
+        if (hipGetLastError() != hipSuccess) rc = MDCN_ERR_LAUNCH;
+        packed = true;
+      }
       if (own_oconv) {
         const long ototal = (long)(g.Cin / pl.KC) * g.taps * 4 * cof * 64 * (16 / (long)es);
         const int ogrid = (int)std::min<long>((ototal + 255) / 256, 1L << 16);
@@ -382,7 +391,23 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
       gc.N = std::min(pl.n_chunk, g.N - n0);
       const E *in = (const E *)p->input + (size_t)n0 * g.Cin * g.H * g.W;
       const bool nhwc = p->input_nhwc != 0;
-      if (!nhwc) {
+      if (!nhwc && vec_relayout) {
+        const int n_pchunks = (gc.H * gc.W + 32 * EPV - 1) / (32 * EPV);
+        const long blocks = (long)gc.N * (gc.Cin / pl.KC) * n_pchunks;
+        tic();
+        if (!packed) {
+          const int pack_blocks = (int)std::max<long>(1, std::min<long>(wtotal / (256 * 8), 512));
+          hipLaunchKernelGGL(prepass_kernel<E>, dim3((unsigned)(blocks + pack_blocks)), dim3(256), 0, st, gc, in, xt,
+                             n_pchunks, g, (const E *)p->weight, wp, pl.CT, pl.KC, pl.n_ctiles, pl.slabs, wtotal,
+                             pack_blocks);
+          packed = true;
+        } else {
+          hipLaunchKernelGGL((relayout_vec_kernel<E, true>), dim3((unsigned)blocks), dim3(256), 0, st, gc, in, xt,
+                             n_pchunks);
+        }
+        if (hipGetLastError() != hipSuccess) rc = MDCN_ERR_LAUNCH;
+        toc(0);
+      } else if (!nhwc) {
         // runs of 128 pixels of the image plane
         const int n_pchunks = (gc.H * gc.W + 127) / 128;
         const long blocks = (long)gc.N * (gc.Cin / pl.KC) * n_pchunks;
@@ -491,6 +516,31 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
   return rc;
 }
 
+// Double precision: one kernel, no workspace.
+int run_f64(const mdcn_params *p, const Geom &g, hipStream_t st, float *ms) {
+  hipEvent_t ev[2] = {nullptr, nullptr};
+  if (ms) {
+    ms[0] = ms[1] = ms[2] = ms[3] = 0.f;
+    if (hipEventCreate(&ev[0]) != hipSuccess || hipEventCreate(&ev[1]) != hipSuccess) return MDCN_ERR_LAUNCH;
+    (void)hipEventRecord(ev[0], st);
+  }
+  const long total = (long)g.N * g.Cout * g.Ho * g.Wo;
+  const int grid = (int)std::min<long>((total + 255) / 256, 1L << 20);
+  hipLaunchKernelGGL(f64_forward_kernel, dim3(grid), dim3(256), 0, st, g, (const double *)p->input,
+                     (const double *)p->offset, (const double *)p->mask, (const double *)p->weight,
+                     (const double *)p->bias, (double *)p->output, total);
+  const int rc = hipGetLastError() == hipSuccess ? MDCN_OK : MDCN_ERR_LAUNCH;
+  if (ms) {
+    (void)hipEventRecord(ev[1], st);
+    (void)hipEventSynchronize(ev[1]);
+    (void)hipEventElapsedTime(&ms[2], ev[0], ev[1]);
+    ms[3] = ms[2];
+    (void)hipEventDestroy(ev[0]);
+    (void)hipEventDestroy(ev[1]);
+  }
+  return rc;
+}
+
 int run(const mdcn_params *p, void *stream, float *ms, const mdcn_pack_params *pp = nullptr) {
   Geom g;
   int rc = check_params(p, &g, true, pp == nullptr);
@@ -508,6 +558,10 @@ int run(const mdcn_params *p, void *stream, float *ms, const mdcn_pack_params *p
     rc = make_plan(p, g, &pl);
   }
   if (rc != MDCN_OK) return rc;
+  if (p->dtype == MDCN_F64) {
+    if (pp) return MDCN_ERR_DTYPE;  // the pack-level call has no double-precision form
+    return run_f64(p, g, (hipStream_t)stream, ms);
+  }
   const size_t need = pl.xt_bytes + pl.wp_bytes + pl.owp_bytes + pl.raw_bytes;
   if (need > 0 && (!p->workspace || p->workspace_bytes < need ||
                    ((uintptr_t)p->workspace % kAlign) != 0))
@@ -561,7 +615,8 @@ struct BwdPlan {
 };
 
 void make_bwd_plan(const mdcn_bwd_params *bp, const Geom &g, BwdPlan *pl) {
-  const bool staged = bp->conv.dtype != MDCN_F32;
+  const bool f64 = bp->conv.dtype == MDCN_F64;
+  const bool staged = bp->conv.dtype != MDCN_F32 && !f64;
   const size_t es = elem_size(bp->conv.dtype);
   pl->gin_bytes = (staged && bp->grad_input) ? align_up((size_t)g.N * g.Cin * g.H * g.W * 4) : 0;
   pl->gw_bytes = (staged && bp->grad_weight) ? align_up((size_t)g.Cout * g.cin_g * g.taps * 4) : 0;
@@ -580,7 +635,7 @@ void make_bwd_plan(const mdcn_bwd_params *bp, const Geom &g, BwdPlan *pl) {
   pl->R = pl->sR = -1;
   pl->WH = pl->WW = pl->sWH = pl->sWW = 0;
   const int path = bp->conv.path == MDCN_PATH_FUSED_SPLIT ? MDCN_PATH_FUSED : bp->conv.path;
-  if (path == MDCN_PATH_DIRECT || g.taps > kBwdTapsMax) return;
+  if (path == MDCN_PATH_DIRECT || g.taps > kBwdTapsMax || f64) return;
   const bool forced = path == MDCN_PATH_FUSED;
   const size_t plane_out = (size_t)g.Ho * g.Wo;
 
@@ -924,6 +979,40 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
   return rc;
 }
 
+// Double precision: grad_input by atomics into the zeroed tensor, everything else
+// has one owner; no workspace.
+int run_backward_f64(const mdcn_bwd_params *bp, const Geom &g, hipStream_t st) {
+  const mdcn_params *p = &bp->conv;
+  const long plane_out = (long)g.Ho * g.Wo;
+  auto blocks_for = [](long n) { return (int)std::max<long>(1, std::min<long>((n + 255) / 256, 1L << 20)); };
+  int rc = MDCN_OK;
+  auto check = [&]() { if (hipGetLastError() != hipSuccess) rc = MDCN_ERR_LAUNCH; };
+  if (bp->grad_input) {
+    const long n_in = (long)g.N * g.Cin * g.H * g.W;
+    hipLaunchKernelGGL(f64_zero_kernel, dim3(blocks_for(n_in)), dim3(256), 0, st, (double *)bp->grad_input, n_in);
+    check();
+    const long total = (long)g.N * g.DG * g.taps * plane_out;
+    hipLaunchKernelGGL(f64_bwd_data_kernel, dim3(blocks_for(total)), dim3(256), 0, st, g, (const double *)p->input,
+                       (const double *)p->offset, (const double *)p->mask, (const double *)p->weight,
+                       (const double *)bp->grad_output, (double *)bp->grad_input, (double *)bp->grad_offset,
+                       (double *)bp->grad_mask, total);
+    check();
+  }
+  if (bp->grad_weight) {
+    const long n_w = (long)g.Cout * g.cin_g * g.taps;
+    hipLaunchKernelGGL(f64_bwd_weight_kernel, dim3((unsigned)std::min<long>(n_w, 1L << 20)), dim3(256), 0, st, g,
+                       (const double *)p->input, (const double *)p->offset, (const double *)p->mask,
+                       (const double *)bp->grad_output, (double *)bp->grad_weight);
+    check();
+  }
+  if (bp->grad_bias) {
+    hipLaunchKernelGGL(f64_bwd_bias_kernel, dim3((unsigned)std::min(g.Cout, 65535)), dim3(256), 0, st, g,
+                       (const double *)bp->grad_output, (double *)bp->grad_bias);
+    check();
+  }
+  return rc;
+}
+
 int check_bwd(const mdcn_bwd_params *bp, Geom *g, bool need_ptrs) {
   if (!bp) return MDCN_ERR_NULL;
   const mdcn_params *p = &bp->conv;
@@ -937,6 +1026,7 @@ int check_bwd(const mdcn_bwd_params *bp, Geom *g, bool need_ptrs) {
   if (data != (bp->grad_offset != nullptr)) return MDCN_ERR_NULL;
   if (p->mask ? (data != (bp->grad_mask != nullptr)) : (bp->grad_mask != nullptr)) return MDCN_ERR_NULL;
   if ((uint64_t)g->N * g->DG * g->taps > 0x7fffffffull) return MDCN_ERR_TOO_LARGE;
+  if (p->dtype == MDCN_F64 && (p->path == MDCN_PATH_FUSED || p->path == MDCN_PATH_FUSED_SPLIT)) return MDCN_ERR_PATH;
   if (p->path == MDCN_PATH_FUSED || p->path == MDCN_PATH_FUSED_SPLIT) {  // asked for the tiled kernels: the shape must allow them
     BwdPlan pl;
     make_bwd_plan(bp, *g, &pl);
@@ -1015,50 +1105,6 @@ int mdcn_forward_noalloc(const mdcn_params *p, void *hip_stream) {
   return run(&q, hip_stream, nullptr);
 }
 
-int mdcn_mfma_probe(int dtype, int waves_per_simd, int zero_data, void *scratch, void *hip_stream, float *tflops) {
-  if (!scratch || !tflops) return MDCN_ERR_NULL;
-  if (dtype != MDCN_BF16 && dtype != MDCN_F16) return MDCN_ERR_DTYPE;
-  if (waves_per_simd < 1 || waves_per_simd > 2) return MDCN_ERR_SHAPE;
-  hipStream_t st = (hipStream_t)hip_stream;
-  // operands: 4096 words of two 16-bit values of magnitude 0.5 .. 2 with random signs and
-  // mantissas (finite in both formats)
-  uint32_t host[4096];
-  uint32_t rng = 12345u;
-  auto next = [&]() { rng = rng * 1664525u + 1013904223u; return rng >> 8; };
-  const uint32_t base = dtype == MDCN_BF16 ? 0x3f00u : 0x3800u;
-  for (int i = 0; i < 4096; ++i) {
-    const uint32_t lo = base + (next() & 0xffu) + ((next() & 1u) << 15);
-    const uint32_t hi = base + (next() & 0xffu) + ((next() & 1u) << 15);
-    host[i] = lo | (hi << 16);
-  }
-  if (hipMemcpyAsync(scratch, host, sizeof(host), hipMemcpyHostToDevice, st) != hipSuccess) return MDCN_ERR_LAUNCH;
-  if (hipStreamSynchronize(st) != hipSuccess) return MDCN_ERR_LAUNCH;
-  const int blocks = num_cus() * waves_per_simd, iters = 20000;
-  hipEvent_t e0, e1;
-  if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) return MDCN_ERR_LAUNCH;
-  auto launch = [&](int n) {
-    if (dtype == MDCN_BF16)
-      hipLaunchKernelGGL(mfma_probe_kernel<bf16_t>, dim3(blocks), dim3(256), 0, st, (const uint4 *)scratch,
-                         (float *)scratch, n, zero_data);
-    else
-      hipLaunchKernelGGL(mfma_probe_kernel<f16_t>, dim3(blocks), dim3(256), 0, st, (const uint4 *)scratch,
-                         (float *)scratch, n, zero_data);
-  };
-  launch(2000);  // warm up (clocks)
-  hipEventRecord(e0, st);
-  launch(iters);
-  hipEventRecord(e1, st);
-  int rc = MDCN_OK;
-  float ms = 0.0f;
-  if (hipEventSynchronize(e1) != hipSuccess || hipEventElapsedTime(&ms, e0, e1) != hipSuccess ||
-      hipGetLastError() != hipSuccess || ms <= 0.0f)
-    rc = MDCN_ERR_LAUNCH;
-  hipEventDestroy(e0);
-  hipEventDestroy(e1);
-  if (rc == MDCN_OK) *tflops = (float)((double)blocks * 4 * iters * 8 * 32768.0 / ms / 1e9);
-  return rc;
-}
-
 int mdcn_forward_timed(const mdcn_params *p, void *hip_stream, float ms[4]) {
   if (!ms) return MDCN_ERR_NULL;
   return run(p, hip_stream, ms);
@@ -1097,6 +1143,7 @@ int mdcn_backward(const mdcn_bwd_params *bp, void *hip_stream) {
     return MDCN_ERR_WORKSPACE;
   hipStream_t st = (hipStream_t)hip_stream;
   switch (p->dtype) {
+    case MDCN_F64: return run_backward_f64(bp, g, st);
     case MDCN_F32: return run_backward_typed<float>(bp, g, pl, st);
     case MDCN_F16: return run_backward_typed<f16_t>(bp, g, pl, st);
     default: return run_backward_typed<bf16_t>(bp, g, pl, st);

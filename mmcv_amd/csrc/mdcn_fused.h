@@ -734,43 +734,4 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
   }
 }
 
-// Back-to-back MFMAs on eight accumulator blocks per wave (the consumers' block
-// shape), operands from `in` (4096 32-bit words) or zeros: what the matrix cores
-// sustain, for the bench to put beside the published peak.
-template <typename E>
-__global__ __launch_bounds__(256) void mfma_probe_kernel(const uint4 *__restrict__ in, float *out, int iters, int zero) {
-  using TR = ElemTraits<E>;
-  const int tid = threadIdx.x;
-  uint4 a[2], b[4];
-#pragma unroll
-  for (int i = 0; i < 2; ++i) a[i] = zero ? make_uint4(0u, 0u, 0u, 0u) : in[(tid * 7 + i * 13) & 1023];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) b[i] = zero ? make_uint4(0u, 0u, 0u, 0u) : in[(tid * 5 + i * 29 + 100) & 1023];
-  f32x16 acc[2][4];
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
-  for (int it = 0; it < iters; ++it) {
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) TR::mma(acc[i][j], a[i], b[j]);
-    if (!zero) {  // keep the operands changing
-      a[0].x ^= (uint32_t)it;
-      b[1].y += 0x00010001u;
-    }
-  }
-  float s = 0.0f;
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) s += acc[i][j][r];
-  if (s == 1.2345f) out[tid] = s;  // (never: keeps the loop alive)
-}
-
 }  // namespace mdcn

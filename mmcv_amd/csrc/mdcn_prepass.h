@@ -103,17 +103,100 @@ __global__ __launch_bounds__(256) void relayout_kernel(Geom g, const E *__restri
       *(uint4 *)(dst_slab + ((long)(g.Hp - 1) * g.Wp) * 128 + (long)i * 16) = zero;
 }
 
+// The same re-layout without LDS, for planes whose channel rows can be read 16
+// bytes at a time (H * W a multiple of 16 / sizeof(E) and a 16-byte aligned
+// tensor).  A thread owns EPV = 16 / sizeof(E) consecutive pixels x EPV
+// consecutive channels: EPV loads of 16 bytes (one channel each), a transpose in
+// registers (16-bit elements: one v_perm_b32 per output word; fp32: none, the
+// words only change names) and EPV stores of 16 bytes (one pixel each).  Eight
+// neighbouring lanes hold the eight channel groups of a pixel run, so a load
+// instruction reads 128 contiguous bytes per channel and a store instruction
+// writes whole 128-byte pixels.  One block = 32 pixel runs x 8 channel groups:
+// one slab of 32 * EPV pixels.  Borders as in relayout_kernel.
+template <typename E, bool BORDER>
+__device__ __forceinline__ void relayout_vec_block(const Geom &g, const E *__restrict__ in, E *__restrict__ xt,
+                                                   int n_pchunks, int b) {
+  constexpr int EPV = 16 / (int)sizeof(E);
+  constexpr int KC = 128 / (int)sizeof(E);
+  constexpr int PXB = 32 * EPV;  // pixels per block
+  const int pc = b % n_pchunks;
+  b /= n_pchunks;
+  const int slabs_total = g.Cin / KC;
+  const int slab = b % slabs_total;
+  const int n = b / slabs_total;
+  const int tid = threadIdx.x;
+  const int cg = tid & 7, pg = tid >> 3;
+  const int plane = g.H * g.W;
+  const int p0 = pc * PXB + pg * EPV;
+  unsigned char *dst_slab =
+      (unsigned char *)xt + (((long)n * slabs_total + slab) * (BORDER ? (long)g.Hp * g.Wp : (long)plane)) * 128;
+  const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+  if (p0 < plane) {  // (plane is a multiple of EPV: the whole run is inside)
+    const E *src = in + ((long)n * g.Cin + slab * KC + cg * EPV) * plane + p0;
+    uint4 r[EPV];
+#pragma unroll
+    for (int j = 0; j < EPV; ++j) r[j] = *(const uint4 *)(src + (long)j * plane);
+    uint4 o[EPV];
+    if constexpr (sizeof(E) == 2) {
+      // r[j] = 8 pixels of channel j; o[i] = 8 channels of pixel i
+      const uint32_t *rw = (const uint32_t *)r;
+      uint32_t *ow = (uint32_t *)o;
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          const uint32_t lo = rw[(2 * a) * 4 + w], hi = rw[(2 * a + 1) * 4 + w];
+          ow[(2 * w) * 4 + a] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);      // low halves: pixel 2w
+          ow[(2 * w + 1) * 4 + a] = __builtin_amdgcn_perm(hi, lo, 0x07060302u);  // high halves: pixel 2w + 1
+        }
+    } else {
+      const uint32_t *rw = (const uint32_t *)r;
+      uint32_t *ow = (uint32_t *)o;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ow[i * 4 + j] = rw[j * 4 + i];
+    }
+    int y = p0 / g.W;
+    int x = p0 - y * g.W;
+#pragma unroll
+    for (int i = 0; i < EPV; ++i) {
+      unsigned char *d = dst_slab + (BORDER ? (long)(y + 1) * g.Wp + (x + 1) : (long)(p0 + i)) * 128 + cg * 16;
+      *(uint4 *)d = o[i];
+      if (BORDER && x == g.W - 1) {
+        *(uint4 *)(d + 128) = zero;
+        *(uint4 *)(d + 256) = zero;
+      }
+      if (++x == g.W) {
+        x = 0;
+        ++y;
+      }
+    }
+  }
+  if (!BORDER) return;
+  if (pc == 0)  // top border row and the left border pixel of the first image row
+    for (int i = tid; i < (g.Wp + 1) * 8; i += 256) *(uint4 *)(dst_slab + (long)i * 16) = zero;
+  if (pc == n_pchunks - 1)  // bottom border row
+    for (int i = tid; i < g.Wp * 8; i += 256)
+      *(uint4 *)(dst_slab + ((long)(g.Hp - 1) * g.Wp) * 128 + (long)i * 16) = zero;
+}
+
+template <typename E, bool BORDER = true>
+__global__ __launch_bounds__(256) void relayout_vec_kernel(Geom g, const E *__restrict__ in, E *__restrict__ xt,
+                                                           int n_pchunks) {
+  relayout_vec_block<E, BORDER>(g, in, xt, n_pchunks, (int)blockIdx.x);
+}
+
 // weight[Cout][Cin/G][kh][kw] -> wp[G][n_ctiles][nk][CT][KC]: for every
 // group, Cout tile and K step (channel slab outer, tap inner) one dense
 // CT x KC tile, K contiguous, zero rows past Cout/G.  The main kernel copies
-// such a tile to LDS with straight 16-byte loads.
+// such a tile to LDS with straight 16-byte loads.  Element idx, idx + stride, ...
 template <typename E>
-__global__ __launch_bounds__(256) void pack_weight_kernel(
-    Geom g, const E *__restrict__ w, E *__restrict__ wp, int CT, int KC,
-    int n_ctiles, int slabs, long total) {
+__device__ __forceinline__ void pack_weight_elems(const Geom &g, const E *__restrict__ w, E *__restrict__ wp, int CT,
+                                                  int KC, int n_ctiles, int slabs, long total, long first,
+                                                  long stride) {
   const int nk = slabs * g.taps;
-  for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
-       idx += (long)gridDim.x * blockDim.x) {
+  for (long idx = first; idx < total; idx += stride) {
     long r = idx;
     const int kc = (int)(r % KC);
     r /= KC;
@@ -133,6 +216,31 @@ __global__ __launch_bounds__(256) void pack_weight_kernel(
     }
     wp[idx] = v;
   }
+}
+
+template <typename E>
+__global__ __launch_bounds__(256) void pack_weight_kernel(
+    Geom g, const E *__restrict__ w, E *__restrict__ wp, int CT, int KC,
+    int n_ctiles, int slabs, long total) {
+  pack_weight_elems<E>(g, w, wp, CT, KC, n_ctiles, slabs, total, (long)blockIdx.x * blockDim.x + threadIdx.x,
+                       (long)gridDim.x * blockDim.x);
+}
+
+// Both pre-passes of a forward call in one launch: the first `pack_blocks`
+// workgroups repack the weights (geometry gw: that of the whole call), the others
+// re-lay the input of one batch chunk (geometry g) as relayout_vec_kernel does.
+// The two are independent, and the small weight repack hides under the copy.
+template <typename E>
+__global__ __launch_bounds__(256) void prepass_kernel(Geom g, const E *__restrict__ in, E *__restrict__ xt,
+                                                      int n_pchunks, Geom gw, const E *__restrict__ w,
+                                                      E *__restrict__ wp, int CT, int KC, int n_ctiles, int slabs,
+                                                      long wtotal, int pack_blocks) {
+  if ((int)blockIdx.x < pack_blocks) {
+    pack_weight_elems<E>(gw, w, wp, CT, KC, n_ctiles, slabs, wtotal, (long)blockIdx.x * 256 + threadIdx.x,
+                         (long)pack_blocks * 256);
+    return;
+  }
+  relayout_vec_block<E, true>(g, in, xt, n_pchunks, (int)blockIdx.x - pack_blocks);
 }
 
 }  // namespace mdcn

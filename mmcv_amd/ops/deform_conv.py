@@ -111,13 +111,13 @@ class DeformConv2dFunction(Function):
             'batch size must be divisible by im2col_step'
         grad_output = grad_output.contiguous()
         if ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
-            grad_input = torch.zeros_like(input)
-            grad_offset = torch.zeros_like(offset)
+            grad_input = torch.zeros_like(input, memory_format=torch.contiguous_format)
+            grad_offset = torch.zeros_like(offset, memory_format=torch.contiguous_format)
             ext_module.deform_conv_backward_input(
                 input, offset, grad_output, grad_input, grad_offset, weight,
                 ctx.bufs_[0], **_ext_kwargs(ctx, weight, step))
         if ctx.needs_input_grad[2]:
-            grad_weight = torch.zeros_like(weight)
+            grad_weight = torch.zeros_like(weight, memory_format=torch.contiguous_format)
             ext_module.deform_conv_backward_parameters(
                 input, offset, grad_output, grad_weight, ctx.bufs_[0],
                 ctx.bufs_[1], scale=1, **_ext_kwargs(ctx, weight, step))
@@ -246,6 +246,7 @@ class DeformConv2dPack(DeformConv2d):
         needs_grad = torch.is_grad_enabled() and (
             x.requires_grad or any(p.requires_grad for p in self.parameters()))
         if self.fuse == 'full' and x.is_cuda and x.dim() == 4 and not needs_grad \
+                and x.dtype != torch.float64 \
                 and not torch.is_autocast_enabled():
             step = min(self.im2col_step, x.size(0))
             assert x.size(0) % step == 0, 'batch size must be divisible by im2col_step'

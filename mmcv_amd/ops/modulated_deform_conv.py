@@ -146,7 +146,9 @@ class ModulatedDeformConv2dFunction(Function):
     @once_differentiable
     def backward(ctx, grad_output: torch.Tensor) -> tuple:
         input, offset, mask, weight, bias = ctx.saved_tensors
-        grads = [torch.zeros_like(t) for t in (input, offset, mask, weight, bias)]
+        # dense gradients whatever the memory format of the saved tensors (the op writes NCHW)
+        grads = [torch.zeros_like(t, memory_format=torch.contiguous_format)
+                 for t in (input, offset, mask, weight, bias)]
         grad_input, grad_offset, grad_mask, grad_weight, grad_bias = grads
         ext_module.modulated_deform_conv_backward(
             input, weight, bias, ctx._bufs[0], offset, mask, ctx._bufs[1],
@@ -306,6 +308,7 @@ class ModulatedDeformConv2dPack(ModulatedDeformConv2d):
         needs_grad = torch.is_grad_enabled() and (
             x.requires_grad or any(p.requires_grad for p in self.parameters()))
         if self.fuse != 'none' and x.is_cuda and x.dim() == 4 and not needs_grad \
+                and x.dtype != torch.float64 \
                 and not torch.is_autocast_enabled():
             return modulated_deform_conv2d_pack(
                 x, self.conv_offset, self.weight, self.bias, self.stride,

@@ -8,9 +8,9 @@ import torch
 
 from mmcv_amd import capi
 
-TOL = {torch.float32: 1e-4, torch.float16: 2e-2, torch.bfloat16: 2e-2}
+TOL = {torch.float32: 1e-4, torch.float16: 2e-2, torch.bfloat16: 2e-2, torch.float64: 1e-12}
 DT = {torch.float32: capi.MDCN_F32, torch.float16: capi.MDCN_F16,
-      torch.bfloat16: capi.MDCN_BF16}
+      torch.bfloat16: capi.MDCN_BF16, torch.float64: capi.MDCN_F64}
 
 
 def pair(v):

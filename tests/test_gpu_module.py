@@ -142,9 +142,9 @@ def test_device_and_shape_errors():
     with pytest.raises(RuntimeError, match='offset must be'):
         modulated_deform_conv2d(case['input'], case['offset'][:, :9], case['mask'],
                                 case['weight'], None, 1, 1)
-    with pytest.raises(RuntimeError, match='not implemented for'):
-        modulated_deform_conv2d(case['input'].double(), case['offset'].double(),
-                                case['mask'].double(), case['weight'].double(), None, 1, 1)
+    with pytest.raises(RuntimeError, match="not implemented for 'Int'"):
+        modulated_deform_conv2d(case['input'].int(), case['offset'].int(),
+                                case['mask'].int(), case['weight'].int(), None, 1, 1)
     # gradients flow (their values are checked in test_gpu_backward.py)
     x = case['input'].clone().requires_grad_(True)
     modulated_deform_conv2d(x, case['offset'], case['mask'], case['weight'], None, 1, 1).sum().backward()
@@ -246,18 +246,3 @@ def test_cfg5_layer_shapes(shape):
         err = rel_err(y[n:n + 1].float().cpu().numpy(), oracle_forward(sub))
         print(f'  cfg5 {shape} sample {n}: err {err:.3e}', flush=True)
         assert err <= TOL[torch.bfloat16], (shape, n, err)
-
-
-def test_mfma_probe_reports_a_plausible_rate():
-    """The measurement-only probe: TFLOP/s of back-to-back MFMAs, for the bench line."""
-    import ctypes
-    from mmcv_amd import capi
-    lib = capi.load()
-    scratch = torch.empty(16384, dtype=torch.uint8, device='cuda')
-    tf = ctypes.c_float()
-    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-    for dtype in (1, 2):
-        rc = lib.mdcn_mfma_probe(dtype, 1, 0, ctypes.c_void_p(scratch.data_ptr()), stream, ctypes.byref(tf))
-        assert rc == 0 and 200.0 < tf.value < 5000.0, (rc, tf.value)
-    assert lib.mdcn_mfma_probe(0, 1, 0, ctypes.c_void_p(scratch.data_ptr()), stream, ctypes.byref(tf)) != 0  # fp32: no
-    assert lib.mdcn_mfma_probe(2, 3, 0, ctypes.c_void_p(scratch.data_ptr()), stream, ctypes.byref(tf)) != 0

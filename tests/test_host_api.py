@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
     assert sorted(names) == sorted(capi.EXPORTS)
     for n in names:
         assert hasattr(lib, n), n
-    assert lib.mdcn_abi_version() == 3
+    assert lib.mdcn_abi_version() == 4
     assert capi.status_string(0) == 'ok'
     assert 'workspace' in capi.status_string(-4)
 
@@ -105,7 +105,7 @@ def test_ext_module_exports():
     from mmcv_amd.utils import ext_loader
     ext = ext_loader.load_ext('_ext', ['modulated_deform_conv_forward',
                                        'modulated_deform_conv_backward'])
-    assert ext.abi_version() == 3
+    assert ext.abi_version() == 4
     with pytest.raises(AssertionError):
         ext_loader.load_ext('_ext', ['no_such_op'])
     with pytest.raises(ImportError):
@@ -226,3 +226,72 @@ def test_dcnv1_python_layer():
     assert not errors
     assert 'dcn.conv_offset.weight' in state and 'dcn.conv_offset.bias' in state
     assert 'dcn_offset.weight' not in state and 'dcn_offset.bias' not in state
+
+
+def _stub_mmcv():
+    """A module tree shaped like the part of mmcv that patch() touches."""
+    import types
+    mmcv = types.ModuleType('mmcv_stub')
+    ops = types.ModuleType('mmcv_stub.ops')
+    mdc = types.ModuleType('mmcv_stub.ops.modulated_deform_conv')
+    dc = types.ModuleType('mmcv_stub.ops.deform_conv')
+    calls = []
+
+    class TheirExt:
+        def modulated_deform_conv_forward(self, *a, **k):
+            calls.append('their_forward')
+
+        def nms(self, *a, **k):
+            return 'their_nms'
+
+    mdc.ext_module = TheirExt()
+    for name in ('ModulatedDeformConv2d', 'ModulatedDeformConv2dPack', 'modulated_deform_conv2d'):
+        setattr(mdc, name, object())
+        setattr(ops, name, getattr(mdc, name))
+    dc.DeformConv2d = ops.DeformConv2d = object()  # (no ext_module: as if mmcv was built without ops)
+    ops.modulated_deform_conv, ops.deform_conv, mmcv.ops = mdc, dc, ops
+
+    class Registry:
+        def __init__(self):
+            self._module_dict = {'DCNv2': 'theirs', 'Conv': 'conv'}
+
+    return mmcv, calls, Registry()
+
+
+def test_patch_rebinds_an_imported_mmcv_and_unpatch_restores_it():
+    import mmcv_amd
+    from mmcv_amd import ops as ours
+    mmcv, calls, reg = _stub_mmcv()
+    before = (mmcv.ops.modulated_deform_conv.ext_module, mmcv.ops.ModulatedDeformConv2dPack, dict(reg._module_dict))
+    done = mmcv_amd.patch(mmcv, registry=reg)
+    assert 'modulated_deform_conv.ext_module' in done and 'MODELS[DCNv2]' in done
+    ext = mmcv.ops.modulated_deform_conv.ext_module
+    # CPU tensors keep going to the module mmcv loaded, ops of other layers too
+    ext.modulated_deform_conv_forward(torch.zeros(1))
+    assert calls == ['their_forward'] and ext.nms() == 'their_nms'
+    # device tensors go to this package's op: here it rejects the bogus call itself
+    class FakeCuda:
+        is_cuda = True
+    with pytest.raises(TypeError):
+        ext.modulated_deform_conv_forward(FakeCuda())
+    assert mmcv.ops.deform_conv.ext_module.deform_conv_forward.__name__ == 'deform_conv_forward'
+    assert mmcv.ops.ModulatedDeformConv2dPack is ours.ModulatedDeformConv2dPack
+    assert mmcv.ops.modulated_deform_conv.modulated_deform_conv2d is ours.modulated_deform_conv2d
+    assert mmcv.ops.DeformConv2d is ours.DeformConv2d
+    assert reg._module_dict['DCNv2'] is ours.ModulatedDeformConv2dPack and reg._module_dict['Conv'] == 'conv'
+    assert reg._module_dict['DCN'] is ours.DeformConv2dPack
+    mmcv_amd.unpatch()
+    assert mmcv.ops.modulated_deform_conv.ext_module is before[0]
+    assert mmcv.ops.ModulatedDeformConv2dPack is before[1]
+    assert reg._module_dict == before[2]
+    assert not hasattr(mmcv.ops.deform_conv, 'ext_module')
+
+
+def test_patch_ext_only_keeps_mmcv_classes():
+    import mmcv_amd
+    mmcv, _, reg = _stub_mmcv()
+    pack = mmcv.ops.ModulatedDeformConv2dPack
+    done = mmcv_amd.patch(mmcv.ops, classes=False, registry=reg)
+    assert done == ['modulated_deform_conv.ext_module', 'deform_conv.ext_module']
+    assert mmcv.ops.ModulatedDeformConv2dPack is pack and reg._module_dict['DCNv2'] == 'theirs'
+    mmcv_amd.unpatch()
