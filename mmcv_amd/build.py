@@ -37,11 +37,35 @@ def _run(cmd):
     subprocess.check_call(cmd)
 
 
-def build_hip(extra=()):
+def build_hip(extra=(), check=True):
+    """Compile the library; with `check`, keep the device assembly of the compile
+    and scan it (asm_check.py) before the library is accepted."""
+    import shutil
+    import tempfile
     os.makedirs(LIBDIR, exist_ok=True)
     hipcc = os.path.join(ROCM, 'bin', 'hipcc')
-    _run([hipcc, *HIPCC_FLAGS, *extra, '-I', os.path.join(ROOT, 'include'),
-          '-o', HIP_LIB, os.path.join(CSRC, 'mdcn_api.hip')])
+    cmd = [hipcc, *HIPCC_FLAGS, *extra, '-I', os.path.join(ROOT, 'include')]
+    src = os.path.join(CSRC, 'mdcn_api.hip')
+    if not check:
+        _run([*cmd, '-o', HIP_LIB, src])
+        return HIP_LIB
+    from . import asm_check
+    tmp = tempfile.mkdtemp(prefix='mdcn_build_')
+    try:
+        out = os.path.join(tmp, 'libmdcn_hip.so')
+        print(' '.join([*cmd, '-save-temps=obj', '-o', out, src]), flush=True)
+        subprocess.check_call([*cmd, '-save-temps=obj', '-o', out, src], cwd=tmp)
+        asm = [os.path.join(tmp, f) for f in os.listdir(tmp) if f.endswith('.s') and 'gfx950' in f]
+        if not asm:
+            raise RuntimeError('no device assembly found to check')
+        bad = sum(asm_check.check_file(f) for f in asm)
+        if bad:
+            raise RuntimeError(f'{bad} inline-asm vector-memory instruction(s) read a scalar register too soon '
+                               'after a vector instruction wrote it (see above)')
+        print(f'asm_check: {len(asm)} device assembly file(s) clean', flush=True)
+        shutil.move(out, HIP_LIB)
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
     return HIP_LIB
 
 

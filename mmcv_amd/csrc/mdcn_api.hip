@@ -136,6 +136,8 @@ struct Plan {
   int n_chunk;       // images per launch of the fused path
   size_t xt_bytes;   // channels-last copy of one chunk
   size_t wp_bytes;   // packed weights
+  size_t split_bytes;  // eight-wave kernel: buffers and counters of the tiles it cuts along K (may be left out)
+  int split_wgs;     // ... one buffer and one counter per workgroup of its grid
   // pack-level call only
   int CO, CO_pad;    // conv_offset channels: 3 (2 when unmodulated) * DG * taps, rounded up to 32
   int mask_kind;     // kMaskLogit, or kMaskNone when unmodulated
@@ -149,13 +151,21 @@ struct PackExtra {
   void *raw;
 };
 
+// 16-bit tensors, 256-channel tiles, one deformable group, enough K steps: the eight-wave kernel
+bool uses_fused2(const mdcn_params *p, const Geom &g, const Plan &pl) {
+  if (pl.CT != 256 || elem_size(p->dtype) != 2 || g.DG != 1 || p->path == MDCN_PATH_FUSED_SPLIT) return false;
+  const int nk_pad = (pl.slabs * g.taps + kF2Unroll - 1) / kF2Unroll * kF2Unroll;
+  return nk_pad >= kF2MinSteps;
+}
+
 int make_plan(const mdcn_params *p, const Geom &g, Plan *pl) {
   const bool ok = fused_ok(p, g);
   if ((p->path == MDCN_PATH_FUSED || p->path == MDCN_PATH_FUSED_SPLIT) && !ok) return MDCN_ERR_PATH;
   if (p->input_nhwc && (!ok || p->path == MDCN_PATH_DIRECT)) return MDCN_ERR_PATH;  // in-place reads: fused kernel only
   pl->fused = ok && p->path != MDCN_PATH_DIRECT;
   pl->CT = pl->KC = pl->n_ctiles = pl->slabs = pl->n_chunk = 0;
-  pl->xt_bytes = pl->wp_bytes = pl->owp_bytes = pl->raw_bytes = 0;
+  pl->xt_bytes = pl->wp_bytes = pl->owp_bytes = pl->raw_bytes = pl->split_bytes = 0;
+  pl->split_wgs = 0;
   pl->CO = 3 * g.DG * g.taps;
   pl->CO_pad = (pl->CO + 31) / 32 * 32;
   pl->mask_kind = kMaskLogit;
@@ -169,6 +179,10 @@ int make_plan(const mdcn_params *p, const Geom &g, Plan *pl) {
   pl->n_chunk = (int)std::min<uint64_t>((uint64_t)g.N, std::max<uint64_t>(1, g_fwd_pass_bytes / img));
   pl->xt_bytes = p->input_nhwc ? 0 : align_up((size_t)img * pl->n_chunk);
   pl->wp_bytes = align_up((size_t)g.G * pl->n_ctiles * pl->slabs * g.taps * pl->CT * pl->KC * es);
+  if (uses_fused2(p, g, *pl)) {
+    pl->split_wgs = num_cus() / 8 * 8;
+    pl->split_bytes = align_up((size_t)pl->split_wgs * kPT * kF2CT * 4) + align_up((size_t)pl->split_wgs * 4);
+  }
   return MDCN_OK;
 }
 
@@ -191,7 +205,8 @@ int make_pack_plan(const mdcn_pack_params *pp, const Geom &g, Plan *pl) {
       if (pl->CO_pad > 128) {  // accumulator blocks of the conv_offset kernel
         if (p->path == MDCN_PATH_FUSED || p->path == MDCN_PATH_FUSED_SPLIT) return MDCN_ERR_PATH;
         pl->fused = false;
-        pl->xt_bytes = pl->wp_bytes = 0;
+        pl->xt_bytes = pl->wp_bytes = pl->split_bytes = 0;
+        pl->split_wgs = 0;
       } else {
         pl->owp_bytes = align_up((size_t)(g.Cin / pl->KC) * g.taps * 4 * (pl->CO_pad / 32) * 64 * 16);
         pl->raw_bytes = align_up((size_t)pl->n_chunk * plane * pl->CO_pad * es);
@@ -360,6 +375,9 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
     E *raw_pm = (E *)(ws + pl.xt_bytes + pl.wp_bytes + pl.owp_bytes);
     const bool own_oconv = px && px->offset_weight;
     const int cof = pl.CO_pad / 32;
+    float *split_part = (float *)(ws + pl.xt_bytes + pl.wp_bytes + pl.owp_bytes + pl.raw_bytes);
+    uint32_t *split_cnt = (uint32_t *)((unsigned char *)split_part + align_up((size_t)pl.split_wgs * kPT * kF2CT * 4));
+    if (!pl.split_bytes) split_part = nullptr, split_cnt = nullptr;
 
     // weights: once per call -- inside the launch that re-lays the first batch chunk when the
     // input allows the vector re-layout (whole 16-byte runs per channel row), else on their own
@@ -373,7 +391,7 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
         const int grid = (int)std::min<long>((wtotal + 255) / 256, 1L << 16);
         hipLaunchKernelGGL(pack_weight_kernel<E>, dim3(grid), dim3(256), 0, st, g,
                            (const E *)p->weight, wp, pl.CT, pl.KC, pl.n_ctiles,
-                           pl.slabs, wtotal);
+                           pl.slabs, wtotal, split_cnt, pl.split_wgs);
         if (hipGetLastError() != hipSuccess) rc = MDCN_ERR_LAUNCH;
         packed = true;
       }
@@ -399,7 +417,7 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
           const int pack_blocks = (int)std::max<long>(1, std::min<long>(wtotal / (256 * 8), 512));
           hipLaunchKernelGGL(prepass_kernel<E>, dim3((unsigned)(blocks + pack_blocks)), dim3(256), 0, st, gc, in, xt,
                              n_pchunks, g, (const E *)p->weight, wp, pl.CT, pl.KC, pl.n_ctiles, pl.slabs, wtotal,
-                             pack_blocks);
+                             pack_blocks, split_cnt, pl.split_wgs);
           packed = true;
         } else {
           hipLaunchKernelGGL((relayout_vec_kernel<E, true>), dim3((unsigned)blocks), dim3(256), 0, st, gc, in, xt,
@@ -476,6 +494,9 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
                            p->mask ? (const E *)p->mask + (size_t)n0 * g.DG * g.taps * plane_out : nullptr, g);
       }
       fa.prof = nullptr;
+      fa.split_max = pl.split_bytes ? kF2SplitMax : 0;
+      fa.split_part = split_part;
+      fa.split_cnt = split_cnt;
 #if defined(MDCN_F2_PROFILE) && MDCN_F2_PROFILE
       {  // profiling build: phase sums land behind the packed weights (the workspace is over-allocated by the harness)
         static void *prof_buf = nullptr;
@@ -562,10 +583,12 @@ int run(const mdcn_params *p, void *stream, float *ms, const mdcn_pack_params *p
     if (pp) return MDCN_ERR_DTYPE;  // the pack-level call has no double-precision form
     return run_f64(p, g, (hipStream_t)stream, ms);
   }
+  // (the split-tile buffers come last and are optional: a workspace without them runs unsplit)
   const size_t need = pl.xt_bytes + pl.wp_bytes + pl.owp_bytes + pl.raw_bytes;
   if (need > 0 && (!p->workspace || p->workspace_bytes < need ||
                    ((uintptr_t)p->workspace % kAlign) != 0))
     return MDCN_ERR_WORKSPACE;
+  if (p->workspace_bytes < need + pl.split_bytes) pl.split_bytes = 0, pl.split_wgs = 0;
   hipStream_t st = (hipStream_t)stream;
   switch (p->dtype) {
     case MDCN_F32: return run_typed<float>(p, g, pl, st, ms, px);
@@ -1081,7 +1104,7 @@ size_t mdcn_workspace_bytes(const mdcn_params *p) {
   if (check_params(p, &g, false) != MDCN_OK) return 0;
   Plan pl;
   if (make_plan(p, g, &pl) != MDCN_OK) return 0;
-  return pl.fused ? pl.xt_bytes + pl.wp_bytes : 0;
+  return pl.fused ? pl.xt_bytes + pl.wp_bytes + pl.split_bytes : 0;
 }
 
 int mdcn_forward(const mdcn_params *p, void *hip_stream) {
@@ -1115,7 +1138,7 @@ size_t mdcn_pack_workspace_bytes(const mdcn_pack_params *pp) {
   if (!pp || check_params(&pp->conv, &g, false) != MDCN_OK) return 0;
   Plan pl;
   if (make_pack_plan(pp, g, &pl) != MDCN_OK) return 0;
-  return pl.xt_bytes + pl.wp_bytes + pl.owp_bytes + pl.raw_bytes;
+  return pl.xt_bytes + pl.wp_bytes + pl.owp_bytes + pl.raw_bytes + pl.split_bytes;
 }
 
 int mdcn_pack_forward(const mdcn_pack_params *pp, void *hip_stream) {

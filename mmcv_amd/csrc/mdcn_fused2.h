@@ -69,9 +69,10 @@ static_assert(kF2VmBlend < 64 && kF2VmBar < 64, "vmcnt holds 6 bits");
 static_assert(kF2Unroll % kF2Sets == 0 && kF2Unroll % 2 == 0 && kF2Unroll % kF2Slots == 0, "static indices");
 
 constexpr int kF2Taps = kTapsSmall;    // table capacity (kh * kw)
+constexpr int kF2SplitMax = 4;         // parts a tile of the schedule's last round is cut into at most
 constexpr int kF2MinSteps = 18;        // padded steps per tile the streaming needs (the next table is built in round 2)
 constexpr size_t fused2_lds_bytes() {
-  return (size_t)2 * kPT * kRowB + (size_t)kF2Slots * kF2CT * kRowB + (size_t)2 * kPT * kF2Taps * 12;
+  return (size_t)2 * kPT * kRowB + (size_t)kF2Slots * kF2CT * kRowB + (size_t)2 * kPT * kF2Taps * 12 + 16;
 }
 
 // 16 bytes per lane from `base` (two SGPRs) + 32-bit byte offset + immediate
@@ -226,6 +227,7 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
   __shared__ uint4 Ws[kF2Slots][CT * kRowChunks];        // weight tiles
   __shared__ uint32_t tpix[2][TBL];                      // (pixel, tap) tables, [tap][PT]: corner byte offset
   __shared__ uint2 tws[2][TBL];                          // ... and the blend weights
+  __shared__ uint32_t part_arrived;                      // parts of a split tile that were there before this one
 
   const Geom &g = a.g;
   const int taps = g.taps;
@@ -265,30 +267,58 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
   const uint32_t wlane = (uint32_t)(wave * kF2WD) * 1024u +
                          (uint32_t)((lane >> 3) * kRowB + (((lane & 7) ^ swz(lane >> 3)) * 16));
 
-  // XCD-aware persistent schedule (as in fused_kernel): this workgroup's tiles
-  // are first, first + stride, ... below tile_end
+  // XCD-aware persistent schedule (as in fused_kernel): XCD x owns a contiguous run
+  // of tiles and hands them out round robin to its `stride` workgroups.  The run
+  // rarely is a multiple of `stride`: the last round has r < stride tiles, and
+  // without further ado r workgroups would compute a whole tile while the others
+  // wait.  Instead each of those r tiles is cut along K into f = stride / r parts
+  // (whole rounds of kF2Unroll steps, at most a.split_max parts), one part per
+  // workgroup: a "unit" is a tile together with a range of K steps, every
+  // workgroup walks whole tiles first and at most one part last.  The parts of a
+  // tile meet in memory (see the epilogue).
   const int total_tiles = a.n_ptiles * a.n_ctiles * g.G;
   const int xcd = (int)(blockIdx.x & 7);
   const int stride = (int)(gridDim.x >> 3);
   const int chunk = (total_tiles + 7) >> 3;
-  const int first = xcd * chunk + (int)(blockIdx.x >> 3);
+  const int wg = (int)(blockIdx.x >> 3);
+  const int first = xcd * chunk + wg;
   const int tile_end = min((xcd + 1) * chunk, total_tiles);
-  if (first >= tile_end) return;
-  const int T = (tile_end - first + stride - 1) / stride;
+  const int chunk_x = max(tile_end - xcd * chunk, 0);
+  const int full_rounds = chunk_x / stride;
+  const int rest = chunk_x - full_rounds * stride;       // tiles of the last, partial round
+  int parts = 1;
+  if (a.split_max > 1 && rest > 0) parts = min(min(stride / rest, a.split_max), nk_pad / kF2Unroll);
+  const bool split = parts > 1;
+  const int T_full = full_rounds + ((!split && wg < rest) ? 1 : 0);
+  const bool has_part = split && wg < rest * parts;
+  const int T = T_full + (has_part ? 1 : 0);
+  if (T == 0) return;
+  // this workgroup's part: tile, index among the tile's parts, K range
+  const int part_tile = xcd * chunk + full_rounds * stride + wg / parts;
+  const int part_idx = wg - (wg / parts) * parts;
+  const int part_kb = (part_idx * (nk_pad / kF2Unroll) / parts) * kF2Unroll;
+  const int part_pad = ((part_idx + 1) * (nk_pad / kF2Unroll) / parts) * kF2Unroll - part_kb;
+  const int part_n = min(nk - part_kb, part_pad);
+  // unit t: first step, number of steps, padded number of steps (macros rather than closures: closures that
+  // capture closures keep their captures in memory)
+#define MDCN_F2_IS_PART(t) (has_part && (t) == T_full)
+#define MDCN_F2_UNIT_KB(t) (MDCN_F2_IS_PART(t) ? part_kb : 0)
+#define MDCN_F2_UNIT_N(t) (MDCN_F2_IS_PART(t) ? part_n : nk)
+#define MDCN_F2_UNIT_PAD(t) (MDCN_F2_IS_PART(t) ? part_pad : nk_pad)
 
-  auto decode = [&](int t, int &ctile, int &grp, int &p0) {
-    int L = first + t * stride;
+  auto decode = [&](int t, int &ctile, int &grp, int &p0) __attribute__((always_inline)) {
+    int L = MDCN_F2_IS_PART(t) ? part_tile : first + t * stride;
     ctile = L % a.n_ctiles;
     L /= a.n_ctiles;
     grp = L % g.G;
     p0 = (L / g.G) * PT;
   };
-  auto weights_of = [&](int t) {
+  auto weights_of = [&](int t) __attribute__((always_inline)) {
     int ctile, grp, p0;
     decode(t, ctile, grp, p0);
-    return (const unsigned char *)a.wp + ((size_t)(grp * a.n_ctiles + ctile) * nk) * (size_t)kWTile;
+    return (const unsigned char *)a.wp + ((size_t)(grp * a.n_ctiles + ctile) * nk + MDCN_F2_UNIT_KB(t)) * (size_t)kWTile;
   };
-  auto slab0_of = [&](int t) {
+  auto slab0_of = [&](int t) __attribute__((always_inline)) {
     int ctile, grp, p0;
     decode(t, ctile, grp, p0);
     return grp * g.cin_g / KC;
@@ -349,9 +379,11 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
   // of tile 0, 1, ...; steps nk .. nk_pad - 1 repeat the last real step (loads
   // nobody uses, which keep the wait counts constant).  Past the last tile the
   // gather and weight cursors stay where they are.
-  int g_t = 0, g_s = 0, g_tap = 0, g_slab = 0, g_slab0 = slab0_of(0);  // gather
-  int b_t = 0, b_s = 0, b_tap = 0;                                     // blend
-  int w_t = 0, w_s = 0;                                                // weight copies
+  // (a unit that is a part starts in the middle of the K range)
+  int g_t = 0, g_s = 0, g_slab = MDCN_F2_UNIT_KB(0) / taps, g_tap = MDCN_F2_UNIT_KB(0) - g_slab * taps, g_slab0 = slab0_of(0);  // gather
+  int g_n = MDCN_F2_UNIT_N(0), g_pad = MDCN_F2_UNIT_PAD(0);
+  int b_t = 0, b_s = 0, b_tap = g_tap, b_n = g_n, b_pad = g_pad;       // blend
+  int w_t = 0, w_s = 0, w_n = g_n, w_pad = g_pad;                      // weight copies
   const unsigned char *w_ptr = weights_of(0);
 
   // gather registers: sets x two halves of the 128-byte row x four corners
@@ -364,18 +396,22 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
     o_bl = o_tl + a.row_bytes;
     o_br = o_bl + pxb;
     ++g_s;
-    if (g_s < nk) {
+    if (g_s < g_n) {
       if (++g_tap == taps) {
         g_tap = 0;
         ++g_slab;
       }
-    } else if (g_s == nk_pad) {
+    } else if (g_s == g_pad) {
       if (g_t + 1 < T) {
         ++g_t;
-        g_s = g_tap = g_slab = 0;
+        g_s = 0;
+        g_slab = MDCN_F2_UNIT_KB(g_t) / taps;
+        g_tap = MDCN_F2_UNIT_KB(g_t) - g_slab * taps;
+        g_n = MDCN_F2_UNIT_N(g_t);
+        g_pad = MDCN_F2_UNIT_PAD(g_t);
         g_slab0 = slab0_of(g_t);
       } else {
-        g_s = nk_pad - 1;
+        g_s = g_pad - 1;
       }
     }
   };
@@ -395,7 +431,7 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
 
   int islot = 0;  // ring slot of the next weight tile to issue
   auto issue_weights = [&](bool advance) {
-    const int kk = min(w_s, nk - 1);
+    const int kk = min(w_s, w_n - 1);
     const uint32_t voff = (uint32_t)kk * kWTile + wlane;
     const uint32_t voff_odd = voff ^ 32u;
     const uint32_t dst = lds_w + (uint32_t)islot * kWTile + (uint32_t)(wave * kF2WD) * 1024u;
@@ -412,13 +448,15 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
     }
     if (!advance) return;
     islot = (islot == kF2Slots - 1) ? 0 : islot + 1;
-    if (++w_s == nk_pad) {
+    if (++w_s == w_pad) {
       if (w_t + 1 < T) {
         ++w_t;
         w_s = 0;
+        w_n = MDCN_F2_UNIT_N(w_t);
+        w_pad = MDCN_F2_UNIT_PAD(w_t);
         w_ptr = weights_of(w_t);
       } else {
-        w_s = nk_pad - 1;
+        w_s = w_pad - 1;
       }
     }
   };
@@ -449,22 +487,26 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
       }                                                                                 \
       MDCN_F2_GATHER_HALF(gs[SI], 1);                                                   \
       ++b_s;                                                                            \
-      if (b_s < nk) {                                                                   \
+      if (b_s < b_n) {                                                                  \
         if (++b_tap == taps) b_tap = 0;                                                 \
-      } else if (b_s == nk_pad) {                                                       \
+      } else if (b_s == b_pad) {                                                        \
         ++b_t;                                                                          \
-        b_s = b_tap = 0;                                                                \
+        b_s = 0;                                                                        \
+        b_tap = MDCN_F2_UNIT_KB(b_t) % taps;                                                    \
+        b_n = MDCN_F2_UNIT_N(b_t);                                                              \
+        b_pad = MDCN_F2_UNIT_PAD(b_t);                                                          \
       }                                                                                 \
     }                                                                                   \
   } while (0)
 
   f32x16 acc[NB][MB];
   int rslot = 0;  // ring slot of the weight tile the next MFMA step reads
+  int c_n = 0;  // steps of the unit the consume side is in
   auto mfma_step = [&](int k) {
     const uint32_t xb = lds_x + ((k & 1) ? kXTile : 0u) + xa0;
     const uint32_t wb = lds_w + (uint32_t)rslot * kWTile + wa0;
     rslot = (rslot == kF2Slots - 1) ? 0 : rslot + 1;
-    if (k >= nk) return;
+    if (k >= c_n) return;
     u32x4 xf[4][NB], wf[4][MB];
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
@@ -568,7 +610,9 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[nb][mb][r] = 0.0f;
 
-    for (int k = 0; k < nk_pad; k += kF2Unroll) {
+    c_n = MDCN_F2_UNIT_N(t);
+    const int c_pad = MDCN_F2_UNIT_PAD(t);
+    for (int k = 0; k < c_pad; k += kF2Unroll) {
       if (k == kF2Unroll && t + 1 < T) {
         // the next tile's table: its buffer was last read in the previous tile, its
         // first reader is the gather cursor near the end of this one
@@ -585,12 +629,100 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
       MDCN_F2_STEP(k + 5, 0);
     }
 
+    // ---- a part of a tile: the parts meet in memory.  Every part stores its
+    // accumulators (fp32, register order) and counts itself in; the part that
+    // arrives last adds all of them up in index order -- so the sum does not
+    // depend on who was last -- and goes on to the epilogue; the others are done.
+    // Nobody waits for anybody.  The last part also resets the counter, which is
+    // thereby zero again for the next launch.  The partial sums are written and
+    // read with device-coherent stores and loads (sc1), which go past the caches
+    // that are private to a CU or an XCD, so no cache has to be written back or
+    // invalidated as a whole; a wave's stores have completed (wait on the
+    // vector-memory counter) before its workgroup counts itself in.
+    bool store_tile = true;
+    if (MDCN_F2_IS_PART(t)) {
+      // First of all nothing is in flight any more: the gathers the cursors issued past the last step
+      // have landed, and every gather register counts as read here, so none of them is handed to another
+      // value while a load may still write it.
+#pragma unroll
+      for (int si = 0; si < kF2Sets; ++si)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) MDCN_VMWAIT4(0, gs[si][h][0], gs[si][h][1], gs[si][h][2], gs[si][h][3]);
+      const int tslot = xcd * stride + wg / parts;                       // the tile's counter
+      const unsigned char *pbase =
+          (const unsigned char *)a.split_part + (size_t)(xcd * stride + (wg / parts) * parts) * (size_t)(PT * CT * 4);
+      const unsigned char *mine = pbase + (size_t)part_idx * (size_t)(PT * CT * 4);
+      // a lane's 64 values travel as 16 quads of 16 bytes; quad j of the wave's lanes is one 1 KiB run.
+      // (The offset is opaque to the optimiser, which would otherwise form the addresses below once,
+      // ahead of the tile loop, and keep them -- spilled -- across the K loop.)
+      uint32_t voff = (uint32_t)((wave * 16 * 64 + lane) * 16);
+      asm volatile("" : "+v"(voff));
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+          for (int qd = 0; qd < 4; ++qd) {
+            const f32x16 &c = acc[nb][mb];
+            const f32x4 v = {c[4 * qd], c[4 * qd + 1], c[4 * qd + 2], c[4 * qd + 3]};
+            const uint32_t vo = voff + (uint32_t)(((nb * MB + mb) * 4 + qd) * 1024);
+            // (s_nop: the compiler may have written the base's scalar registers with a vector instruction --
+            // a reload of spilled scalars -- right in front of this statement, and a vector-memory
+            // instruction must not read such a register within the next five issue slots; the compiler
+            // keeps that distance for its own instructions but does not look into assembly text)
+            asm volatile("s_nop 4\n\tglobal_store_dwordx4 %0, %1, %2 sc1" : : "v"(vo), "v"(v), "s"(mine) : "memory");
+          }
+      // this wave's stores -- and whatever gathers and weight copies it still had in flight -- are done
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      if (tid == 0)
+        part_arrived = __hip_atomic_fetch_add((uint32_t *)a.split_cnt + tslot, 1u, __ATOMIC_RELAXED,
+                                              __HIP_MEMORY_SCOPE_AGENT);
+      __syncthreads();
+      store_tile = part_arrived == (uint32_t)(parts - 1);
+      if (store_tile) {
+        // the gather registers are free now (nothing is in flight): sets 0 and 1 take the 16 quads of a part
+        // (two parts: a + b is the same in either order, so the last one adds the other's values to
+        // the ones it still holds; more parts: everything from memory, in index order)
+        const bool two = parts == 2;
+        const unsigned char *src = two ? pbase + (size_t)(1 - part_idx) * (size_t)(PT * CT * 4) : pbase;
+        for (int i = two ? 1 : 0; i < parts; ++i) {
+#pragma unroll
+          for (int j = 0; j < 16; ++j) {
+            const uint32_t vo = voff + (uint32_t)(j * 1024);
+            asm volatile("s_nop 4\n\tglobal_load_dwordx4 %0, %1, %2 sc1"
+                         : "=v"(gs[j >> 3][(j >> 2) & 1][j & 3])
+                         : "v"(vo), "s"(src));
+          }
+          MDCN_VMWAIT4(0, gs[0][0][0], gs[0][0][1], gs[0][0][2], gs[0][0][3]);
+          MDCN_VMWAIT4(0, gs[0][1][0], gs[0][1][1], gs[0][1][2], gs[0][1][3]);
+          MDCN_VMWAIT4(0, gs[1][0][0], gs[1][0][1], gs[1][0][2], gs[1][0][3]);
+          MDCN_VMWAIT4(0, gs[1][1][0], gs[1][1][1], gs[1][1][2], gs[1][1][3]);
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+              for (int qd = 0; qd < 4; ++qd) {
+                const int j = (nb * MB + mb) * 4 + qd;
+                const f32x4 v = __builtin_bit_cast(f32x4, gs[j >> 3][(j >> 2) & 1][j & 3]);
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                  acc[nb][mb][4 * qd + e] = i == 0 ? v[e] : acc[nb][mb][4 * qd + e] + v[e];
+              }
+          src += PT * CT * 4;
+        }
+        if (tid == 0)
+          __hip_atomic_store((uint32_t *)a.split_cnt + tslot, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+
     // ---- epilogue: bias, one rounding, NCHW store straight from the accumulators.
     // Accumulator block (A = samples, B = weights): register r of lane l holds
     //   pixel = (r/4)*8 + (l/32)*4 + r%4,  channel = l%32.
     // The two halves of the wave exchange packed pixel pairs, after which a lane
     // holds 8 consecutive pixels = 16 bytes of one channel.
-    {
+    if (store_tile) {
       int ctile, grp, p0;
       decode(t, ctile, grp, p0);
       E *out = (E *)a.out;
@@ -660,6 +792,10 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
   // copies issued past the last step must have landed before the workgroup gives up its LDS
   MDCN_VMWAIT4(0, gs[0][0][0], gs[0][1][0], gs[1][0][0], gs[2][1][0]);
 #undef MDCN_F2_STEP
+#undef MDCN_F2_IS_PART
+#undef MDCN_F2_UNIT_KB
+#undef MDCN_F2_UNIT_N
+#undef MDCN_F2_UNIT_PAD
 #undef MDCN_F2_BLOCK
 #undef MDCN_F2_GATHER
 #undef MDCN_F2_GATHER_HALF

@@ -191,10 +191,12 @@ __global__ __launch_bounds__(256) void relayout_vec_kernel(Geom g, const E *__re
 // group, Cout tile and K step (channel slab outer, tap inner) one dense
 // CT x KC tile, K contiguous, zero rows past Cout/G.  The main kernel copies
 // such a tile to LDS with straight 16-byte loads.  Element idx, idx + stride, ...
+// Also clears the `zero_n` words at `zero_ptr` (the main kernel's split-tile counters).
 template <typename E>
 __device__ __forceinline__ void pack_weight_elems(const Geom &g, const E *__restrict__ w, E *__restrict__ wp, int CT,
                                                   int KC, int n_ctiles, int slabs, long total, long first,
-                                                  long stride) {
+                                                  long stride, uint32_t *__restrict__ zero_ptr, int zero_n) {
+  for (long i = first; i < zero_n; i += stride) zero_ptr[i] = 0u;
   const int nk = slabs * g.taps;
   for (long idx = first; idx < total; idx += stride) {
     long r = idx;
@@ -221,9 +223,9 @@ __device__ __forceinline__ void pack_weight_elems(const Geom &g, const E *__rest
 template <typename E>
 __global__ __launch_bounds__(256) void pack_weight_kernel(
     Geom g, const E *__restrict__ w, E *__restrict__ wp, int CT, int KC,
-    int n_ctiles, int slabs, long total) {
+    int n_ctiles, int slabs, long total, uint32_t *__restrict__ zero_ptr, int zero_n) {
   pack_weight_elems<E>(g, w, wp, CT, KC, n_ctiles, slabs, total, (long)blockIdx.x * blockDim.x + threadIdx.x,
-                       (long)gridDim.x * blockDim.x);
+                       (long)gridDim.x * blockDim.x, zero_ptr, zero_n);
 }
 
 // Both pre-passes of a forward call in one launch: the first `pack_blocks`
@@ -234,10 +236,11 @@ template <typename E>
 __global__ __launch_bounds__(256) void prepass_kernel(Geom g, const E *__restrict__ in, E *__restrict__ xt,
                                                       int n_pchunks, Geom gw, const E *__restrict__ w,
                                                       E *__restrict__ wp, int CT, int KC, int n_ctiles, int slabs,
-                                                      long wtotal, int pack_blocks) {
+                                                      long wtotal, int pack_blocks,
+                                                      uint32_t *__restrict__ zero_ptr, int zero_n) {
   if ((int)blockIdx.x < pack_blocks) {
     pack_weight_elems<E>(gw, w, wp, CT, KC, n_ctiles, slabs, wtotal, (long)blockIdx.x * 256 + threadIdx.x,
-                         (long)pack_blocks * 256);
+                         (long)pack_blocks * 256, zero_ptr, zero_n);
     return;
   }
   relayout_vec_block<E, true>(g, in, xt, n_pchunks, (int)blockIdx.x - pack_blocks);

@@ -188,8 +188,17 @@ def test_full_size_configs(name):
         rev = dict(dev)
         for k in ('input', 'offset', 'mask'):
             rev[k] = dev[k].flip(0).contiguous()
-        y_rev = capi_forward(rev, path=capi.PATH_FUSED)
-        assert torch.equal(y_rev.flip(0), y)
+        # A tile's sum does not depend on where in the batch its image sits -- as long as one workgroup
+        # forms it.  (With the split buffers in the workspace, tiles of the schedule's last round are cut
+        # along K and their parts added in fp32, which rounds differently from one long sum.)
+        y_one = capi_forward(dev, path=capi.PATH_FUSED, unsplit=True)
+        y_rev = capi_forward(rev, path=capi.PATH_FUSED, unsplit=True)
+        assert torch.equal(y_rev.flip(0), y_one)
+        # cut tiles: same result on every run, and within an output ulp or so of the uncut sums
+        assert torch.equal(capi_forward(dev, path=capi.PATH_FUSED), y)
+        diff = (y.float() - y_one.float()).abs()
+        assert float(diff.max() / y_one.float().abs().max()) <= (1e-6 if dtype == torch.float32 else 4e-3)
+        assert float((diff > 0).float().mean()) < 0.02
 
 
 def test_full_size_zero_offset_matches_conv2d():

@@ -67,7 +67,10 @@ def test_eligibility_and_workspace():
     assert lib.mdcn_fused_eligible(ctypes.byref(p)) == 1
     ws = lib.mdcn_workspace_bytes(ctypes.byref(p))
     assert ws >= 16 * 102 * 154 * 256 * 2 + 256 * 256 * 9 * 2
-    assert ws < 1.02 * (16 * 102 * 154 * 256 * 2 + 256 * 256 * 9 * 2) + 4096
+    # ... and, for 16-bit 256-channel tiles, one 128 x 256 fp32 buffer and a counter per workgroup
+    # for the tiles that are cut along K (256 workgroups when no device tells the CU count)
+    split = 256 * 128 * 256 * 4 + 256 * 4
+    assert ws < 1.02 * (16 * 102 * 154 * 256 * 2 + 256 * 256 * 9 * 2) + split + 4096
     # a K step is 128 bytes of channels: Cin/groups and Cin/deform_groups must be
     # multiples of 32 (fp32) resp. 64 (fp16, bf16)
     p = capi.make_params(capi.MDCN_F32, 1, 32, 8, 8, 4, 3, 3)
@@ -295,3 +298,39 @@ def test_patch_ext_only_keeps_mmcv_classes():
     assert done == ['modulated_deform_conv.ext_module', 'deform_conv.ext_module']
     assert mmcv.ops.ModulatedDeformConv2dPack is pack and reg._module_dict['DCNv2'] == 'theirs'
     mmcv_amd.unpatch()
+
+
+def test_asm_check_flags_scalar_written_too_close_to_inline_vector_memory():
+    """The build's scan of the device assembly (mmcv_amd/asm_check.py) on synthetic text."""
+    from mmcv_amd import asm_check
+    bad = '''
+	v_readlane_b32 s7, v253, 57
+	;;#ASMSTART
+	global_store_dwordx4 v1, v[66:69], s[6:7] sc1
+	;;#ASMEND
+'''
+    hits = asm_check.violations(bad)
+    assert len(hits) == 1 and hits[0][2] == [7] and hits[0][3] == 0
+    # enough wait states, another register, or an instruction the compiler emitted itself: fine
+    ok = '''
+	v_readlane_b32 s7, v253, 57
+	;;#ASMSTART
+	s_nop 4
+	global_store_dwordx4 v1, v[66:69], s[6:7] sc1
+	;;#ASMEND
+	v_readlane_b32 s9, v253, 58
+	;;#ASMSTART
+	global_load_dwordx4 v[2:5], v1, s[6:7] offset:64
+	;;#ASMEND
+	v_readfirstlane_b32 s10, v4
+	s_nop 4
+	global_load_dword v9, v1, s[10:11]
+	v_readlane_b32 s12, v253, 1
+	global_load_dword v9, v1, s[12:13]
+'''
+    assert asm_check.violations(ok) == []
+    # five instructions in between are as good as an s_nop
+    spaced = '\tv_readlane_b32 s7, v253, 57\n' + '\tv_mov_b32_e32 v2, v3\n' * 5 + \
+        '\t;;#ASMSTART\n\tglobal_load_dwordx4 v[2:5], v1, s[6:7]\n\t;;#ASMEND\n'
+    assert asm_check.violations(spaced) == []
+    assert len(asm_check.violations(spaced.replace('\tv_mov_b32_e32 v2, v3\n' * 5, '\tv_mov_b32_e32 v2, v3\n' * 4))) == 1
