@@ -112,10 +112,12 @@ int mdcn_abi_version(void);
  * pass), the backward keeps at most 1.5 GiB of column gradient (and as much of
  * columns) at a time.  This lowers the two limits for the whole process (0
  * restores a default; values above the defaults are clipped): a knob for memory
- * constrained callers and for tests of the pass loops.  Not thread safe against
- * concurrent calls into the library; workspace sizes must be queried again
- * after a change.  (No counterpart in the reference, whose im2col_step plays
- * this role for DCNv1.) */
+ * constrained callers and for tests of the pass loops.  The two values are
+ * atomic: a call that runs while another thread changes them uses the old or
+ * the new value, never a mixture.  Workspace sizes depend on them and must be
+ * queried again after a change; a caller that changes the limits between
+ * sizing a workspace and using it gets MDCN_ERR_WORKSPACE at worst.  (No
+ * counterpart in the reference, whose im2col_step plays this role for DCNv1.) */
 void mdcn_set_pass_limits(uint64_t forward_bytes, uint64_t backward_bytes);
 
 /* Static text for a status code. */
@@ -124,13 +126,22 @@ const char *mdcn_status_string(int status);
 /* Output height/width for the shape in *p; returns MDCN_OK or MDCN_ERR_SHAPE. */
 int mdcn_output_size(const mdcn_params *p, int32_t *Ho, int32_t *Wo);
 
-/* 1 when the fused MFMA kernel covers the shape/dtype in *p, else 0. */
+/* 1 when the fused MFMA kernel covers the shape/dtype in *p, else 0.  Of the
+ * pointer fields only `input` is looked at, and only with input_nhwc = 1: a
+ * channels-last input is read in place, so it must be 16-byte aligned -- set it
+ * before this query and before mdcn_workspace_bytes(). */
 int mdcn_fused_eligible(const mdcn_params *p);
 
-/* Bytes of device scratch mdcn_forward() needs for *p (pointer fields are not
- * read).  The fused path keeps a zero-bordered channels-last copy of the input
- * and the repacked weights there; the direct path needs none.  Returns 0 for an
- * invalid *p (mdcn_forward then reports the error). */
+/* Bytes of device scratch mdcn_forward() asks for (of the pointer fields only
+ * `input` is looked at, see mdcn_fused_eligible()).  The fused path keeps a
+ * zero-bordered channels-last copy of the input and the repacked weights there;
+ * the direct path and MDCN_F64 need none.  For 16-bit tensors with 256-channel
+ * output tiles the figure ends with an optional region (one 128 x 256 fp32 tile
+ * and a counter per workgroup, 32 MiB on a 256-CU device) through which
+ * workgroups that would otherwise idle in the last round of the schedule share
+ * the K range of a tile: a workspace that is smaller by that region is accepted
+ * too and only runs that last round unshared.  Returns 0 for an invalid *p
+ * (mdcn_forward then reports the error). */
 size_t mdcn_workspace_bytes(const mdcn_params *p);
 
 /* Enqueue the forward on `hip_stream` (a hipStream_t; NULL = the null stream).
@@ -147,7 +158,8 @@ int mdcn_forward(const mdcn_params *p, void *hip_stream);
  * to a buffer of MDCN_NOALLOC_SCRATCH_BYTES that is part of the library's
  * device image (each device the library runs on holds one until the process
  * ends).  Calls whose mdcn_workspace_bytes() exceeds that size return
- * MDCN_ERR_SCRATCH_LIMIT and enqueue nothing.  The call allocates and frees
+ * MDCN_ERR_SCRATCH_LIMIT and enqueue nothing (the optional region at the end
+ * of the workspace is used when it fits as well and left out otherwise).  The call allocates and frees
  * nothing, on the host or on the device.  All calls on one device share the
  * buffer: calls that overlap in time on one device (different streams or
  * threads) race; calls on one stream are ordered by the stream.  Nothing in the

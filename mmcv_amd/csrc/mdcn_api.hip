@@ -6,6 +6,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cstdio>
 #include <mutex>
 #include <type_traits>
@@ -30,9 +31,11 @@ constexpr size_t kMaxLds = 160 * 1024;
 constexpr uint64_t kMaxXtBytes = 0xF0000000ull;
 // Column gradient (and columns) held in memory per pass of the backward's matrix-core paths.
 constexpr uint64_t kBwdColGradCap = (uint64_t)3 << 29;  // 1.5 GiB each
-// Per-pass limits in force (mdcn_set_pass_limits lowers them; process wide).
-uint64_t g_fwd_pass_bytes = kMaxXtBytes;
-uint64_t g_bwd_pass_bytes = kBwdColGradCap;
+// Per-pass limits in force (mdcn_set_pass_limits lowers them; process wide).  Atomic, so that a
+// call that runs while another thread changes them reads one of the two values; a workspace that was
+// sized under one value and used under another is still the caller's to avoid.
+std::atomic<uint64_t> g_fwd_pass_bytes{kMaxXtBytes};
+std::atomic<uint64_t> g_bwd_pass_bytes{kBwdColGradCap};
 
 inline size_t align_up(size_t v) { return (v + kAlign - 1) / kAlign * kAlign; }
 
@@ -176,7 +179,7 @@ int make_plan(const mdcn_params *p, const Geom &g, Plan *pl) {
   pl->n_ctiles = (g.cout_g + pl->CT - 1) / pl->CT;
   pl->slabs = g.cin_g / pl->KC;
   const uint64_t img = (uint64_t)g.Hp * g.Wp * g.Cin * es;
-  pl->n_chunk = (int)std::min<uint64_t>((uint64_t)g.N, std::max<uint64_t>(1, g_fwd_pass_bytes / img));
+  pl->n_chunk = (int)std::min<uint64_t>((uint64_t)g.N, std::max<uint64_t>(1, g_fwd_pass_bytes.load() / img));
   pl->xt_bytes = p->input_nhwc ? 0 : align_up((size_t)img * pl->n_chunk);
   pl->wp_bytes = align_up((size_t)g.G * pl->n_ctiles * pl->slabs * g.taps * pl->CT * pl->KC * es);
   if (uses_fused2(p, g, *pl)) {
@@ -688,7 +691,7 @@ void make_bwd_plan(const mdcn_bwd_params *bp, const Geom &g, BwdPlan *pl) {
     pl->wgemm = bp->grad_weight != nullptr;
   }
   if (pl->gemm || pl->wgemm) {
-    pl->n_chunk = (int)std::min<uint64_t>((uint64_t)g.N, std::max<uint64_t>(1, g_bwd_pass_bytes / d_img));
+    pl->n_chunk = (int)std::min<uint64_t>((uint64_t)g.N, std::max<uint64_t>(1, g_bwd_pass_bytes.load() / d_img));
     pl->xt_bytes = align_up((size_t)g.N * (g.Cin / KC) * g.Hp * g.Wp * 128);
   }
   if (pl->gemm) {
@@ -1065,8 +1068,8 @@ extern "C" {
 int mdcn_abi_version(void) { return MDCN_ABI_VERSION; }
 
 void mdcn_set_pass_limits(uint64_t forward_bytes, uint64_t backward_bytes) {
-  g_fwd_pass_bytes = forward_bytes ? std::min<uint64_t>(forward_bytes, kMaxXtBytes) : kMaxXtBytes;
-  g_bwd_pass_bytes = backward_bytes ? std::min<uint64_t>(backward_bytes, kBwdColGradCap) : kBwdColGradCap;
+  g_fwd_pass_bytes.store(forward_bytes ? std::min<uint64_t>(forward_bytes, kMaxXtBytes) : kMaxXtBytes);
+  g_bwd_pass_bytes.store(backward_bytes ? std::min<uint64_t>(backward_bytes, kBwdColGradCap) : kBwdColGradCap);
 }
 
 const char *mdcn_status_string(int status) {

@@ -184,3 +184,86 @@ def test_full_size_layer_gradients_spot_check():
         err = rel_err(_np(o[:1]), r)
         print(f'  {nm}: {err:.2e}', flush=True)
         assert err <= TOL[dtype], (nm, err)
+
+
+def test_full_size_grad_weight_and_bias_at_cfg4_shape():
+    """grad_weight / grad_bias at the full cfg-4 shape (N = 16, 243 200 pixels: the 256-tile split-K
+    product and its fixed-order reduction).  With zero offsets and unit mask the layer is a plain
+    convolution, whose weight gradient torch computes in fp32; grad_bias is the sum of grad_output."""
+    dtype = torch.bfloat16
+    case = make_case(99, N=16, Cin=256, Cout=256, H=100, W=152, sigma=0.0)
+    case['mask'] = torch.ones_like(case['mask'])
+    dev = cast_case(case, dtype, 'cuda')
+    gy = torch.randn(16, 256, 100, 152, generator=torch.Generator().manual_seed(2)).to(dtype).cuda()
+    got = capi_backward(dev, gy, path=capi.PATH_FUSED)
+    gw_ref = torch.nn.grad.conv2d_weight(dev['input'].float(), dev['weight'].shape, gy.float(), stride=1, padding=1)
+    gb_ref = gy.double().sum(dim=(0, 2, 3))
+    gi_ref = torch.nn.grad.conv2d_input(dev['input'].shape, dev['weight'].float(), gy.float(), stride=1, padding=1)
+    for nm, o, r in (('grad_weight', got[3], gw_ref), ('grad_bias', got[4], gb_ref), ('grad_input', got[0], gi_ref)):
+        err = rel_err(_np(o), r.float().cpu().numpy())
+        print(f'  {nm}: {err:.2e}', flush=True)
+        assert err <= TOL[dtype], (nm, err)
+
+
+def test_full_size_grad_weight_adds_up_over_batch_halves():
+    """Random offsets at the cfg-4 shape: the weight and bias gradients of the whole batch are the sums of
+    those of its two halves (each a call of its own, with its own K-range shares)."""
+    dtype = torch.bfloat16
+    case = cast_case(make_case(4243, N=16, Cin=256, Cout=256, H=100, W=152, sigma=2.0), dtype, 'cuda')
+    gy = torch.randn(16, 256, 100, 152, generator=torch.Generator().manual_seed(5)).to(dtype).cuda()
+    full = capi_backward(case, gy, path=capi.PATH_FUSED, want_data=False)
+
+    def half(sl):
+        sub = dict(case)
+        for k in ('input', 'offset', 'mask'):
+            sub[k] = case[k][sl].contiguous()
+        return capi_backward(sub, gy[sl].contiguous(), path=capi.PATH_FUSED, want_data=False)
+
+    a, b = half(slice(0, 8)), half(slice(8, 16))
+    for i, nm in ((3, 'grad_weight'), (4, 'grad_bias')):
+        err = rel_err(_np(full[i]), _np(a[i]) + _np(b[i]))
+        print(f'  {nm}: {err:.2e}', flush=True)
+        assert err <= 8e-3, (nm, err)  # (three roundings to bf16 instead of one)
+
+
+def test_full_size_all_five_gradients_against_oracle():
+    """cfg-4-shaped layer, N = 2: every gradient of the whole call against the oracle."""
+    dtype = torch.bfloat16
+    case = cast_case(make_case(4244, N=2, Cin=256, Cout=256, H=100, W=152, sigma=2.0), dtype)
+    gy = torch.randn(2, 256, 100, 152, generator=torch.Generator().manual_seed(7)).to(dtype)
+    got = capi_backward(cast_case(case, dtype, 'cuda'), gy.cuda(), path=capi.PATH_FUSED)
+    ref = oracle.backward(*[case[k].float().numpy() for k in ('input', 'offset', 'mask', 'weight')],
+                          gy.float().numpy(), True, stride=(1, 1), padding=(1, 1), dilation=(1, 1), groups=1,
+                          deform_groups=1)
+    for nm, r, o in zip(NAMES, ref, got):
+        err = rel_err(_np(o), r)
+        print(f'  {nm}: {err:.2e}', flush=True)
+        assert err <= TOL[dtype], (nm, err)
+
+
+def test_fixed_point_window_with_wide_dynamic_range():
+    """16-bit tensors sum grad_input in a 32-bit fixed-point window scaled by the largest column
+    gradient of the call.  With grad_output spanning six decades, the gradient as a whole stays
+    within tolerance of the oracle (error against the largest element), and the region whose
+    contributions are a million times smaller than the largest carries an absolute error of at most
+    a few window quanta, i.e. far below the 16-bit rounding of the large elements -- but not a
+    small relative error of its own, which is what the window gives up."""
+    dtype = torch.bfloat16
+    case = cast_case(make_case(606, N=1, Cin=64, Cout=64, H=40, W=48, sigma=1.0), dtype)
+    g = torch.Generator().manual_seed(8)
+    gy = torch.randn(1, 64, 40, 48, generator=g) * 1e-5
+    gy[:, :, 2:6, 2:6] = torch.randn(1, 64, 4, 4, generator=g) * 10.0
+    gy = gy.to(dtype)
+    got = capi_backward(cast_case(case, dtype, 'cuda'), gy.cuda(), path=capi.PATH_FUSED)
+    ref = oracle.backward(*[case[k].float().numpy() for k in ('input', 'offset', 'mask', 'weight')],
+                          gy.float().numpy(), True, stride=(1, 1), padding=(1, 1), dilation=(1, 1), groups=1,
+                          deform_groups=1)
+    gi, gi_ref = _np(got[0]), ref[0]
+    big = float(np.abs(gi_ref).max())
+    assert rel_err(gi, gi_ref) <= TOL[dtype]
+    far = np.abs(gi - gi_ref)[:, :, 20:, 24:]   # sampled only by pixels with tiny grad_output
+    assert float(np.abs(gi_ref[:, :, 20:, 24:]).max()) < 1e-4 * big
+    print(f'  far region: max abs err {far.max():.3e}, largest element of the gradient {big:.3e}', flush=True)
+    assert float(far.max()) <= 2e-5 * big
+    for nm, r, o in zip(NAMES[1:], ref[1:], got[1:]):
+        assert rel_err(_np(o), r) <= TOL[dtype], nm
