@@ -758,12 +758,15 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
           }
         }
       };
+      // the common case: the wave's 64 pixels lie in one image and every run is one 16-byte store
+      const bool plain = vec_ok && pw0 + 64 <= total_px && rem0 + 64 <= plane_out;
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
         const int col = ctile * CT + wave_c * 64 + mb * 32 + frow;
         const bool col_ok = col < g.cout_g;
         const long cbase = (long)grp * g.cout_g + col;
         const float bvm = bv[mb];
+        E *row = out + ((long)n0 * g.Cout + cbase) * plane_out + rem0 + 8 * fhalf;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
           const f32x16 &c = acc[nb][mb];
@@ -779,7 +782,11 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
             const auto s1 = __builtin_amdgcn_permlane32_swap(a1, b1, false, false);
             u32x4 val;
             val.x = s0[0]; val.y = s1[0]; val.z = s0[1]; val.w = s1[1];
-            if (col_ok) store_run(cbase, nb * 32 + 8 * (fhalf ? gb : ga), val);
+            if (plain) {
+              if (col_ok) *(u32x4 *)(row + nb * 32 + 16 * g2) = val;
+            } else if (col_ok) {
+              store_run(cbase, nb * 32 + 8 * (fhalf ? gb : ga), val);
+            }
           }
         }
       }
