@@ -102,6 +102,12 @@ typedef struct mdcn_params {
                              in memory (torch.channels_last); the fused kernel then reads it in place, without
                              the re-laid-out copy.  Fused path of mdcn_forward() only (H, W >= 2); every
                              other tensor keeps its layout. */
+  int32_t no_k_split;     /* 0: workgroups that would idle in the last round of the fused kernel's schedule
+                             take over parts of the K range of that round's tiles (partial sums meet in
+                             the workspace, added in a fixed order: results are the same on every run).
+                             1: every tile is summed by one workgroup, as a single fp32 sum over K; an
+                             image's output then does not depend on where in the batch it sits.  The two
+                             settings differ by fp32 rounding of the sums only. */
 } mdcn_params;
 
 /* ABI version of the loaded library (== MDCN_ABI_VERSION it was built with). */

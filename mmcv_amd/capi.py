@@ -27,7 +27,7 @@ class MdcnParams(ctypes.Structure):
                 [('workspace_bytes', ctypes.c_size_t)] +
                 [(n, ctypes.c_int32) for n in
                  ('dtype', 'path', 'N', 'Cin', 'H', 'W', 'Cout', 'kh', 'kw',
-                  'sh', 'sw', 'ph', 'pw', 'dh', 'dw', 'groups', 'dgroups', 'input_nhwc')])
+                  'sh', 'sw', 'ph', 'pw', 'dh', 'dw', 'groups', 'dgroups', 'input_nhwc', 'no_k_split')])
 
 
 class MdcnPackParams(ctypes.Structure):

@@ -23,6 +23,8 @@ using at::Tensor;
 
 // device path of every op of this module (set_path); read once per call
 std::atomic<int> g_path{MDCN_PATH_AUTO};
+// mdcn_params.no_k_split of every forward of this module (set_k_split)
+std::atomic<int> g_no_k_split{0};
 
 std::string device_str(const at::Device &d) {
   std::string s = c10::DeviceTypeName(d.type(), /*lower_case=*/true);
@@ -89,6 +91,7 @@ void prepare(Prepared &pr, const Tensor &input, const Tensor &weight,
   p = mdcn_params{};
   p.dtype = mdcn_dtype_of(input);
   p.path = g_path.load();
+  p.no_k_split = g_no_k_split.load();
   p.N = (int)batch; p.Cin = (int)channels; p.H = (int)height; p.W = (int)width;
   p.Cout = (int)channels_out; p.kh = kernel_h; p.kw = kernel_w;
   p.sh = stride_h; p.sw = stride_w; p.ph = pad_h; p.pw = pad_w;
@@ -224,6 +227,7 @@ std::vector<double> modulated_deform_conv_pack_forward(
   mdcn_params &p = pp.conv;
   p.dtype = mdcn_dtype_of(input);
   p.path = g_path.load();
+  p.no_k_split = g_no_k_split.load();
   p.N = (int)batch; p.Cin = (int)channels; p.H = (int)input.size(2); p.W = (int)input.size(3);
   p.Cout = (int)channels_out; p.kh = kernel_h; p.kw = kernel_w;
   p.sh = stride_h; p.sw = stride_w; p.ph = pad_h; p.pw = pad_w;
@@ -336,6 +340,7 @@ void deform_conv_forward(Tensor input, Tensor weight, Tensor offset, Tensor outp
   mdcn_params p{};
   p.dtype = mdcn_dtype_of(input);
   p.path = g_path.load();
+  p.no_k_split = g_no_k_split.load();
   p.N = (int)batch; p.Cin = (int)planes; p.H = (int)input.size(2); p.W = (int)input.size(3);
   p.Cout = (int)weight.size(0); p.kh = kH; p.kw = kW;
   p.sh = dH; p.sw = dW; p.ph = padH; p.pw = padW; p.dh = dilationH; p.dw = dilationW;
@@ -408,6 +413,7 @@ void run_backward(const char *op, const Tensor &input, const Tensor &weight, con
   p.sh = stride_h; p.sw = stride_w; p.ph = pad_h; p.pw = pad_w; p.dh = dilation_h; p.dw = dilation_w;
   p.groups = group; p.dgroups = deformable_group;
   p.path = g_path.load();
+  p.no_k_split = g_no_k_split.load();
   int32_t Ho = 0, Wo = 0;
   int rc = mdcn_output_size(&p, &Ho, &Wo);
   TORCH_CHECK(rc == MDCN_OK, op, ": ", mdcn_status_string(rc));
@@ -573,5 +579,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         }, "choose the device path of forward and backward: 0 auto, 1 fused / matrix-core kernels, 2 direct kernels, "
            "3 fused with the specialised-wave forward kernel", py::arg("path"));
   m.def("get_path", []() { return g_path.load(); });
+  m.def("set_k_split", [](bool on) { g_no_k_split.store(on ? 0 : 1); },
+        "true (default): idle workgroups of the fused forward kernel's last round take parts of the K range of its "
+        "tiles; false: every tile is one fp32 sum formed by one workgroup", py::arg("on"));
+  m.def("get_k_split", []() { return g_no_k_split.load() == 0; });
   m.def("abi_version", []() { return mdcn_abi_version(); });
 }

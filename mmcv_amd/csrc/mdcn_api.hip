@@ -182,7 +182,7 @@ int make_plan(const mdcn_params *p, const Geom &g, Plan *pl) {
   pl->n_chunk = (int)std::min<uint64_t>((uint64_t)g.N, std::max<uint64_t>(1, g_fwd_pass_bytes.load() / img));
   pl->xt_bytes = p->input_nhwc ? 0 : align_up((size_t)img * pl->n_chunk);
   pl->wp_bytes = align_up((size_t)g.G * pl->n_ctiles * pl->slabs * g.taps * pl->CT * pl->KC * es);
-  if (uses_fused2(p, g, *pl)) {
+  if (!p->no_k_split) {  // one 128 x 256 fp32 tile and a counter per workgroup of the persistent grid
     pl->split_wgs = num_cus() / 8 * 8;
     pl->split_bytes = align_up((size_t)pl->split_wgs * kPT * kF2CT * 4) + align_up((size_t)pl->split_wgs * 4);
   }
@@ -258,8 +258,10 @@ hipError_t launch_oconv(OconvArgs oa, hipStream_t st) {
 template <typename E, int CT, int TMAX, bool MULTI_DG>
 hipError_t launch_fused_ct(const FusedArgs &fa, bool unbordered, hipStream_t st) {
   // persistent workgroups: one per CU, a multiple of the 8 XCDs
+  // (with tiles cut along K, workgroups beyond the tile count take parts of tiles: the whole chip)
   const int total_wg = fa.n_ptiles * fa.n_ctiles * fa.g.G;
-  const int per_xcd = std::max(1, std::min((total_wg + 7) / 8, num_cus() / 8));
+  const int per_xcd = fa.split_max > 1 ? std::max(1, num_cus() / 8)
+                                       : std::max(1, std::min((total_wg + 7) / 8, num_cus() / 8));
   if (unbordered)
     hipLaunchKernelGGL((fused_kernel<E, CT, TMAX, MULTI_DG, true>), dim3(per_xcd * 8), dim3(kThreads),
                        0, st, fa);
@@ -273,7 +275,8 @@ hipError_t launch_fused_ct(const FusedArgs &fa, bool unbordered, hipStream_t st)
 template <typename E>
 hipError_t launch_fused2(const FusedArgs &fa, bool unbordered, hipStream_t st) {
   const int total_wg = fa.n_ptiles * fa.n_ctiles * fa.g.G;
-  const int per_xcd = std::max(1, std::min((total_wg + 7) / 8, num_cus() / 8));
+  const int per_xcd = fa.split_max > 1 ? std::max(1, num_cus() / 8)
+                                       : std::max(1, std::min((total_wg + 7) / 8, num_cus() / 8));
   if (unbordered)
     hipLaunchKernelGGL((fused2_kernel<E, true>), dim3(per_xcd * 8), dim3(kF2Threads), 0, st, fa);
   else

@@ -289,7 +289,7 @@ static_assert(2 * 32 * (64 * 4 + 16) <= kWeightSlots * 64 * kRowB,
 // LDS of one workgroup: two sample tiles, the ring of weight tiles, the
 // (pixel, tap) table (corner index + four weights per entry).
 constexpr size_t fused_lds_bytes(int CT, int tmax) {
-  return (size_t)2 * kPT * kRowB + (size_t)kWeightSlots * CT * kRowB + (size_t)kPT * tmax * 20;
+  return (size_t)2 * kPT * kRowB + (size_t)kWeightSlots * CT * kRowB + (size_t)kPT * tmax * 20 + 16;
 }
 
 // Table capacities the kernel is instantiated for (taps = kh * kw).
@@ -319,17 +319,72 @@ __device__ __forceinline__ void copy16_global_to_lds(const void *src, uint32_t l
                : "memory");
 }
 
+// A pointer every lane of the wave holds the same value of, moved to scalar
+// registers (for an "s" operand of an asm statement: the compiler does not always
+// see that a value is uniform, and then hands such an operand vector registers).
+__device__ __forceinline__ const unsigned char *uniform_ptr(const unsigned char *p) {
+  const uint64_t v = (uint64_t)(uintptr_t)p;
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+  return (const unsigned char *)(uintptr_t)(((uint64_t)hi << 32) | lo);
+}
+
+// Work of one workgroup under the XCD-aware persistent schedule: XCD x owns a
+// contiguous run of tiles and hands them out round robin to its `stride`
+// workgroups.  The run rarely is a multiple of `stride`: its last round has
+// rest < stride tiles, and without further ado `rest` workgroups would compute a
+// whole tile while the others wait.  Instead each of those tiles is cut along K
+// into parts = stride / rest ranges (whole multiples of `round` steps, at most
+// split_max of them, each at least `min_rounds` rounds long), one per workgroup:
+// a "unit" is a tile together with a range of K steps; a workgroup walks whole
+// tiles first (units 0 .. T_full - 1) and at most one part last.  The parts of
+// a tile meet in memory.
+struct UnitSchedule {
+  int xcd, wg, stride, chunk;
+  int T_full, T;
+  bool has_part;
+  int parts, part_tile, part_idx, part_kb, part_pad;
+
+  __device__ __forceinline__ void init(int total_tiles, int nk_pad, int round, int min_rounds, int split_max) {
+    xcd = (int)(blockIdx.x & 7);
+    wg = (int)(blockIdx.x >> 3);
+    stride = (int)(gridDim.x >> 3);
+    chunk = (total_tiles + 7) >> 3;
+    const int tile_end = min((xcd + 1) * chunk, total_tiles);
+    const int chunk_x = max(tile_end - xcd * chunk, 0);
+    const int full_rounds = chunk_x / stride;
+    const int rest = chunk_x - full_rounds * stride;
+    const int rounds = nk_pad / round;
+    parts = 1;
+    if (split_max > 1 && rest > 0) parts = max(1, min(min(stride / rest, split_max), rounds / min_rounds));
+    const bool split = parts > 1;
+    T_full = full_rounds + ((!split && wg < rest) ? 1 : 0);
+    has_part = split && wg < rest * parts;
+    T = T_full + (has_part ? 1 : 0);
+    part_tile = xcd * chunk + full_rounds * stride + wg / parts;
+    part_idx = wg - (wg / parts) * parts;
+    part_kb = (part_idx * rounds / parts) * round;
+    part_pad = ((part_idx + 1) * rounds / parts) * round - part_kb;
+  }
+  __device__ __forceinline__ bool is_part(int u) const { return has_part && u == T_full; }
+  __device__ __forceinline__ int tile_of(int u) const { return is_part(u) ? part_tile : xcd * chunk + wg + u * stride; }
+  // the counter of this workgroup's cut tile and the first of the tile's buffers (one per workgroup of the grid)
+  __device__ __forceinline__ int counter_slot() const { return xcd * stride + wg / parts; }
+  __device__ __forceinline__ int buffer_slot0() const { return xcd * stride + (wg / parts) * parts; }
+};
+
 // Walks the K steps of a tile in issue order (channel slab outer, tap inner) and
 // reports when a step starts a new deformable group.  Producers and consumers
 // run identical cursors, so both know when the table is rebuilt.
 struct StepCursor {
   int step, slab, tap, dgrem;
   bool new_dg;
-  __device__ __forceinline__ void init(int slab0, int spd) {
+  // `step` counts from the unit's first step kb (0 for a whole tile)
+  __device__ __forceinline__ void init(int slab0, int spd, int kb, int taps) {
     step = 0;
-    slab = 0;
-    tap = 0;
-    dgrem = slab0 % spd;
+    slab = kb / taps;
+    tap = kb - slab * taps;
+    dgrem = (slab0 + slab) % spd;
     new_dg = false;
   }
   // Move to the next step; past the last step the cursor stays on it.
@@ -384,11 +439,12 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
   __shared__ uint4 Ws[kWeightSlots][CT * kRowChunks];     // weight tiles
   __shared__ uint32_t tpix[PT * TMAX];                    // (pixel, tap) table, [tap][PT]: corner byte offset
   __shared__ uint4 tws[PT * TMAX];                        // ... and the four weights
+  __shared__ uint32_t part_arrived;                       // parts of a cut tile that were there before this one
 
   const Geom &g = a.g;
   const int taps = g.taps;
-  const int nk = a.slabs * taps;
-  const int nk_pad = (nk + kGatherAhead - 1) / kGatherAhead * kGatherAhead;
+  const int nk_tile = a.slabs * taps;
+  const int nk_tile_pad = (nk_tile + kGatherAhead - 1) / kGatherAhead * kGatherAhead;
   const int plane_out = g.Ho * g.Wo;
   const int total_px = (int)a.total_px;
   const int spd = g.ch_per_dg / KC;  // slabs per deformable group
@@ -400,17 +456,20 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
 
   // XCD-aware persistent schedule: consecutive workgroup ids sit on different
   // XCDs; each XCD walks one contiguous run of tiles so that the halo rows
-  // neighbouring tiles share stay in its L2.
-  const int total_tiles = a.n_ptiles * a.n_ctiles * g.G;
-  const int xcd = (int)(blockIdx.x & 7);
-  const int wg_in_xcd = (int)(blockIdx.x >> 3);
-  const int wgs_per_xcd = (int)(gridDim.x >> 3);
-  const int chunk = (total_tiles + 7) >> 3;
-  const int tile_end = min((xcd + 1) * chunk, total_tiles);
+  // neighbouring tiles share stay in its L2.  Tiles of the run's last round are
+  // cut along K (UnitSchedule): parts of at least 8 steps.
+  UnitSchedule us;
+  us.init(a.n_ptiles * a.n_ctiles * g.G, nk_tile_pad, kGatherAhead, 8 / kGatherAhead, a.split_max);
   bool first_tile = true;
 
-  for (int tile = xcd * chunk + wg_in_xcd; tile < tile_end; tile += wgs_per_xcd, first_tile = false) {
-    int L = tile;
+  for (int u = 0; u < us.T; ++u, first_tile = false) {
+    const bool is_part = us.is_part(u);
+    // K range of the unit: steps kb .. kb + nk - 1 of the tile, padded to nk_pad
+    const int kb = is_part ? us.part_kb : 0;
+    const int nk_pad = is_part ? us.part_pad : nk_tile_pad;
+    const int nk = min(nk_tile - kb, nk_pad);
+    const bool more_units = u + 1 < us.T;
+    int L = us.tile_of(u);
     const int ctile = L % a.n_ctiles;
     L /= a.n_ctiles;
     const int grp = L % g.G;
@@ -420,7 +479,7 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
     const int slab0 = ch0 / KC;
 
     StepCursor cur;  // the next step whose gather is issued
-    cur.init(slab0, spd);
+    cur.init(slab0, spd, kb, taps);
 
     if (producer) {
       // =================== PRODUCER ===================
@@ -552,7 +611,7 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
         cur.advance(nk, taps, spd);
       };
 
-      build_table(ch0 / g.ch_per_dg);
+      build_table((ch0 + cur.slab * KC) / g.ch_per_dg);
       MDCN_BARRIER_LDS();  // B0: table visible
 
 #pragma unroll
@@ -580,6 +639,10 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
       // registers with vmcnt waits that also wait for their in-flight weight copies.
       __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), other counters untouched
       MDCN_BARRIER_LDS();   // E0: the K loop is over for everybody
+      if (is_part) {        // the consumers' two barriers around the arrival count of a cut tile
+        MDCN_BARRIER_LDS();
+        MDCN_BARRIER_LDS();
+      }
       if (!OVL) MDCN_BARRIER_LDS();   // E1: epilogue done, tiles and table may be rewritten
     } else {
       // =================== CONSUMER ===================
@@ -619,7 +682,7 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
       // the K loop, WDMA per step, so "at most kWeightAhead*WDMA outstanding"
       // means the next step's tile has landed.
       const unsigned char *wp_tile = (const unsigned char *)a.wp +
-                                     ((size_t)(grp * a.n_ctiles + ctile) * nk) * (size_t)(CT * kRowB);
+                                     ((size_t)(grp * a.n_ctiles + ctile) * nk_tile + kb) * (size_t)(CT * kRowB);
       uint32_t wlane[WDMA];  // byte offset of this lane's source chunk inside a tile
 #pragma unroll
       for (int c = 0; c < WDMA; ++c) {
@@ -676,7 +739,80 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
       MDCN_BARRIER(0);  // E0: copies issued past the end have landed; tiles become staging
       // B0 of the next tile, taken early: the producers need nothing from the
       // consumers for its table, gathers and first sample tile
-      if (OVL && tile + wgs_per_xcd < tile_end) MDCN_BARRIER_LDS();
+      if (OVL && more_units) MDCN_BARRIER_LDS();
+
+      // ---- a part of a tile: the parts meet in memory.  Every part stores its
+      // accumulators (fp32, register order) and counts itself in; the part that
+      // arrives last adds them up -- two parts: its own registers plus the other's
+      // values, the same in either order; more: all from memory in index order, so
+      // the sum does not depend on who was last -- and goes on to the epilogue; the
+      // others are done.  Nobody waits for anybody; the last part leaves the counter
+      // at zero for the next launch.  Stores and loads are device coherent (sc1):
+      // they go past the caches private to a CU or an XCD.  A part is a workgroup's
+      // last unit, and the producers take part in the two barriers.
+      bool store_tile = true;
+      if (is_part) {
+        constexpr int NQ = NB * MB * 4;           // 16-byte quads of accumulators per lane
+        constexpr int CQ = 8;                     // quads read back at a time (NQ is a multiple of 8)
+        const int tslot = us.counter_slot();
+        const unsigned char *pbase =
+            (const unsigned char *)a.split_part + (size_t)us.buffer_slot0() * (size_t)(PT * 256 * 4);
+        const unsigned char *mine = uniform_ptr(pbase + (size_t)us.part_idx * (size_t)(PT * 256 * 4));
+        // quad j of the 256 consumer lanes is one 4 KiB run.  (The offset is opaque to the optimiser,
+        // which would otherwise form the addresses below ahead of the unit loop and keep them live.)
+        uint32_t voff = (uint32_t)tid * 16u;
+        asm volatile("" : "+v"(voff));
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int qd = 0; qd < 4; ++qd) {
+              const f32x16 &c = acc[nb][mb];
+              const f32x4 v = {c[4 * qd], c[4 * qd + 1], c[4 * qd + 2], c[4 * qd + 3]};
+              const uint32_t vo = voff + (uint32_t)(((nb * MB + mb) * 4 + qd) * 4096);
+              // (s_nop: a vector-memory instruction must not read a scalar register within five issue
+              // slots of a vector instruction writing it -- a reload of spilled scalars, say -- and the
+              // compiler does not look into assembly text to keep that distance)
+              asm volatile("s_nop 4\n\tglobal_store_dwordx4 %0, %1, %2 sc1" : : "v"(vo), "v"(v), "s"(mine) : "memory");
+            }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        MDCN_BARRIER_LDS();
+        if (tid == 0)
+          part_arrived = __hip_atomic_fetch_add((uint32_t *)a.split_cnt + tslot, 1u, __ATOMIC_RELAXED,
+                                                __HIP_MEMORY_SCOPE_AGENT);
+        MDCN_BARRIER_LDS();
+        store_tile = part_arrived == (uint32_t)(us.parts - 1);
+        if (store_tile) {
+          const bool two = us.parts == 2;
+          const unsigned char *src0 = two ? pbase + (size_t)(1 - us.part_idx) * (size_t)(PT * 256 * 4) : pbase;
+          for (int i = two ? 1 : 0; i < us.parts; ++i) {
+            const unsigned char *src = uniform_ptr(src0);
+#pragma unroll
+            for (int q0 = 0; q0 < NQ; q0 += CQ) {
+              f32x4 tmp[CQ];
+#pragma unroll
+              for (int j = 0; j < CQ; ++j) {
+                const uint32_t vo = voff + (uint32_t)((q0 + j) * 4096);
+                asm volatile("s_nop 4\n\tglobal_load_dwordx4 %0, %1, %2 sc1" : "=v"(tmp[j]) : "v"(vo), "s"(src));
+              }
+#pragma unroll
+              for (int j = 0; j < CQ; ++j) asm volatile("s_waitcnt vmcnt(0)" : "+v"(tmp[j]));
+#pragma unroll
+              for (int j = 0; j < CQ; ++j) {
+                const int qi = q0 + j, blk = qi >> 2, qd = qi & 3;
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                  acc[blk / MB][blk % MB][4 * qd + e] =
+                      i == 0 ? tmp[j][e] : acc[blk / MB][blk % MB][4 * qd + e] + tmp[j][e];
+              }
+            }
+            src0 += PT * 256 * 4;
+          }
+          if (tid == 0)
+            __hip_atomic_store((uint32_t *)a.split_cnt + tslot, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      }
 
       // ---- epilogue: bias, round once, transpose through LDS, NCHW store ----
       // Accumulator block (A = samples, B = weights): register r of lane l holds
@@ -692,6 +828,7 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
       const bool vec_ok = a.out_vec_ok != 0;      // 16-byte chunks never straddle images, aligned
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
+        if (!store_tile) break;  // a part that was not the last to arrive has nothing to store
         const int col0 = ctile * CT + wave_c * (CT / 2) + mb * 32;  // channel within the group
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {

@@ -48,7 +48,6 @@ namespace mdcn {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 
@@ -651,7 +650,7 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
       const int tslot = xcd * stride + wg / parts;                       // the tile's counter
       const unsigned char *pbase =
           (const unsigned char *)a.split_part + (size_t)(xcd * stride + (wg / parts) * parts) * (size_t)(PT * CT * 4);
-      const unsigned char *mine = pbase + (size_t)part_idx * (size_t)(PT * CT * 4);
+      const unsigned char *mine = uniform_ptr(pbase + (size_t)part_idx * (size_t)(PT * CT * 4));
       // a lane's 64 values travel as 16 quads of 16 bytes; quad j of the wave's lanes is one 1 KiB run.
       // (The offset is opaque to the optimiser, which would otherwise form the addresses below once,
       // ahead of the tile loop, and keep them -- spilled -- across the K loop.)
@@ -685,8 +684,9 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
         // (two parts: a + b is the same in either order, so the last one adds the other's values to
         // the ones it still holds; more parts: everything from memory, in index order)
         const bool two = parts == 2;
-        const unsigned char *src = two ? pbase + (size_t)(1 - part_idx) * (size_t)(PT * CT * 4) : pbase;
+        const unsigned char *src0 = two ? pbase + (size_t)(1 - part_idx) * (size_t)(PT * CT * 4) : pbase;
         for (int i = two ? 1 : 0; i < parts; ++i) {
+          const unsigned char *src = uniform_ptr(src0);
 #pragma unroll
           for (int j = 0; j < 16; ++j) {
             const uint32_t vo = voff + (uint32_t)(j * 1024);
@@ -710,7 +710,7 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
                 for (int e = 0; e < 4; ++e)
                   acc[nb][mb][4 * qd + e] = i == 0 ? v[e] : acc[nb][mb][4 * qd + e] + v[e];
               }
-          src += PT * CT * 4;
+          src0 += PT * CT * 4;
         }
         if (tid == 0)
           __hip_atomic_store((uint32_t *)a.split_cnt + tslot, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -72,9 +72,8 @@ def cast_case(case, dtype, device=None):
 
 def capi_forward(case, path=capi.PATH_AUTO, timed=False, unsplit=False):
     """Run the C ABI on device tensors of `case`; returns the output tensor
-    (and the per-stage milliseconds when `timed`).  `unsplit`: hand over a
-    workspace without the optional buffers for tiles cut along K, so that every
-    tile is summed by one workgroup."""
+    (and the per-stage milliseconds when `timed`).  `unsplit`: no tile is cut
+    along K (mdcn_params.no_k_split), every tile is summed by one workgroup."""
     lib = capi.load()
     x, off, msk, w, b = (case[k] for k in ('input', 'offset', 'mask', 'weight', 'bias'))
     assert x.is_cuda
@@ -86,12 +85,8 @@ def capi_forward(case, path=capi.PATH_AUTO, timed=False, unsplit=False):
     rc, Ho, Wo = capi.output_size(p)
     assert rc == 0, capi.status_string(rc)
     out = torch.empty(N, Cout, Ho, Wo, dtype=x.dtype, device=x.device)
+    p.no_k_split = 1 if unsplit else 0
     ws_bytes = lib.mdcn_workspace_bytes(ctypes.byref(p))
-    if unsplit and ws_bytes:
-        # the specialised-wave kernel never cuts tiles: its workspace is the input copy and the weights
-        p.path = capi.PATH_FUSED_SPLIT
-        ws_bytes = lib.mdcn_workspace_bytes(ctypes.byref(p))
-        p.path = path
     ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=x.device)
     keep = [t.contiguous() for t in (x, off, w)]
     p.input, p.offset, p.weight = (t.data_ptr() for t in keep)
