@@ -133,6 +133,19 @@ int num_cus() {
   return cached[dev];
 }
 
+// Length of the persistent schedule of `tiles` tiles of nk K steps in tile times, as UnitSchedule lays it
+// out: whole rounds, then the last round's tiles whole or cut into parts.
+double schedule_rounds(long tiles, int nk, bool may_cut) {
+  const int stride = std::max(1, num_cus() / 8);
+  const long chunk = (tiles + 7) / 8;  // the fullest XCD
+  const long full = chunk / stride, rest = chunk % stride;
+  if (rest == 0) return (double)full;
+  const int rounds = (nk + kGatherAhead - 1) / kGatherAhead;
+  long parts = 1;
+  if (may_cut) parts = std::max<long>(1, std::min<long>(std::min<long>(stride / rest, kF2SplitMax), rounds / (8 / kGatherAhead)));
+  return (double)full + 1.0 / (double)parts;
+}
+
 struct Plan {
   bool fused;
   int CT, KC, n_ctiles, slabs;
@@ -176,10 +189,22 @@ int make_plan(const mdcn_params *p, const Geom &g, Plan *pl) {
   const size_t es = elem_size(p->dtype);
   pl->KC = slab_channels(p->dtype);
   pl->CT = pick_ct(g.cout_g, g.taps);
-  pl->n_ctiles = (g.cout_g + pl->CT - 1) / pl->CT;
   pl->slabs = g.cin_g / pl->KC;
   const uint64_t img = (uint64_t)g.Hp * g.Wp * g.Cin * es;
   pl->n_chunk = (int)std::min<uint64_t>((uint64_t)g.N, std::max<uint64_t>(1, g_fwd_pass_bytes.load() / img));
+  if (p->dtype == MDCN_F32 && pl->CT == 256) {
+    // fp32 tiles are bound by the matrix pipe (a K step of a 128 x 256 tile is some 7 000 clocks of
+    // 32x32x2 MFMAs against 3 000 of sampling), so a tile's time goes with its width and what counts is
+    // how evenly the tiles fill the workgroups: take the 128-wide tile when its schedule is shorter
+    const long px_tiles = ((long)pl->n_chunk * g.Ho * g.Wo + kPT - 1) / kPT;
+    const int nk = pl->slabs * g.taps;
+    auto cost = [&](int ct) {
+      const long tiles = px_tiles * ((g.cout_g + ct - 1) / ct) * g.G;
+      return schedule_rounds(tiles, nk, !p->no_k_split) * std::max(7000.0 * ct / 256, 3000.0);
+    };
+    if (cost(128) < 0.95 * cost(256)) pl->CT = 128;
+  }
+  pl->n_ctiles = (g.cout_g + pl->CT - 1) / pl->CT;
   pl->xt_bytes = p->input_nhwc ? 0 : align_up((size_t)img * pl->n_chunk);
   pl->wp_bytes = align_up((size_t)g.G * pl->n_ctiles * pl->slabs * g.taps * pl->CT * pl->KC * es);
   if (!p->no_k_split) {  // one 128 x 256 fp32 tile and a counter per workgroup of the persistent grid
