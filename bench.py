@@ -20,6 +20,9 @@ per-stage breakdown go to stderr.
   configs     the other benchmark configurations (cfg 1-3, cfg 4 in fp16, the 13
               layers of cfg 5) with fewer steps: ms, TFLOP/s, fraction of the
               dtype's matrix peak
+  sustained_load  the headline loop repeated at the end of the run (the headline
+              itself starts on an idle card, whose clocks sag under the first
+              few dozen calls)
 """
 import argparse
 import json
@@ -35,7 +38,8 @@ PEAK_TFLOPS = {'bf16': 2500.0, 'f16': 2500.0, 'f32': 157.3}
 HBM_PEAK_GBS = 8000.0
 # (workload, dominant kernel) -> (HBM bytes per launch from rocprofv3 counters, the profile they are in)
 TRAFFIC = {
-    ('cfg4', 'fused2_kernel<bf16>'): (None, None),
+    ('cfg4', 'fused2_kernel<bf16>'): (420.1e6, 'profiles/fused2_kernel_bf16_cfg4.md (FETCH_SIZE 129 690.8 KiB x 2.00 '
+                                               '+ WRITE_SIZE 150 861.1 KiB x 1.00)'),
 }
 
 WORKLOADS = {
@@ -471,6 +475,23 @@ def main():
                           'summed_ms_pack_fused': round(tot_pack, 4), 'steps': a5.steps, 'warmup': a5.warmup,
                           'per_layer_ms': {r['layer']: r['dcn_ms'] for r in rows}}
         rec['configs'] = others
+    # The same K steps once more, now that the card has been under load for a while.  The headline
+    # above is taken from a cold start, where the clocks first sag and then recover over some tens
+    # of calls; this is the rate a pipeline that keeps the GPU busy sees.
+    for _ in range(max(a.warmup, 60)):
+        step()
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(a.steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    warm_ms = e0.elapsed_time(e1) / a.steps
+    log(f'under sustained load: step {warm_ms:.4f} ms')
+    rec['sustained_load'] = {'ms_per_step': round(warm_ms, 4), 'steps': a.steps,
+                             'TFLOPs': round(flops / (warm_ms * 1e-3) / 1e12, 2),
+                             'pct_mfma_peak': round(100.0 * flops / (warm_ms * 1e-3) / 1e12 / peak, 2),
+                             'what': 'the timed loop repeated at the end of the run, after 60 more untimed calls'}
     if not a.no_cpu:
         log('timing the CPU baseline ...')
         # the CPU path gets the values the device saw (rounded to the tensor dtype, up-cast), so its
