@@ -69,7 +69,7 @@ static_assert(kF2Unroll % kF2Sets == 0 && kF2Unroll % 2 == 0 && kF2Unroll % kF2S
 
 constexpr int kF2Taps = kTapsSmall;    // table capacity (kh * kw)
 constexpr int kF2SplitMax = 4;         // parts a tile of the schedule's last round is cut into at most
-constexpr int kF2MinSteps = 18;        // padded steps per tile the streaming needs (the next table is built in round 2)
+constexpr int kF2MinSteps = 18;        // padded steps per tile the streaming needs (the next table is built in the second pass of the K loop)
 constexpr size_t fused2_lds_bytes() {
   return (size_t)2 * kPT * kRowB + (size_t)kF2Slots * kF2CT * kRowB + (size_t)2 * kPT * kF2Taps * 12 + 16;
 }
