@@ -140,3 +140,38 @@ def test_outside_taps_never_touch_the_image(path, dtype):
     y = capi_forward(cast_case(case, dtype, 'cuda'), path=path).float().cpu().numpy()
     assert np.isfinite(y).all()
     assert rel_err(y, ref) <= TOL[dtype]
+
+
+# Tiles of the schedule's last round cut along K (both fused kernels): shapes whose tile counts give
+# two, three and four parts per tile on a 256-CU grid, and one with whole rounds in front of the cut one.
+CUT = {
+    'eight_wave_4_parts': (dict(N=1, Cin=256, Cout=256, H=12, W=20), [torch.bfloat16, torch.float16]),       # 2 tiles
+    'eight_wave_3_parts': (dict(N=5, Cin=256, Cout=256, H=32, W=64), [torch.bfloat16]),                       # 80 tiles: 10 per XCD
+    'eight_wave_2_parts': (dict(N=8, Cin=256, Cout=256, H=32, W=56), [torch.bfloat16]),                       # 112 tiles: 14 per XCD
+    'eight_wave_rounds_then_cut': (dict(N=16, Cin=256, Cout=256, H=48, W=50), [torch.bfloat16]),              # 300 tiles: 32 + 6 per XCD
+    'eight_wave_two_ctiles': (dict(N=2, Cin=128, Cout=512, H=16, W=24), [torch.float16]),                      # 6 x 2 tiles
+    'specialised_fp32_4_parts': (dict(N=1, Cin=256, Cout=256, H=16, W=16), [torch.float32]),                   # 72 steps
+    'specialised_fp32_dg4_s2': (dict(N=2, Cin=512, Cout=512, H=20, W=20, stride=2, deform_groups=4), [torch.float32]),
+    'specialised_c128': (dict(N=4, Cin=128, Cout=128, H=24, W=40), [torch.bfloat16, torch.float32]),
+    'specialised_c64_25_taps': (dict(N=2, Cin=128, Cout=64, H=16, W=16, k=5, padding=2), [torch.float16]),
+}
+
+
+@pytest.mark.parametrize('name', sorted(CUT))
+def test_tiles_cut_along_k(name):
+    """Cut and uncut runs both meet the oracle, agree with one another to fp32 rounding of the sums, and the
+    cut run gives the same bits every time (the parts are added in a fixed order)."""
+    kw, dtypes = CUT[name]
+    for dtype in dtypes:
+        case = make_case(31, **kw)
+        dev = cast_case(case, dtype, 'cuda')
+        ref = oracle_forward(cast_case(case, dtype))
+        y_cut = capi_forward(dev, path=capi.PATH_FUSED)
+        y_one = capi_forward(dev, path=capi.PATH_FUSED, unsplit=True)
+        assert rel_err(y_cut.float().cpu().numpy(), ref) <= TOL[dtype]
+        assert rel_err(y_one.float().cpu().numpy(), ref) <= TOL[dtype]
+        diff = float((y_cut.float() - y_one.float()).abs().max() / y_one.float().abs().max())
+        print(f'  {name} {dtype}: cut vs uncut {diff:.2e}', flush=True)
+        assert diff <= (1e-5 if dtype == torch.float32 else 8e-3)
+        for _ in range(3):
+            assert torch.equal(capi_forward(dev, path=capi.PATH_FUSED), y_cut)
