@@ -169,7 +169,9 @@ struct PackExtra {
 
 // 16-bit tensors, 256-channel tiles, one deformable group, enough K steps: the eight-wave kernel
 bool uses_fused2(const mdcn_params *p, const Geom &g, const Plan &pl) {
-  if (pl.CT != 256 || elem_size(p->dtype) != 2 || g.DG != 1 || p->path == MDCN_PATH_FUSED_SPLIT) return false;
+  if ((pl.CT != 256 && pl.CT != 128) || g.taps > kTapsSmall || elem_size(p->dtype) != 2 || g.DG != 1 ||
+      p->path == MDCN_PATH_FUSED_SPLIT)
+    return false;
   const int nk_pad = (pl.slabs * g.taps + kF2Unroll - 1) / kF2Unroll * kF2Unroll;
   return nk_pad >= kF2MinSteps;
 }
@@ -296,27 +298,27 @@ hipError_t launch_fused_ct(const FusedArgs &fa, bool unbordered, hipStream_t st)
   return hipGetLastError();
 }
 
-// 256-channel tiles: the eight-wave kernel of mdcn_fused2.h
-template <typename E>
+// 16-bit tensors, 256- and 128-channel tiles: the eight-wave kernel of mdcn_fused2.h
+template <typename E, int CT>
 hipError_t launch_fused2(const FusedArgs &fa, bool unbordered, hipStream_t st) {
   const int total_wg = fa.n_ptiles * fa.n_ctiles * fa.g.G;
   const int per_xcd = fa.split_max > 1 ? std::max(1, num_cus() / 8)
                                        : std::max(1, std::min((total_wg + 7) / 8, num_cus() / 8));
   if (unbordered)
-    hipLaunchKernelGGL((fused2_kernel<E, true>), dim3(per_xcd * 8), dim3(kF2Threads), 0, st, fa);
+    hipLaunchKernelGGL((fused2_kernel<E, CT, true>), dim3(per_xcd * 8), dim3(kF2Threads), 0, st, fa);
   else
-    hipLaunchKernelGGL((fused2_kernel<E, false>), dim3(per_xcd * 8), dim3(kF2Threads), 0, st, fa);
+    hipLaunchKernelGGL((fused2_kernel<E, CT, false>), dim3(per_xcd * 8), dim3(kF2Threads), 0, st, fa);
   return hipGetLastError();
 }
 
 template <typename E, int CT>
 hipError_t launch_fused_tm(const FusedArgs &fa, bool ub, bool split, hipStream_t st) {
   const bool small = fa.g.taps <= kTapsSmall;
+  if constexpr (sizeof(E) == 2 && (CT == 256 || CT == 128)) {
+    const int nk_pad = (fa.slabs * fa.g.taps + kF2Unroll - 1) / kF2Unroll * kF2Unroll;
+    if (!split && small && fa.g.DG == 1 && nk_pad >= kF2MinSteps) return launch_fused2<E, CT>(fa, ub, st);
+  }
   if constexpr (CT == 256) {  // (pick_ct never pairs the 256-wide tile with the large table)
-    if constexpr (sizeof(E) == 2) {
-      const int nk_pad = (fa.slabs * fa.g.taps + kF2Unroll - 1) / kF2Unroll * kF2Unroll;
-      if (!split && fa.g.DG == 1 && nk_pad >= kF2MinSteps) return launch_fused2<E>(fa, ub, st);
-    }
     return fa.g.DG > 1 ? launch_fused_ct<E, CT, kTapsSmall, true>(fa, ub, st)
                        : launch_fused_ct<E, CT, kTapsSmall, false>(fa, ub, st);
   } else {

@@ -52,26 +52,18 @@ typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kF2Threads = 512;
-constexpr int kF2CT = 256;             // output channels per tile
+constexpr int kF2CT = 256;             // output channels per tile at most (the template parameter CT: 256 or 128)
 constexpr int kF2Slots = 3;            // ring of weight tiles
 constexpr int kF2GL = 8;               // gather loads per wave and K step
-constexpr int kF2WD = kF2CT / 64;      // 1 KiB weight copies per wave and K step
 constexpr int kF2Sets = 3;             // gather register sets: a gather is in flight for kF2Sets steps
 constexpr int kF2Unroll = 6;           // steps per round of the K loop: sets, sample tiles and ring slots are static
-// vector-memory operations younger than the last load of a gather group (half a
-// set) when that group is blended: the rest of its set, the copies and loads of
-// the steps issued since, the copies of the current step, the refills issued so far
-constexpr int kF2VmBlend = (kF2GL - 4) + (kF2Sets - 1) * (kF2WD + kF2GL) + kF2WD;
-// ... younger than the weight copies that must have landed at a step's barrier
-constexpr int kF2VmBar = 2 * kF2GL + kF2WD;
-static_assert(kF2VmBlend < 64 && kF2VmBar < 64, "vmcnt holds 6 bits");
 static_assert(kF2Unroll % kF2Sets == 0 && kF2Unroll % 2 == 0 && kF2Unroll % kF2Slots == 0, "static indices");
 
 constexpr int kF2Taps = kTapsSmall;    // table capacity (kh * kw)
 constexpr int kF2SplitMax = 4;         // parts a tile of the schedule's last round is cut into at most
 constexpr int kF2MinSteps = 18;        // padded steps per tile the streaming needs (the next table is built in the second pass of the K loop)
-constexpr size_t fused2_lds_bytes() {
-  return (size_t)2 * kPT * kRowB + (size_t)kF2Slots * kF2CT * kRowB + (size_t)2 * kPT * kF2Taps * 12 + 16;
+constexpr size_t fused2_lds_bytes(int CT) {
+  return (size_t)2 * kPT * kRowB + (size_t)kF2Slots * CT * kRowB + (size_t)2 * kPT * kF2Taps * 12 + 16;
 }
 
 // 16 bytes per lane from `base` (two SGPRs) + 32-bit byte offset + immediate
@@ -100,8 +92,9 @@ constexpr size_t fused2_lds_bytes() {
   asm volatile("s_waitcnt vmcnt(%4)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) : "n"(N))
 #define MDCN_LGKMWAIT4(N, a, b, c, d) \
   asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) : "n"(N))
+#define MDCN_LGKMWAIT3(N, a, b, c) \
+  asm volatile("s_waitcnt lgkmcnt(%3)" : "+v"(a), "+v"(b), "+v"(c) : "n"(N))
 typedef __attribute__((address_space(3))) u32x4 *lds_u32x4_ptr;
-static_assert(kF2WD == 4, "issue_weights spells out four copies");
 
 // Blend of one 16-byte chunk (8 channels) from the same chunk at the four
 // corners.  The table keeps the four mask-scaled bilinear weights as two words of
@@ -208,18 +201,27 @@ struct Blend2<f16_t> {
   }
 };
 
-template <typename E, bool UNBORDERED>
+template <typename E, int CT, bool UNBORDERED>
 __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
   using TR = ElemTraits<E>;
   using BL = Blend2<E>;
   static_assert(sizeof(E) == 2, "16-bit element types");
+  static_assert(CT == 256 || CT == 128, "a wave owns 64 pixels x CT / 4 channels");
   constexpr int PT = kPT;
-  constexpr int CT = kF2CT;
   constexpr int KC = TR::KC;
   constexpr int TMAX = kF2Taps;
   constexpr int TBL = PT * TMAX;               // entries of one table
   constexpr int TPT = (TMAX + 3) / 4;          // table entries per lane and build
-  constexpr int NB = 2, MB = 2;                // 32 x 32 accumulator blocks per wave: pixels x channels
+  constexpr int NB = 2, MB = CT / 128;         // 32 x 32 accumulator blocks per wave: pixels x channels
+  constexpr int WCH = CT / 4;                  // output channels per wave
+  constexpr int kF2WD = CT / 64;               // 1 KiB weight copies per wave and K step
+  // vector-memory operations younger than the last load of a gather group (half a
+  // set) when that group is blended: the rest of its set, the copies and loads of
+  // the steps issued since, the copies of the current step, the refills issued so far
+  constexpr int kF2VmBlend = (kF2GL - 4) + (kF2Sets - 1) * (kF2WD + kF2GL) + kF2WD;
+  // ... younger than the weight copies that must have landed at a step's barrier
+  constexpr int kF2VmBar = 2 * kF2GL + kF2WD;
+  static_assert(kF2VmBlend < 64 && kF2VmBar < 64, "vmcnt holds 6 bits");
   constexpr uint32_t kXTile = PT * kRowB, kWTile = CT * kRowB;
 
   __shared__ uint4 Xs[2][PT * kRowChunks];               // sample tiles
@@ -256,7 +258,7 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
   const int wave_p = wave & 1, wave_c = wave >> 1;
   const int frow = lane & 31, fhalf = lane >> 5;
   const uint32_t xa0 = (uint32_t)tile_chunk(wave_p * 64 + frow, fhalf) * 16u;   // K sub-step s: ^ (s << 5)
-  const uint32_t wa0 = (uint32_t)tile_chunk(wave_c * 64 + frow, fhalf) * 16u;
+  const uint32_t wa0 = (uint32_t)tile_chunk(wave_c * WCH + frow, fhalf) * 16u;
 
   // weight copies: a wave copies kF2WD consecutive 1 KiB blocks (8 rows each) of
   // the tile; lane i of a copy writes chunk i of the block and reads the source
@@ -436,14 +438,22 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
     const uint32_t dst = lds_w + (uint32_t)islot * kWTile + (uint32_t)(wave * kF2WD) * 1024u;
     if (!(MDCN_F2_ABLATE & 2)) {
       // (the instruction's offset moves the LDS side along with the global one)
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
-                   "global_load_lds_dwordx4 %1, %3\n\t"
-                   "global_load_lds_dwordx4 %2, %3 offset:1024\n\t"
-                   "global_load_lds_dwordx4 %1, %3 offset:2048\n\t"
-                   "global_load_lds_dwordx4 %2, %3 offset:3072"
-                   :
-                   : "s"(dst), "v"(voff), "v"(voff_odd), "s"(w_ptr)
-                   : "memory");
+      if constexpr (kF2WD == 4)
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+                     "global_load_lds_dwordx4 %1, %3\n\t"
+                     "global_load_lds_dwordx4 %2, %3 offset:1024\n\t"
+                     "global_load_lds_dwordx4 %1, %3 offset:2048\n\t"
+                     "global_load_lds_dwordx4 %2, %3 offset:3072"
+                     :
+                     : "s"(dst), "v"(voff), "v"(voff_odd), "s"(w_ptr)
+                     : "memory");
+      else
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+                     "global_load_lds_dwordx4 %1, %3\n\t"
+                     "global_load_lds_dwordx4 %2, %3 offset:1024"
+                     :
+                     : "s"(dst), "v"(voff), "v"(voff_odd), "s"(w_ptr)
+                     : "memory");
     }
     if (!advance) return;
     islot = (islot == kF2Slots - 1) ? 0 : islot + 1;
@@ -459,7 +469,7 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
       }
     }
   };
-  static_assert(kF2WD == 4, "issue_weights spells out four copies");
+  static_assert(kF2WD == 4 || kF2WD == 2, "issue_weights spells out the copies");
 
   // One produce block: the weight copies of the step after the blend cursor's,
   // the blend of the cursor's step (gather set SI) into its sample tile, the
@@ -511,12 +521,19 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
     for (int s = 0; s < 2; ++s) {
       const uint32_t xk = xb ^ (uint32_t)(s << 5), wk = wb ^ (uint32_t)(s << 5);
       MDCN_DSREAD(xf[s][0], xk, 0); MDCN_DSREAD(xf[s][1], xk, 4096);
-      MDCN_DSREAD(wf[s][0], wk, 0); MDCN_DSREAD(wf[s][1], wk, 4096);
+      MDCN_DSREAD(wf[s][0], wk, 0);
+      if constexpr (MB == 2) MDCN_DSREAD(wf[s][1], wk, 4096);
     }
+    constexpr int kRd = 2 + MB;  // fragment reads per K sub-step
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
-      if (s < 3) MDCN_LGKMWAIT4(4, xf[s][0], xf[s][1], wf[s][0], wf[s][1]);
-      else MDCN_LGKMWAIT4(0, xf[s][0], xf[s][1], wf[s][0], wf[s][1]);
+      if constexpr (MB == 2) {
+        if (s < 3) MDCN_LGKMWAIT4(kRd, xf[s][0], xf[s][1], wf[s][0], wf[s][1]);
+        else MDCN_LGKMWAIT4(0, xf[s][0], xf[s][1], wf[s][0], wf[s][1]);
+      } else {
+        if (s < 3) MDCN_LGKMWAIT3(kRd, xf[s][0], xf[s][1], wf[s][0]);
+        else MDCN_LGKMWAIT3(0, xf[s][0], xf[s][1], wf[s][0]);
+      }
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
@@ -526,7 +543,8 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
       if (s + 2 < 4) {
         const uint32_t xk = xb ^ (uint32_t)((s + 2) << 5), wk = wb ^ (uint32_t)((s + 2) << 5);
         MDCN_DSREAD(xf[s + 2][0], xk, 0); MDCN_DSREAD(xf[s + 2][1], xk, 4096);
-        MDCN_DSREAD(wf[s + 2][0], wk, 0); MDCN_DSREAD(wf[s + 2][1], wk, 4096);
+        MDCN_DSREAD(wf[s + 2][0], wk, 0);
+        if constexpr (MB == 2) MDCN_DSREAD(wf[s + 2][1], wk, 4096);
       }
     }
   };
@@ -551,7 +569,7 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
     decode(t, ctile, grp, p0);
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
-      const int col = ctile * CT + wave_c * 64 + mb * 32 + frow;
+      const int col = ctile * CT + wave_c * WCH + mb * 32 + frow;
       b[mb] = (a.bias && col < g.cout_g) ? to_f32(((const E *)a.bias)[(long)grp * g.cout_g + col]) : 0.0f;
     }
   };
@@ -654,7 +672,8 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
       // a lane's 64 values travel as 16 quads of 16 bytes; quad j of the wave's lanes is one 1 KiB run.
       // (The offset is opaque to the optimiser, which would otherwise form the addresses below once,
       // ahead of the tile loop, and keep them -- spilled -- across the K loop.)
-      uint32_t voff = (uint32_t)((wave * 16 * 64 + lane) * 16);
+      constexpr int NQ = NB * MB * 4;   // quads per lane
+      uint32_t voff = (uint32_t)((wave * NQ * 64 + lane) * 16);
       asm volatile("" : "+v"(voff));
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
@@ -688,7 +707,7 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
         for (int i = two ? 1 : 0; i < parts; ++i) {
           const unsigned char *src = uniform_ptr(src0);
 #pragma unroll
-          for (int j = 0; j < 16; ++j) {
+          for (int j = 0; j < NQ; ++j) {
             const uint32_t vo = voff + (uint32_t)(j * 1024);
             asm volatile("s_nop 4\n\tglobal_load_dwordx4 %0, %1, %2 sc1"
                          : "=v"(gs[j >> 3][(j >> 2) & 1][j & 3])
@@ -696,8 +715,10 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
           }
           MDCN_VMWAIT4(0, gs[0][0][0], gs[0][0][1], gs[0][0][2], gs[0][0][3]);
           MDCN_VMWAIT4(0, gs[0][1][0], gs[0][1][1], gs[0][1][2], gs[0][1][3]);
-          MDCN_VMWAIT4(0, gs[1][0][0], gs[1][0][1], gs[1][0][2], gs[1][0][3]);
-          MDCN_VMWAIT4(0, gs[1][1][0], gs[1][1][1], gs[1][1][2], gs[1][1][3]);
+          if constexpr (NQ > 8) {
+            MDCN_VMWAIT4(0, gs[1][0][0], gs[1][0][1], gs[1][0][2], gs[1][0][3]);
+            MDCN_VMWAIT4(0, gs[1][1][0], gs[1][1][1], gs[1][1][2], gs[1][1][3]);
+          }
 #pragma unroll
           for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
@@ -762,7 +783,7 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
       const bool plain = vec_ok && pw0 + 64 <= total_px && rem0 + 64 <= plane_out;
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
-        const int col = ctile * CT + wave_c * 64 + mb * 32 + frow;
+        const int col = ctile * CT + wave_c * WCH + mb * 32 + frow;
         const bool col_ok = col < g.cout_g;
         const long cbase = (long)grp * g.cout_g + col;
         const float bvm = bv[mb];
