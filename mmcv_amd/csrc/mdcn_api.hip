@@ -142,7 +142,7 @@ double schedule_rounds(long tiles, int nk, bool may_cut) {
   if (rest == 0) return (double)full;
   const int rounds = (nk + kGatherAhead - 1) / kGatherAhead;
   long parts = 1;
-  if (may_cut) parts = std::max<long>(1, std::min<long>(std::min<long>(stride / rest, kF2SplitMax), rounds / (8 / kGatherAhead)));
+  if (may_cut) parts = std::max<long>(1, std::min<long>(std::min<long>(stride / rest, kCutMax), rounds / (8 / kGatherAhead)));
   return (double)full + 1.0 / (double)parts;
 }
 
@@ -152,8 +152,8 @@ struct Plan {
   int n_chunk;       // images per launch of the fused path
   size_t xt_bytes;   // channels-last copy of one chunk
   size_t wp_bytes;   // packed weights
-  size_t split_bytes;  // eight-wave kernel: buffers and counters of the tiles it cuts along K (may be left out)
-  int split_wgs;     // ... one buffer and one counter per workgroup of its grid
+  size_t cut_bytes;  // eight-wave kernel: buffers and counters of the tiles it cuts along K (may be left out)
+  int cut_wgs;     // ... one buffer and one counter per workgroup of its grid
   // pack-level call only
   int CO, CO_pad;    // conv_offset channels: 3 (2 when unmodulated) * DG * taps, rounded up to 32
   int mask_kind;     // kMaskLogit, or kMaskNone when unmodulated
@@ -182,8 +182,8 @@ int make_plan(const mdcn_params *p, const Geom &g, Plan *pl) {
   if (p->input_nhwc && (!ok || p->path == MDCN_PATH_DIRECT)) return MDCN_ERR_PATH;  // in-place reads: fused kernel only
   pl->fused = ok && p->path != MDCN_PATH_DIRECT;
   pl->CT = pl->KC = pl->n_ctiles = pl->slabs = pl->n_chunk = 0;
-  pl->xt_bytes = pl->wp_bytes = pl->owp_bytes = pl->raw_bytes = pl->split_bytes = 0;
-  pl->split_wgs = 0;
+  pl->xt_bytes = pl->wp_bytes = pl->owp_bytes = pl->raw_bytes = pl->cut_bytes = 0;
+  pl->cut_wgs = 0;
   pl->CO = 3 * g.DG * g.taps;
   pl->CO_pad = (pl->CO + 31) / 32 * 32;
   pl->mask_kind = kMaskLogit;
@@ -210,8 +210,8 @@ int make_plan(const mdcn_params *p, const Geom &g, Plan *pl) {
   pl->xt_bytes = p->input_nhwc ? 0 : align_up((size_t)img * pl->n_chunk);
   pl->wp_bytes = align_up((size_t)g.G * pl->n_ctiles * pl->slabs * g.taps * pl->CT * pl->KC * es);
   if (!p->no_k_split) {  // one 128 x 256 fp32 tile and a counter per workgroup of the persistent grid
-    pl->split_wgs = num_cus() / 8 * 8;
-    pl->split_bytes = align_up((size_t)pl->split_wgs * kPT * kF2CT * 4) + align_up((size_t)pl->split_wgs * 4);
+    pl->cut_wgs = num_cus() / 8 * 8;
+    pl->cut_bytes = align_up((size_t)pl->cut_wgs * kPT * kF2CT * 4) + align_up((size_t)pl->cut_wgs * 4);
   }
   return MDCN_OK;
 }
@@ -235,8 +235,8 @@ int make_pack_plan(const mdcn_pack_params *pp, const Geom &g, Plan *pl) {
       if (pl->CO_pad > 128) {  // accumulator blocks of the conv_offset kernel
         if (p->path == MDCN_PATH_FUSED || p->path == MDCN_PATH_FUSED_SPLIT) return MDCN_ERR_PATH;
         pl->fused = false;
-        pl->xt_bytes = pl->wp_bytes = pl->split_bytes = 0;
-        pl->split_wgs = 0;
+        pl->xt_bytes = pl->wp_bytes = pl->cut_bytes = 0;
+        pl->cut_wgs = 0;
       } else {
         pl->owp_bytes = align_up((size_t)(g.Cin / pl->KC) * g.taps * 4 * (pl->CO_pad / 32) * 64 * 16);
         pl->raw_bytes = align_up((size_t)pl->n_chunk * plane * pl->CO_pad * es);
@@ -287,7 +287,7 @@ hipError_t launch_fused_ct(const FusedArgs &fa, bool unbordered, hipStream_t st)
   // persistent workgroups: one per CU, a multiple of the 8 XCDs
   // (with tiles cut along K, workgroups beyond the tile count take parts of tiles: the whole chip)
   const int total_wg = fa.n_ptiles * fa.n_ctiles * fa.g.G;
-  const int per_xcd = fa.split_max > 1 ? std::max(1, num_cus() / 8)
+  const int per_xcd = fa.cut_max > 1 ? std::max(1, num_cus() / 8)
                                        : std::max(1, std::min((total_wg + 7) / 8, num_cus() / 8));
   if (unbordered)
     hipLaunchKernelGGL((fused_kernel<E, CT, TMAX, MULTI_DG, true>), dim3(per_xcd * 8), dim3(kThreads),
@@ -302,7 +302,7 @@ hipError_t launch_fused_ct(const FusedArgs &fa, bool unbordered, hipStream_t st)
 template <typename E, int CT>
 hipError_t launch_fused2(const FusedArgs &fa, bool unbordered, hipStream_t st) {
   const int total_wg = fa.n_ptiles * fa.n_ctiles * fa.g.G;
-  const int per_xcd = fa.split_max > 1 ? std::max(1, num_cus() / 8)
+  const int per_xcd = fa.cut_max > 1 ? std::max(1, num_cus() / 8)
                                        : std::max(1, std::min((total_wg + 7) / 8, num_cus() / 8));
   if (unbordered)
     hipLaunchKernelGGL((fused2_kernel<E, CT, true>), dim3(per_xcd * 8), dim3(kF2Threads), 0, st, fa);
@@ -408,9 +408,9 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
     E *raw_pm = (E *)(ws + pl.xt_bytes + pl.wp_bytes + pl.owp_bytes);
     const bool own_oconv = px && px->offset_weight;
     const int cof = pl.CO_pad / 32;
-    float *split_part = (float *)(ws + pl.xt_bytes + pl.wp_bytes + pl.owp_bytes + pl.raw_bytes);
-    uint32_t *split_cnt = (uint32_t *)((unsigned char *)split_part + align_up((size_t)pl.split_wgs * kPT * kF2CT * 4));
-    if (!pl.split_bytes) split_part = nullptr, split_cnt = nullptr;
+    float *cut_part = (float *)(ws + pl.xt_bytes + pl.wp_bytes + pl.owp_bytes + pl.raw_bytes);
+    uint32_t *cut_cnt = (uint32_t *)((unsigned char *)cut_part + align_up((size_t)pl.cut_wgs * kPT * kF2CT * 4));
+    if (!pl.cut_bytes) cut_part = nullptr, cut_cnt = nullptr;
 
     // weights: once per call -- inside the launch that re-lays the first batch chunk when the
     // input allows the vector re-layout (whole 16-byte runs per channel row), else on their own
@@ -424,7 +424,7 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
         const int grid = (int)std::min<long>((wtotal + 255) / 256, 1L << 16);
         hipLaunchKernelGGL(pack_weight_kernel<E>, dim3(grid), dim3(256), 0, st, g,
                            (const E *)p->weight, wp, pl.CT, pl.KC, pl.n_ctiles,
-                           pl.slabs, wtotal, split_cnt, pl.split_wgs);
+                           pl.slabs, wtotal, cut_cnt, pl.cut_wgs);
         if (hipGetLastError() != hipSuccess) rc = MDCN_ERR_LAUNCH;
         packed = true;
       }
@@ -450,7 +450,7 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
           const int pack_blocks = (int)std::max<long>(1, std::min<long>(wtotal / (256 * 8), 512));
           hipLaunchKernelGGL(prepass_kernel<E>, dim3((unsigned)(blocks + pack_blocks)), dim3(256), 0, st, gc, in, xt,
                              n_pchunks, g, (const E *)p->weight, wp, pl.CT, pl.KC, pl.n_ctiles, pl.slabs, wtotal,
-                             pack_blocks, split_cnt, pl.split_wgs);
+                             pack_blocks, cut_cnt, pl.cut_wgs);
           packed = true;
         } else {
           hipLaunchKernelGGL((relayout_vec_kernel<E, true>), dim3((unsigned)blocks), dim3(256), 0, st, gc, in, xt,
@@ -527,9 +527,9 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
                            p->mask ? (const E *)p->mask + (size_t)n0 * g.DG * g.taps * plane_out : nullptr, g);
       }
       fa.prof = nullptr;
-      fa.split_max = pl.split_bytes ? kF2SplitMax : 0;
-      fa.split_part = split_part;
-      fa.split_cnt = split_cnt;
+      fa.cut_max = pl.cut_bytes ? kCutMax : 0;
+      fa.cut_part = cut_part;
+      fa.cut_cnt = cut_cnt;
 #if defined(MDCN_F2_PROFILE) && MDCN_F2_PROFILE
       {  // profiling build: phase sums land behind the packed weights (the workspace is over-allocated by the harness)
         static void *prof_buf = nullptr;
@@ -621,7 +621,7 @@ int run(const mdcn_params *p, void *stream, float *ms, const mdcn_pack_params *p
   if (need > 0 && (!p->workspace || p->workspace_bytes < need ||
                    ((uintptr_t)p->workspace % kAlign) != 0))
     return MDCN_ERR_WORKSPACE;
-  if (p->workspace_bytes < need + pl.split_bytes) pl.split_bytes = 0, pl.split_wgs = 0;
+  if (p->workspace_bytes < need + pl.cut_bytes) pl.cut_bytes = 0, pl.cut_wgs = 0;
   hipStream_t st = (hipStream_t)stream;
   switch (p->dtype) {
     case MDCN_F32: return run_typed<float>(p, g, pl, st, ms, px);
@@ -1137,7 +1137,7 @@ size_t mdcn_workspace_bytes(const mdcn_params *p) {
   if (check_params(p, &g, false) != MDCN_OK) return 0;
   Plan pl;
   if (make_plan(p, g, &pl) != MDCN_OK) return 0;
-  return pl.fused ? pl.xt_bytes + pl.wp_bytes + pl.split_bytes : 0;
+  return pl.fused ? pl.xt_bytes + pl.wp_bytes + pl.cut_bytes : 0;
 }
 
 int mdcn_forward(const mdcn_params *p, void *hip_stream) {
@@ -1171,7 +1171,7 @@ size_t mdcn_pack_workspace_bytes(const mdcn_pack_params *pp) {
   if (!pp || check_params(&pp->conv, &g, false) != MDCN_OK) return 0;
   Plan pl;
   if (make_pack_plan(pp, g, &pl) != MDCN_OK) return 0;
-  return pl.xt_bytes + pl.wp_bytes + pl.owp_bytes + pl.raw_bytes + pl.split_bytes;
+  return pl.xt_bytes + pl.wp_bytes + pl.owp_bytes + pl.raw_bytes + pl.cut_bytes;
 }
 
 int mdcn_pack_forward(const mdcn_pack_params *pp, void *hip_stream) {

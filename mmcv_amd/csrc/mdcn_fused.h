@@ -54,6 +54,7 @@ constexpr int kProducerWaves = 4;                        // waves 4 .. 4 + kProd
 constexpr int kThreads = 256 + 64 * kProducerWaves;
 constexpr int kPxPerLane = 8 / kProducerWaves;           // pixels of the tile a producer lane serves
 constexpr int kTapGroups = kProducerWaves / 2;           // producer lanes per pixel in the table build
+constexpr int kCutMax = 4;         // parts a tile of the schedule's last round is cut into at most
 
 struct FusedArgs {
   Geom g;
@@ -73,11 +74,11 @@ struct FusedArgs {
   uint32_t img_bytes;  // bytes between images
   void *prof;          // per-phase clock sums of a profiling build, else unused
   // fused2_kernel only: tiles of the last, partial round of the schedule are cut along K into up to
-  // split_max parts (0 or 1: never) that meet in split_part, gridDim.x buffers of kPT x 256 floats,
-  // counted in split_cnt, gridDim.x words that are zero when the kernel starts
-  int split_max;
-  void *split_part;
-  void *split_cnt;
+  // cut_max parts (0 or 1: never) that meet in cut_part, gridDim.x buffers of kPT x 256 floats,
+  // counted in cut_cnt, gridDim.x words that are zero when the kernel starts
+  int cut_max;
+  void *cut_part;
+  void *cut_cnt;
 };
 
 typedef __attribute__((address_space(3))) void *lptr_t;
@@ -335,7 +336,7 @@ __device__ __forceinline__ const unsigned char *uniform_ptr(const unsigned char 
 // rest < stride tiles, and without further ado `rest` workgroups would compute a
 // whole tile while the others wait.  Instead each of those tiles is cut along K
 // into parts = stride / rest ranges (whole multiples of `round` steps, at most
-// split_max of them, each at least `min_rounds` rounds long), one per workgroup:
+// cut_max of them, each at least `min_rounds` rounds long), one per workgroup:
 // a "unit" is a tile together with a range of K steps; a workgroup walks whole
 // tiles first (units 0 .. T_full - 1) and at most one part last.  The parts of
 // a tile meet in memory.
@@ -345,7 +346,7 @@ struct UnitSchedule {
   bool has_part;
   int parts, part_tile, part_idx, part_kb, part_pad;
 
-  __device__ __forceinline__ void init(int total_tiles, int nk_pad, int round, int min_rounds, int split_max) {
+  __device__ __forceinline__ void init(int total_tiles, int nk_pad, int round, int min_rounds, int cut_max) {
     xcd = (int)(blockIdx.x & 7);
     wg = (int)(blockIdx.x >> 3);
     stride = (int)(gridDim.x >> 3);
@@ -356,10 +357,10 @@ struct UnitSchedule {
     const int rest = chunk_x - full_rounds * stride;
     const int rounds = nk_pad / round;
     parts = 1;
-    if (split_max > 1 && rest > 0) parts = max(1, min(min(stride / rest, split_max), rounds / min_rounds));
-    const bool split = parts > 1;
-    T_full = full_rounds + ((!split && wg < rest) ? 1 : 0);
-    has_part = split && wg < rest * parts;
+    if (cut_max > 1 && rest > 0) parts = max(1, min(min(stride / rest, cut_max), rounds / min_rounds));
+    const bool cut = parts > 1;
+    T_full = full_rounds + ((!cut && wg < rest) ? 1 : 0);
+    has_part = cut && wg < rest * parts;
     T = T_full + (has_part ? 1 : 0);
     part_tile = xcd * chunk + full_rounds * stride + wg / parts;
     part_idx = wg - (wg / parts) * parts;
@@ -459,7 +460,7 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
   // neighbouring tiles share stay in its L2.  Tiles of the run's last round are
   // cut along K (UnitSchedule): parts of at least 8 steps.
   UnitSchedule us;
-  us.init(a.n_ptiles * a.n_ctiles * g.G, nk_tile_pad, kGatherAhead, 8 / kGatherAhead, a.split_max);
+  us.init(a.n_ptiles * a.n_ctiles * g.G, nk_tile_pad, kGatherAhead, 8 / kGatherAhead, a.cut_max);
   bool first_tile = true;
 
   for (int u = 0; u < us.T; ++u, first_tile = false) {
@@ -756,7 +757,7 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
         constexpr int CQ = 8;                     // quads read back at a time (NQ is a multiple of 8)
         const int tslot = us.counter_slot();
         const unsigned char *pbase =
-            (const unsigned char *)a.split_part + (size_t)us.buffer_slot0() * (size_t)(PT * 256 * 4);
+            (const unsigned char *)a.cut_part + (size_t)us.buffer_slot0() * (size_t)(PT * 256 * 4);
         const unsigned char *mine = uniform_ptr(pbase + (size_t)us.part_idx * (size_t)(PT * 256 * 4));
         // quad j of the 256 consumer lanes is one 4 KiB run.  (The offset is opaque to the optimiser,
         // which would otherwise form the addresses below ahead of the unit loop and keep them live.)
@@ -779,7 +780,7 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         MDCN_BARRIER_LDS();
         if (tid == 0)
-          part_arrived = __hip_atomic_fetch_add((uint32_t *)a.split_cnt + tslot, 1u, __ATOMIC_RELAXED,
+          part_arrived = __hip_atomic_fetch_add((uint32_t *)a.cut_cnt + tslot, 1u, __ATOMIC_RELAXED,
                                                 __HIP_MEMORY_SCOPE_AGENT);
         MDCN_BARRIER_LDS();
         store_tile = part_arrived == (uint32_t)(us.parts - 1);
@@ -810,7 +811,7 @@ __global__ __launch_bounds__(kThreads, 2) void fused_kernel(FusedArgs a) {
             src0 += PT * 256 * 4;
           }
           if (tid == 0)
-            __hip_atomic_store((uint32_t *)a.split_cnt + tslot, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store((uint32_t *)a.cut_cnt + tslot, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
       }
 

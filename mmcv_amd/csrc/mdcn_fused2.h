@@ -60,7 +60,6 @@ constexpr int kF2Unroll = 6;           // steps per round of the K loop: sets, s
 static_assert(kF2Unroll % kF2Sets == 0 && kF2Unroll % 2 == 0 && kF2Unroll % kF2Slots == 0, "static indices");
 
 constexpr int kF2Taps = kTapsSmall;    // table capacity (kh * kw)
-constexpr int kF2SplitMax = 4;         // parts a tile of the schedule's last round is cut into at most
 constexpr int kF2MinSteps = 18;        // padded steps per tile the streaming needs (the next table is built in the second pass of the K loop)
 constexpr size_t fused2_lds_bytes(int CT) {
   return (size_t)2 * kPT * kRowB + (size_t)kF2Slots * CT * kRowB + (size_t)2 * kPT * kF2Taps * 12 + 16;
@@ -228,7 +227,7 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
   __shared__ uint4 Ws[kF2Slots][CT * kRowChunks];        // weight tiles
   __shared__ uint32_t tpix[2][TBL];                      // (pixel, tap) tables, [tap][PT]: corner byte offset
   __shared__ uint2 tws[2][TBL];                          // ... and the blend weights
-  __shared__ uint32_t part_arrived;                      // parts of a split tile that were there before this one
+  __shared__ uint32_t part_arrived;                      // parts of a cut tile that were there before this one
 
   const Geom &g = a.g;
   const int taps = g.taps;
@@ -273,7 +272,7 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
   // rarely is a multiple of `stride`: the last round has r < stride tiles, and
   // without further ado r workgroups would compute a whole tile while the others
   // wait.  Instead each of those r tiles is cut along K into f = stride / r parts
-  // (whole rounds of kF2Unroll steps, at most a.split_max parts), one part per
+  // (whole rounds of kF2Unroll steps, at most a.cut_max parts), one part per
   // workgroup: a "unit" is a tile together with a range of K steps, every
   // workgroup walks whole tiles first and at most one part last.  The parts of a
   // tile meet in memory (see the epilogue).
@@ -288,10 +287,10 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
   const int full_rounds = chunk_x / stride;
   const int rest = chunk_x - full_rounds * stride;       // tiles of the last, partial round
   int parts = 1;
-  if (a.split_max > 1 && rest > 0) parts = min(min(stride / rest, a.split_max), nk_pad / kF2Unroll);
-  const bool split = parts > 1;
-  const int T_full = full_rounds + ((!split && wg < rest) ? 1 : 0);
-  const bool has_part = split && wg < rest * parts;
+  if (a.cut_max > 1 && rest > 0) parts = min(min(stride / rest, a.cut_max), nk_pad / kF2Unroll);
+  const bool cut = parts > 1;
+  const int T_full = full_rounds + ((!cut && wg < rest) ? 1 : 0);
+  const bool has_part = cut && wg < rest * parts;
   const int T = T_full + (has_part ? 1 : 0);
   if (T == 0) return;
   // this workgroup's part: tile, index among the tile's parts, K range
@@ -667,7 +666,7 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
         for (int h = 0; h < 2; ++h) MDCN_VMWAIT4(0, gs[si][h][0], gs[si][h][1], gs[si][h][2], gs[si][h][3]);
       const int tslot = xcd * stride + wg / parts;                       // the tile's counter
       const unsigned char *pbase =
-          (const unsigned char *)a.split_part + (size_t)(xcd * stride + (wg / parts) * parts) * (size_t)(PT * CT * 4);
+          (const unsigned char *)a.cut_part + (size_t)(xcd * stride + (wg / parts) * parts) * (size_t)(PT * CT * 4);
       const unsigned char *mine = uniform_ptr(pbase + (size_t)part_idx * (size_t)(PT * CT * 4));
       // a lane's 64 values travel as 16 quads of 16 bytes; quad j of the wave's lanes is one 1 KiB run.
       // (The offset is opaque to the optimiser, which would otherwise form the addresses below once,
@@ -694,7 +693,7 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
       if (tid == 0)
-        part_arrived = __hip_atomic_fetch_add((uint32_t *)a.split_cnt + tslot, 1u, __ATOMIC_RELAXED,
+        part_arrived = __hip_atomic_fetch_add((uint32_t *)a.cut_cnt + tslot, 1u, __ATOMIC_RELAXED,
                                               __HIP_MEMORY_SCOPE_AGENT);
       __syncthreads();
       store_tile = part_arrived == (uint32_t)(parts - 1);
@@ -734,7 +733,7 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
           src0 += PT * CT * 4;
         }
         if (tid == 0)
-          __hip_atomic_store((uint32_t *)a.split_cnt + tslot, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store((uint32_t *)a.cut_cnt + tslot, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
 

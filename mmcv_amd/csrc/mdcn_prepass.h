@@ -191,7 +191,7 @@ __global__ __launch_bounds__(256) void relayout_vec_kernel(Geom g, const E *__re
 // group, Cout tile and K step (channel slab outer, tap inner) one dense
 // CT x KC tile, K contiguous, zero rows past Cout/G.  The main kernel copies
 // such a tile to LDS with straight 16-byte loads.  Element idx, idx + stride, ...
-// Also clears the `zero_n` words at `zero_ptr` (the main kernel's split-tile counters).
+// Also clears the `zero_n` words at `zero_ptr` (the main kernel's cut-tile counters).
 template <typename E>
 __device__ __forceinline__ void pack_weight_elems(const Geom &g, const E *__restrict__ w, E *__restrict__ wp, int CT,
                                                   int KC, int n_ctiles, int slabs, long total, long first,
