@@ -94,6 +94,8 @@ def cpu_baseline(case, flops_per_sample, budget_s=20.0):
                    f'({tn / n * 1e3:.0f} ms/sample; im2col stage is single-threaded, '
                    f'GEMM uses {threads} threads)'),
         'ms_per_layer_extrapolated': round(tn / n * N * 1e3, 1),
+        'host': {'cpu_count': os.cpu_count(), 'affinity': len(os.sched_getaffinity(0)),
+                 'torch_threads': torch.get_num_threads()},
     }, y_ref
 
 
@@ -507,7 +509,12 @@ def main():
         y_gpu = out[:n_ref].float().cpu().numpy()
         err = float(np.abs(y_gpu - y_ref).max() / np.abs(y_ref).max())
         tol = 1e-4 if dname == 'f32' else 2e-2
+        # element-wise as well: |y - y_ref| <= tol * |y_ref| + tol * rms(y_ref)
+        rms = float(np.sqrt(np.mean(np.square(y_ref, dtype=np.float64))))
+        viol = int((np.abs(y_gpu - y_ref) > tol * np.abs(y_ref) + tol * rms).sum())
         rec['parity'] = {'max_abs_err_over_max_abs_ref': float(f'{err:.3e}'), 'tolerance': tol,
+                         'allclose_rtol_tol_atol_tol_rms': viol == 0, 'violating_elements': viol,
+                         'elements': int(y_ref.size),
                          'samples_checked': n_ref, 'of': N, 'ok': bool(err <= tol and np.isfinite(y_gpu).all()),
                          'against': rec['cpu_baseline']['kind'] + ' CPU path on the same rounded inputs'}
         log('parity', rec['parity'])
