@@ -5,7 +5,8 @@
 // Eight wavefronts, all alike.  Per K step (128 bytes of channels of one tap)
 // every wave
 //   * "produces" 16 of the tile's 128 pixels: waits for the gather it issued
-//     three steps earlier (4 corners x 2 x 16 bytes per lane, held in registers),
+//     three steps earlier (4 corners x 16 bytes of each of two pixels per lane,
+//     held in registers: eight lanes read a pixel's whole 128-byte row),
 //     blends the corners into 2 x 16 bytes of the sample tile, writes them to
 //     LDS and refills the registers with the gather of three steps ahead;
 //   * issues its share (4 x 1 KiB) of the direct-to-LDS copy of the weight tile
@@ -245,11 +246,15 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
   const uint32_t lds_x = (uint32_t)(uintptr_t)(lptr_t)(&Xs[0][0]);
   const uint32_t lds_w = (uint32_t)(uintptr_t)(lptr_t)(&Ws[0][0]);
 
-  // ---- produce role: lane serves 16-byte chunks q and q + 4 of pixel pl
-  const int q = lane & 3;
-  const int pl = wave * 16 + (lane >> 2);
-  const uint32_t xw0 = lds_x + (uint32_t)tile_chunk(pl, q) * 16u;       // where its two chunks go in X[0]
-  const uint32_t xw1 = lds_x + (uint32_t)tile_chunk(pl, q + 4) * 16u;
+  // ---- produce role: lane serves 16-byte chunk ck of pixels pl and pl + 8, so that
+  // one load instruction of the wave reads whole 128-byte rows of 8 pixels (half as
+  // many cache lines per instruction as half rows of 16 pixels, which the vector
+  // cache serves measurably faster)
+  const int q = lane & 3;            // row of the lane in its block of four (the matrix-pipe blend)
+  const int ck = lane & 7;
+  const int pl = wave * 16 + (lane >> 3);
+  const uint32_t xw0 = lds_x + (uint32_t)tile_chunk(pl, ck) * 16u;       // where the two chunks go in X[0]
+  const uint32_t xw1 = lds_x + (uint32_t)tile_chunk(pl + 8, ck) * 16u;
   const unsigned char *xt = (const unsigned char *)a.xt;
   const uint32_t pxb = UNBORDERED ? a.px_bytes : (uint32_t)kRowB;
 
@@ -389,12 +394,12 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
   // gather registers: sets x two halves of the 128-byte row x four corners
   u32x4 gs[kF2Sets][2][4];
 
-  uint32_t o_tl, o_tr, o_bl, o_br;
+  uint32_t o_px[2];  // top-left corner of the lane's two pixels
   auto next_addresses = [&]() {
-    o_tl = tpix[g_t & 1][g_tap * PT + pl] + (uint32_t)(g_slab0 + g_slab) * a.slab_bytes + (uint32_t)q * 16u;
-    o_tr = o_tl + pxb;
-    o_bl = o_tl + a.row_bytes;
-    o_br = o_bl + pxb;
+    const uint32_t *tp_ = &tpix[g_t & 1][g_tap * PT + pl];
+    const uint32_t add_ = (uint32_t)(g_slab0 + g_slab) * a.slab_bytes + (uint32_t)ck * 16u;
+    o_px[0] = tp_[0] + add_;
+    o_px[1] = tp_[8] + add_;
     ++g_s;
     if (g_s < g_n) {
       if (++g_tap == taps) {
@@ -417,10 +422,14 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
   };
 #define MDCN_F2_GATHER_HALF(S, H)                     \
   do {                                                \
-    MDCN_GLOAD(S[H][0], o_tl, xt, 0 + 64 * (H));      \
-    MDCN_GLOAD(S[H][1], o_tr, xt, 0 + 64 * (H));      \
-    MDCN_GLOAD(S[H][2], o_bl, xt, 0 + 64 * (H));      \
-    MDCN_GLOAD(S[H][3], o_br, xt, 0 + 64 * (H));      \
+    const uint32_t tl_ = o_px[H];                     \
+    const uint32_t tr_ = tl_ + pxb;                   \
+    const uint32_t bl_ = tl_ + a.row_bytes;           \
+    const uint32_t br_ = bl_ + pxb;                   \
+    MDCN_GLOAD(S[H][0], tl_, xt, 0);                  \
+    MDCN_GLOAD(S[H][1], tr_, xt, 0);                  \
+    MDCN_GLOAD(S[H][2], bl_, xt, 0);                  \
+    MDCN_GLOAD(S[H][3], br_, xt, 0);                  \
   } while (0)
 #define MDCN_F2_GATHER(SI)                            \
   do {                                                \
@@ -478,17 +487,20 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
     if (b_t < T) {                                                                      \
       issue_weights(true);                                                              \
       next_addresses();                                                                 \
-      const typename BL::Wt w_ = BL::prep(tws[b_t & 1][b_tap * PT + pl], q);               \
+      const uint2 *tw_ = &tws[b_t & 1][b_tap * PT + pl];                                \
+      const uint2 tw0_ = tw_[0], tw1_ = tw_[8];                                         \
       const uint32_t xo_ = (b_s & 1) ? kXTile : 0u;                                     \
-      MDCN_VMWAIT4(kF2VmBlend, gs[SI][0][0], gs[SI][0][1], gs[SI][0][2], gs[SI][0][3]); \
       {                                                                                 \
+        const typename BL::Wt w_ = BL::prep(tw0_, q);                                   \
+        MDCN_VMWAIT4(kF2VmBlend, gs[SI][0][0], gs[SI][0][1], gs[SI][0][2], gs[SI][0][3]); \
         const u32x4 o_ = (MDCN_F2_ABLATE & 4) ? (gs[SI][0][0] ^ gs[SI][0][1] ^ gs[SI][0][2] ^ gs[SI][0][3]) \
                                               : BL::run(gs[SI][0], w_);                 \
         *(lds_u32x4_ptr)(xw0 + xo_) = o_;                                               \
       }                                                                                 \
       MDCN_F2_GATHER_HALF(gs[SI], 0);                                                   \
-      MDCN_VMWAIT4(kF2VmBlend, gs[SI][1][0], gs[SI][1][1], gs[SI][1][2], gs[SI][1][3]); \
       {                                                                                 \
+        const typename BL::Wt w_ = BL::prep(tw1_, q);                                   \
+        MDCN_VMWAIT4(kF2VmBlend, gs[SI][1][0], gs[SI][1][1], gs[SI][1][2], gs[SI][1][3]); \
         const u32x4 o_ = (MDCN_F2_ABLATE & 4) ? (gs[SI][1][0] ^ gs[SI][1][1] ^ gs[SI][1][2] ^ gs[SI][1][3]) \
                                               : BL::run(gs[SI][1], w_);                 \
         *(lds_u32x4_ptr)(xw1 + xo_) = o_;                                               \
