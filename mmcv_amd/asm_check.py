@@ -9,6 +9,19 @@ into assembly text, so a reload it places right in front of an asm statement
 would make the statement read a stale base address.  This scan fails the build
 when it finds such a pair; the cure is an ``s_nop`` at the head of the asm
 statement or fewer live scalars around it.
+
+Second check: the loads (global_load, ds_read) those asm statements issue
+complete asynchronously, and the code waits for them with explicit ``s_waitcnt``
+counts.  The compiler believes an asm statement's outputs are valid when the
+statement ends, so it is free to copy such a register elsewhere, or to reuse it
+as a temporary, between the load and the wait -- reading stale data, or having
+the landing load overwrite an address.  The waits of the kernels therefore name
+the registers they release in a trailing comment (``s_waitcnt vmcnt(32) ; v[4:7]
+...``).  The scan follows every path through a kernel's basic blocks with the
+set of registers that may still be locked -- locked by an asm-issued load,
+released by an asm wait that names them or by any wait for count 0 -- and
+fails the build when an instruction touches a locked register.  (Whether the
+count of a wait is right is not checked here; the parity tests do that.)
 """
 import re
 import sys
@@ -70,12 +83,144 @@ def violations(asm_text):
     return found
 
 
+_VREG = re.compile(r'\bv\[(\d+):(\d+)\]|\bv(\d+)\b')
+_VMCNT = re.compile(r'vmcnt\((\d+)\)')
+_LGKMCNT = re.compile(r'lgkmcnt\((\d+)\)')
+_BRANCH = re.compile(r'^s_c?branch\w*\s+(\.?\w+)')
+
+
+def _vregs(text):
+    regs = set()
+    for m in _VREG.finditer(text):
+        if m.group(1):
+            regs |= set(range(int(m.group(1)), int(m.group(2)) + 1))
+        else:
+            regs.add(int(m.group(3)))
+    return regs
+
+
+def _wait_counts(t):
+    """(vmcnt, lgkmcnt) of an s_waitcnt; None for a counter it leaves alone."""
+    vm, lg = _VMCNT.search(t), _LGKMCNT.search(t)
+    if vm or lg or 'expcnt' in t:
+        return (int(vm.group(1)) if vm else None, int(lg.group(1)) if lg else None)
+    try:
+        imm = int(t.split(None, 1)[1].strip(), 0)
+    except (ValueError, IndexError):
+        return (None, None)
+    vmc = (imm & 0xF) | (((imm >> 14) & 0x3) << 4)
+    lgc = (imm >> 8) & 0xF
+    return (None if vmc == 63 else vmc, None if lgc == 15 else lgc)
+
+
+def _kernels(asm_text):
+    """[(name, [(line number, instruction, comment, inside inline asm)], {label: index})] per function."""
+    out, cur, labels, in_asm = [], None, None, False
+    for no, line in enumerate(asm_text.split('\n'), 1):
+        t = line.strip()
+        if t.startswith(';;#ASMSTART'):
+            in_asm = True
+            continue
+        if t.startswith(';;#ASMEND'):
+            in_asm = False
+            continue
+        if not t or t[0] == ';':
+            continue
+        code, _, comment = t.partition(';')
+        code = code.strip()
+        if code.endswith(':') and t[0] != '.':
+            cur, labels = [], {}
+            out.append((code[:-1], cur, labels))
+            continue
+        if cur is None:
+            continue
+        if code.endswith(':') and t.startswith('.L'):
+            labels[code[:-1]] = len(cur)
+            continue
+        if t[0] == '.':
+            continue
+        cur.append((no, code, comment, in_asm))
+    return out
+
+
+def inflight_violations(asm_text):
+    """[(kernel, line number, instruction, registers)] for every instruction that
+    touches a register which a load issued from inline asm may still be writing."""
+    found = set()
+    for name, ins, labels in _kernels(asm_text):
+        if not any(a and (c.startswith('ds_read') or (c.startswith(_VMEM) and 'load' in c and '_lds_' not in c))
+                   for _, c, _, a in ins):
+            continue
+        n = len(ins)
+        leaders = {0} | {i for i in labels.values() if i < n}
+        succ_of = {}
+        for k, (no, t, _, _) in enumerate(ins):
+            m = _BRANCH.match(t)
+            if m:
+                tgt = labels.get(m.group(1))
+                nxt = [tgt] if tgt is not None and tgt < n else []
+                if t.startswith('s_cbranch') and k + 1 < n:
+                    nxt.append(k + 1)
+                succ_of[k] = nxt
+                if k + 1 < n:
+                    leaders.add(k + 1)
+            elif t.startswith(('s_endpgm', 's_setpc', 's_swappc')):
+                succ_of[k] = []
+                if k + 1 < n:
+                    leaders.add(k + 1)
+        starts = sorted(leaders)
+        end_of = {b: (starts[i + 1] if i + 1 < len(starts) else n) for i, b in enumerate(starts)}
+        at_entry = {0: (frozenset(), frozenset())}
+        work = [0]
+        while work:
+            b = work.pop()
+            vm, lg = set(at_entry[b][0]), set(at_entry[b][1])
+            for k in range(b, end_of[b]):
+                no, t, comment, in_asm = ins[k]
+                if t.startswith('s_waitcnt'):
+                    vmc, lgc = _wait_counts(t)
+                    named = _vregs(comment) if in_asm else set()
+                    if vmc == 0:
+                        vm.clear()
+                    elif vmc is not None:
+                        vm -= named
+                    if lgc == 0:
+                        lg.clear()
+                    elif lgc is not None:
+                        lg -= named
+                    continue
+                touched = _vregs(t.split(None, 1)[1]) if ' ' in t else set()
+                hit = touched & (vm | lg)
+                if hit:
+                    found.add((name, no, t, tuple(sorted(hit))))
+                if in_asm:
+                    op, _, rest = t.partition(' ')
+                    if op.startswith(_VMEM) and 'load' in op and '_lds_' not in op:
+                        vm |= _vregs(rest.split(',')[0])
+                    elif op.startswith('ds_read'):
+                        lg |= _vregs(rest.split(',')[0])
+            last = end_of[b] - 1
+            out_state = (frozenset(vm), frozenset(lg))
+            for nb in succ_of.get(last, [end_of[b]] if end_of[b] < n else []):
+                old = at_entry.get(nb)
+                new = out_state if old is None else (old[0] | out_state[0], old[1] | out_state[1])
+                if new != old:
+                    at_entry[nb] = new
+                    work.append(nb)
+    return sorted(found, key=lambda v: (v[0], v[1]))
+
+
 def check_file(path):
     with open(path) as f:
-        bad = violations(f.read())
+        text = f.read()
+    bad = violations(text)
     for no, t, regs, dist, writer in bad:
         print(f'{path}:{no}: "{t}" reads s{regs} {dist} slot(s) after "{writer}"', file=sys.stderr)
-    return len(bad)
+    early = inflight_violations(text)
+    for name, no, t, regs in early:
+        print(f'{path}:{no}: {name}: "{t}" touches v{list(regs)} while a load issued from inline asm may still '
+              'be writing it', file=sys.stderr)
+    return len(bad) + len(early)
 
 
 if __name__ == '__main__':

@@ -60,8 +60,8 @@ def build_hip(extra=(), check=True):
             raise RuntimeError('no device assembly found to check')
         bad = sum(asm_check.check_file(f) for f in asm)
         if bad:
-            raise RuntimeError(f'{bad} inline-asm vector-memory instruction(s) read a scalar register too soon '
-                               'after a vector instruction wrote it (see above)')
+            raise RuntimeError(f'{bad} finding(s) in the device assembly around inline-asm memory instructions '
+                               '(see above and asm_check.py)')
         print(f'asm_check: {len(asm)} device assembly file(s) clean', flush=True)
         shutil.move(out, HIP_LIB)
     finally:

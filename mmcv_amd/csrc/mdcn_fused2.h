@@ -87,13 +87,14 @@ constexpr size_t fused2_lds_bytes(int CT) {
 #define MDCN_DSREAD(dst, addr, imm) \
   asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(imm))
 // wait until at most N vector-memory (LDS) operations of this wave are outstanding;
-// the four registers become usable only afterwards
+// the four registers become usable only afterwards (the comment names them for the
+// build's scan of the assembly, asm_check.py)
 #define MDCN_VMWAIT4(N, a, b, c, d) \
-  asm volatile("s_waitcnt vmcnt(%4)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) : "n"(N))
+  asm volatile("s_waitcnt vmcnt(%4) ; %0 %1 %2 %3" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) : "n"(N))
 #define MDCN_LGKMWAIT4(N, a, b, c, d) \
-  asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) : "n"(N))
+  asm volatile("s_waitcnt lgkmcnt(%4) ; %0 %1 %2 %3" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) : "n"(N))
 #define MDCN_LGKMWAIT3(N, a, b, c) \
-  asm volatile("s_waitcnt lgkmcnt(%3)" : "+v"(a), "+v"(b), "+v"(c) : "n"(N))
+  asm volatile("s_waitcnt lgkmcnt(%3) ; %0 %1 %2" : "+v"(a), "+v"(b), "+v"(c) : "n"(N))
 typedef __attribute__((address_space(3))) u32x4 *lds_u32x4_ptr;
 
 // Blend of one 16-byte chunk (8 channels) from the same chunk at the four
@@ -495,7 +496,7 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
         MDCN_VMWAIT4(kF2VmBlend, gs[SI][0][0], gs[SI][0][1], gs[SI][0][2], gs[SI][0][3]); \
         const u32x4 o_ = (MDCN_F2_ABLATE & 4) ? (gs[SI][0][0] ^ gs[SI][0][1] ^ gs[SI][0][2] ^ gs[SI][0][3]) \
                                               : BL::run(gs[SI][0], w_);                 \
-        *(lds_u32x4_ptr)(xw0 + xo_) = o_;                                               \
+        *(lds_u32x4_ptr)(uintptr_t)(xw0 + xo_) = o_;                                    \
       }                                                                                 \
       MDCN_F2_GATHER_HALF(gs[SI], 0);                                                   \
       {                                                                                 \
@@ -503,7 +504,7 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
         MDCN_VMWAIT4(kF2VmBlend, gs[SI][1][0], gs[SI][1][1], gs[SI][1][2], gs[SI][1][3]); \
         const u32x4 o_ = (MDCN_F2_ABLATE & 4) ? (gs[SI][1][0] ^ gs[SI][1][1] ^ gs[SI][1][2] ^ gs[SI][1][3]) \
                                               : BL::run(gs[SI][1], w_);                 \
-        *(lds_u32x4_ptr)(xw1 + xo_) = o_;                                               \
+        *(lds_u32x4_ptr)(uintptr_t)(xw1 + xo_) = o_;                                    \
       }                                                                                 \
       MDCN_F2_GATHER_HALF(gs[SI], 1);                                                   \
       ++b_s;                                                                            \

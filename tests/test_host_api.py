@@ -334,3 +334,41 @@ def test_asm_check_flags_scalar_written_too_close_to_inline_vector_memory():
         '\t;;#ASMSTART\n\tglobal_load_dwordx4 v[2:5], v1, s[6:7]\n\t;;#ASMEND\n'
     assert asm_check.violations(spaced) == []
     assert len(asm_check.violations(spaced.replace('\tv_mov_b32_e32 v2, v3\n' * 5, '\tv_mov_b32_e32 v2, v3\n' * 4))) == 1
+
+
+def test_asm_check_flags_registers_touched_while_an_inline_load_is_in_flight():
+    """Second scan of mmcv_amd/asm_check.py: a register that an asm-issued load has not
+    delivered yet (no wait that names it, no wait for count 0) must not be touched --
+    the compiler would otherwise copy stale data or reuse the register as a temporary."""
+    from mmcv_amd import asm_check
+    head = 'kern:\n'
+    load = '\t;;#ASMSTART\n\tglobal_load_dwordx4 v[2:5], v[8:9], off\n\t;;#ASMEND\n'
+    wait = '\t;;#ASMSTART\n\ts_waitcnt vmcnt(8) ; v[2:5] v[10:13]\n\t;;#ASMEND\n'
+    use = '\tv_xor_b32_e32 v20, v2, v20\n'
+    assert asm_check.inflight_violations(head + load + wait + use + '\ts_endpgm\n') == []
+    # a copy before the wait, or a wait that names other registers
+    early = asm_check.inflight_violations(head + load + '\tv_mov_b64_e32 v[36:37], v[4:5]\n' + wait + use + '\ts_endpgm\n')
+    assert [(v[1], v[3]) for v in early] == [(5, (4, 5))]
+    other = wait.replace('v[2:5]', 'v[14:17]')
+    assert len(asm_check.inflight_violations(head + load + other + use + '\ts_endpgm\n')) == 1
+    # a wait for everything releases everything, named or not, asm or compiler
+    assert asm_check.inflight_violations(head + load + '\ts_waitcnt vmcnt(0)\n' + use + '\ts_endpgm\n') == []
+    assert len(asm_check.inflight_violations(head + load + '\ts_waitcnt vmcnt(3)\n' + use + '\ts_endpgm\n')) == 1
+    # loads the compiler issued itself are its own business
+    assert asm_check.inflight_violations(head + '\tglobal_load_dwordx4 v[2:5], v[8:9], off\n' + use + '\ts_endpgm\n') == []
+    # around a loop: the load at the bottom of the body is in flight at the top
+    loop = (head + load + '.LBB0_1:\n' + '\tv_mov_b32_e32 v30, v3\n' + wait + use + load +
+            '\ts_cbranch_scc1 .LBB0_1\n\ts_endpgm\n')
+    hits = asm_check.inflight_violations(loop)
+    assert len(hits) == 1 and hits[0][2].startswith('v_mov_b32_e32 v30, v3')
+    # a rotated loop (latch placed before the header in the text) is followed along its edges, not in text order
+    rotated = (head + load + '\ts_branch .LBB0_2\n' + '.LBB0_1:\n' + use + load + '.LBB0_2:\n' + wait +
+               '\ts_cbranch_scc1 .LBB0_1\n\ts_endpgm\n')
+    assert asm_check.inflight_violations(rotated) == []
+    # LDS reads: the other counter
+    ds = '\t;;#ASMSTART\n\tds_read_b128 v[40:43], v7 offset:4096\n\t;;#ASMEND\n'
+    dwait = '\t;;#ASMSTART\n\ts_waitcnt lgkmcnt(2) ; v[40:43]\n\t;;#ASMEND\n'
+    mfma = '\tv_mfma_f32_32x32x16_bf16 v[100:115], v[40:43], v[44:47], v[100:115]\n'
+    assert asm_check.inflight_violations(head + ds + dwait + mfma + '\ts_endpgm\n') == []
+    assert len(asm_check.inflight_violations(head + ds + mfma + dwait + '\ts_endpgm\n')) == 1
+    assert len(asm_check.inflight_violations(head + ds + '\ts_waitcnt vmcnt(0)\n' + mfma + '\ts_endpgm\n')) == 1
