@@ -528,6 +528,13 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
     const uint32_t wb = lds_w + (uint32_t)rslot * kWTile + wa0;
     rslot = (rslot == kF2Slots - 1) ? 0 : rslot + 1;
     if (k >= c_n) return;
+    // The two waves of a SIMD are in opposite phases most of the time.  The MFMA phase is a
+    // stream of long instructions that keeps the matrix pipe busy whenever it gets an issue
+    // slot; the produce block is a chain of short dependent steps (table read, wait, blend,
+    // sample write, gather issue) whose delay moves the step barrier.  So the arbiter is told
+    // to prefer the wave that produces: priority 0 here, 2 from the end of this phase on
+    // (measured: 3 % off the kernel; the opposite preference costs 1 %).
+    __builtin_amdgcn_s_setprio(0);
     u32x4 xf[4][NB], wf[4][MB];
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
@@ -559,6 +566,7 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
         if constexpr (MB == 2) MDCN_DSREAD(wf[s + 2][1], wk, 4096);
       }
     }
+    __builtin_amdgcn_s_setprio(2);
   };
 
 #if MDCN_F2_PROFILE
