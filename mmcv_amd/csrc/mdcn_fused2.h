@@ -446,9 +446,10 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
     const uint32_t voff_odd = voff ^ 32u;
     const uint32_t dst = lds_w + (uint32_t)islot * kWTile + (uint32_t)(wave * kF2WD) * 1024u;
     if (!(MDCN_F2_ABLATE & 2)) {
-      // (the instruction's offset moves the LDS side along with the global one)
+      // (the instruction's offset moves the LDS side along with the global one; the five idle slots
+      // cover a reload of the spilled base pointer right in front of the statement)
       if constexpr (kF2WD == 4)
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\t"
                      "global_load_lds_dwordx4 %1, %3\n\t"
                      "global_load_lds_dwordx4 %2, %3 offset:1024\n\t"
                      "global_load_lds_dwordx4 %1, %3 offset:2048\n\t"
@@ -457,7 +458,7 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
                      : "s"(dst), "v"(voff), "v"(voff_odd), "s"(w_ptr)
                      : "memory");
       else
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\t"
                      "global_load_lds_dwordx4 %1, %3\n\t"
                      "global_load_lds_dwordx4 %2, %3 offset:1024"
                      :
