@@ -142,6 +142,29 @@ def test_outside_taps_never_touch_the_image(path, dtype):
     assert rel_err(y, ref) <= TOL[dtype]
 
 
+@pytest.mark.parametrize('path', [capi.PATH_FUSED, capi.PATH_FUSED_SPLIT, capi.PATH_DIRECT])
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16, torch.float16])
+def test_non_finite_offsets_are_outside(path, dtype):
+    """An offset that is NaN or infinite fails the reference's position test
+    (cpu/modulated_deform_conv.cpp:160: every comparison with NaN is false), so
+    the tap adds nothing and nothing is read for it.  A third of the taps get
+    such offsets here; the rest sample normally."""
+    kw = dict(N=2, Cin=128, Cout=256, H=20, W=26, sigma=1.5)
+    print(f'path={path} dtype={dtype} non-finite offsets', flush=True)
+    case = make_case(9, **kw)
+    off = case['offset']
+    g = torch.Generator().manual_seed(4)
+    kind = torch.randint(0, 9, off.shape, generator=g)
+    off[kind == 0] = float('nan')
+    off[kind == 1] = float('inf')
+    off[kind == 2] = float('-inf')
+    ref = oracle_forward(cast_case(case, dtype))
+    assert np.isfinite(ref).all()
+    y = capi_forward(cast_case(case, dtype, 'cuda'), path=path).float().cpu().numpy()
+    assert np.isfinite(y).all()
+    assert rel_err(y, ref) <= TOL[dtype]
+
+
 # Tiles of the schedule's last round cut along K (both fused kernels): shapes whose tile counts give
 # two, three and four parts per tile on a 256-CU grid, and one with whole rounds in front of the cut one.
 CUT = {
