@@ -52,7 +52,9 @@ struct Prepared {
 // Checks in the order of the reference host op
 // (mmcv/ops/csrc/pytorch/modulated_deform_conv.cpp:68-90), then the dispatch
 // checks (pytorch_device_registry.hpp:115-128).
-void prepare(Prepared &pr, const Tensor &input, const Tensor &weight,
+// false: the batch is empty and there is nothing to do (the reference's loop over
+// samples, modulated_deform_conv.cpp:108-130, runs zero times)
+bool prepare(Prepared &pr, const Tensor &input, const Tensor &weight,
              const Tensor &bias, const Tensor &offset, const Tensor &mask,
              Tensor &output, int kernel_h, int kernel_w, int stride_h,
              int stride_w, int pad_h, int pad_w, int dilation_h, int dilation_w,
@@ -86,6 +88,7 @@ void prepare(Prepared &pr, const Tensor &input, const Tensor &weight,
                 "modulated_deform_conv_forward: expected ", names[i],
                 " to have dtype ", c10::toString(st), " but got ",
                 c10::toString(all[i]->scalar_type()));
+  if (batch == 0) return false;
 
   mdcn_params &p = pr.p;
   p = mdcn_params{};
@@ -146,6 +149,7 @@ void prepare(Prepared &pr, const Tensor &input, const Tensor &weight,
     p.workspace = pr.keep.back().data_ptr();
     p.workspace_bytes = ws;
   }
+  return true;
 }
 
 void modulated_deform_conv_forward(
@@ -160,9 +164,10 @@ void modulated_deform_conv_forward(
   (void)columns;
   c10::DeviceGuard guard(input.device());
   Prepared pr;
-  prepare(pr, input, weight, bias, offset, mask, output, kernel_h, kernel_w,
-          stride_h, stride_w, pad_h, pad_w, dilation_h, dilation_w, group,
-          deformable_group, with_bias);
+  if (!prepare(pr, input, weight, bias, offset, mask, output, kernel_h, kernel_w,
+               stride_h, stride_w, pad_h, pad_w, dilation_h, dilation_w, group,
+               deformable_group, with_bias))
+    return;
   void *stream = (void *)c10::hip::getCurrentHIPStream().stream();
   const int rc = mdcn_forward(&pr.p, stream);
   TORCH_CHECK(rc == MDCN_OK, "modulated_deform_conv_forward: ", mdcn_status_string(rc));
@@ -176,9 +181,10 @@ std::vector<double> modulated_deform_conv_forward_timed(
     int deformable_group, bool with_bias) {
   c10::DeviceGuard guard(input.device());
   Prepared pr;
-  prepare(pr, input, weight, bias, offset, mask, output, kernel_h, kernel_w,
-          stride_h, stride_w, pad_h, pad_w, dilation_h, dilation_w, group,
-          deformable_group, with_bias);
+  if (!prepare(pr, input, weight, bias, offset, mask, output, kernel_h, kernel_w,
+               stride_h, stride_w, pad_h, pad_w, dilation_h, dilation_w, group,
+               deformable_group, with_bias))
+    return {0, 0, 0, 0};
   void *stream = (void *)c10::hip::getCurrentHIPStream().stream();
   float ms[4] = {0, 0, 0, 0};
   const int rc = mdcn_forward_timed(&pr.p, stream, ms);
@@ -222,6 +228,7 @@ std::vector<double> modulated_deform_conv_pack_forward(
     TORCH_CHECK(all[i]->scalar_type() == st, op, ": expected ", names[i], " to have dtype ",
                 c10::toString(st), " but got ", c10::toString(all[i]->scalar_type()));
   }
+  if (batch == 0) return {0, 0, 0, 0, 0};  // nothing to compute, nothing to write
 
   mdcn_pack_params pp{};
   mdcn_params &p = pp.conv;
@@ -404,6 +411,11 @@ void run_backward(const char *op, const Tensor &input, const Tensor &weight, con
     TORCH_CHECK(all[i]->scalar_type() == st, op, ": expected ", names[i], " to have dtype ",
                 c10::toString(st), " but got ", c10::toString(all[i]->scalar_type()));
     if (i >= 4) TORCH_CHECK(all[i]->is_contiguous(), op, ": ", names[i], " must be contiguous");
+  }
+  if (input.size(0) == 0) {  // no sample contributes: the parameter gradients are zero, the others empty
+    if (grad_weight.numel()) grad_weight.zero_();
+    if (grad_bias.numel()) grad_bias.zero_();
+    return;
   }
   mdcn_bwd_params bp{};
   mdcn_params &p = bp.conv;

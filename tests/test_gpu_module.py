@@ -254,3 +254,33 @@ def test_cfg5_layer_shapes(shape):
         err = rel_err(y[n:n + 1].float().cpu().numpy(), oracle_forward(sub))
         print(f'  cfg5 {shape} sample {n}: err {err:.3e}', flush=True)
         assert err <= TOL[torch.bfloat16], (shape, n, err)
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+def test_empty_batch(dtype):
+    """The reference's Python layer refuses an empty batch (its _output_size counts the
+    batch among the sizes that must be positive, mmcv/ops/modulated_deform_conv.py:226-229);
+    its extension op loops over the samples (modulated_deform_conv.cpp:108-130, :186-246)
+    and with none returns without touching anything but the zeroed parameter gradients.
+    Same here at both levels."""
+    from mmcv_amd import _ext
+    from mmcv_amd.ops import modulated_deform_conv2d
+    x = torch.zeros(0, 64, 9, 11, dtype=dtype, device='cuda')
+    off = torch.zeros(0, 18, 9, 11, dtype=dtype, device='cuda')
+    msk = torch.zeros(0, 9, 9, 11, dtype=dtype, device='cuda')
+    w = torch.randn(32, 64, 3, 3, dtype=dtype, device='cuda')
+    b = torch.randn(32, dtype=dtype, device='cuda')
+    with pytest.raises(ValueError, match='convolution input is too small'):
+        modulated_deform_conv2d(x, off, msk, w, b, 1, 1, 1, 1, 1)
+    geo = dict(kernel_h=3, kernel_w=3, stride_h=1, stride_w=1, pad_h=1, pad_w=1, dilation_h=1, dilation_w=1,
+               group=1, deformable_group=1, with_bias=True)
+    out = x.new_empty(0, 32, 9, 11)
+    empty = x.new_empty(0)
+    _ext.modulated_deform_conv_forward(x, w, b, empty, off, msk, out, empty, **geo)
+    gw, gb = torch.full_like(w, 7.0), torch.full_like(b, 7.0)
+    _ext.modulated_deform_conv_backward(x, w, b, empty, off, msk, empty, torch.zeros_like(x), gw, gb,
+                                        torch.zeros_like(off), torch.zeros_like(msk), out, **geo)
+    assert torch.count_nonzero(gw) == 0 and torch.count_nonzero(gb) == 0
+    # mismatched shapes are still refused (the reference checks before it loops)
+    with pytest.raises(RuntimeError, match="kernel channels won't match"):
+        _ext.modulated_deform_conv_forward(x[:, :32], w, b, empty, off, msk, out, empty, **geo)
