@@ -22,6 +22,13 @@ set of registers that may still be locked -- locked by an asm-issued load,
 released by an asm wait that names them or by any wait for count 0 -- and
 fails the build when an instruction touches a locked register.  (Whether the
 count of a wait is right is not checked here; the parity tests do that.)
+Paths are followed without regard to what the branches test, with one
+exception: code that only one kind of wave executes can say so with an asm
+statement that is nothing but the comment ``; mdcn-role <name>``.  A wave keeps
+its role for the whole kernel, so a path that passes markers of two different
+roles cannot occur and is dropped; without this, a kernel that branches on the
+role in several places (first gather sets in another order, barrier at another
+place) is reported for paths that mix the two.
 """
 import re
 import sys
@@ -124,6 +131,9 @@ def _kernels(asm_text):
         if t.startswith(';;#ASMEND'):
             in_asm = False
             continue
+        if in_asm and t.startswith('; mdcn-role ') and cur is not None:
+            cur.append((no, 'role ' + t[len('; mdcn-role '):].strip(), '', True))
+            continue
         if not t or t[0] == ';':
             continue
         code, _, comment = t.partition(';')
@@ -170,13 +180,20 @@ def inflight_violations(asm_text):
                     leaders.add(k + 1)
         starts = sorted(leaders)
         end_of = {b: (starts[i + 1] if i + 1 < len(starts) else n) for i, b in enumerate(starts)}
-        at_entry = {0: (frozenset(), frozenset())}
-        work = [0]
+        at_entry = {(0, None): (frozenset(), frozenset())}  # (block, role of the wave so far) -> locked registers
+        work = [(0, None)]
         while work:
-            b = work.pop()
-            vm, lg = set(at_entry[b][0]), set(at_entry[b][1])
+            b, role = work.pop()
+            vm, lg = set(at_entry[(b, role)][0]), set(at_entry[(b, role)][1])
+            feasible = True
             for k in range(b, end_of[b]):
                 no, t, comment, in_asm = ins[k]
+                if t.startswith('role '):
+                    if role is not None and role != t[5:]:
+                        feasible = False  # a wave of one role never reaches code of another
+                        break
+                    role = t[5:]
+                    continue
                 if t.startswith('s_waitcnt'):
                     vmc, lgc = _wait_counts(t)
                     named = _vregs(comment) if in_asm else set()
@@ -199,14 +216,16 @@ def inflight_violations(asm_text):
                         vm |= _vregs(rest.split(',')[0])
                     elif op.startswith('ds_read'):
                         lg |= _vregs(rest.split(',')[0])
+            if not feasible:
+                continue
             last = end_of[b] - 1
             out_state = (frozenset(vm), frozenset(lg))
             for nb in succ_of.get(last, [end_of[b]] if end_of[b] < n else []):
-                old = at_entry.get(nb)
+                old = at_entry.get((nb, role))
                 new = out_state if old is None else (old[0] | out_state[0], old[1] | out_state[1])
                 if new != old:
-                    at_entry[nb] = new
-                    work.append(nb)
+                    at_entry[(nb, role)] = new
+                    work.append((nb, role))
     return sorted(found, key=lambda v: (v[0], v[1]))
 
 

@@ -96,6 +96,9 @@ constexpr size_t fused2_lds_bytes(int CT) {
 #define MDCN_LGKMWAIT3(N, a, b, c) \
   asm volatile("s_waitcnt lgkmcnt(%3) ; %0 %1 %2" : "+v"(a), "+v"(b), "+v"(c) : "n"(N))
 typedef __attribute__((address_space(3))) u32x4 *lds_u32x4_ptr;
+// Marks code that only waves of one role execute (a comment in the assembly, no instruction): the
+// build's scan of the assembly drops paths that would pass markers of two roles (asm_check.py).
+#define MDCN_ROLE(name) asm volatile("; mdcn-role " name)
 
 // Blend of one 16-byte chunk (8 channels) from the same chunk at the four
 // corners.  The table keeps the four mask-scaled bilinear weights as two words of
@@ -601,6 +604,7 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
   MDCN_BARRIER_LDS();  // table visible
   __builtin_amdgcn_sched_barrier(0);
   if (!late) {
+    MDCN_ROLE("early");
     MDCN_F2_GATHER(0);
     issue_weights(true);
     MDCN_F2_GATHER(1);
@@ -608,6 +612,7 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
     MDCN_F2_GATHER(2);
     MDCN_F2_BLOCK(0);
   } else {
+    MDCN_ROLE("late");
     MDCN_F2_GATHER(2);
     issue_weights(true);
     MDCN_F2_GATHER(0);
@@ -629,13 +634,19 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
     mfma_step(K);                                             \
     __builtin_amdgcn_sched_barrier(0);                        \
     MDCN_PROF(3);                                             \
-    if (late) MDCN_BARRIER(kF2VmBar);                         \
+    if (late) {                                               \
+      MDCN_ROLE("late");                                      \
+      MDCN_BARRIER(kF2VmBar);                                 \
+    }                                                         \
     __builtin_amdgcn_sched_barrier(0);                        \
     MDCN_PROF(5);                                             \
     MDCN_F2_BLOCK(SI);                                        \
     __builtin_amdgcn_sched_barrier(0);                        \
     MDCN_PROF(4);                                             \
-    if (!late) MDCN_BARRIER(kF2VmBar);                        \
+    if (!late) {                                              \
+      MDCN_ROLE("early");                                     \
+      MDCN_BARRIER(kF2VmBar);                                 \
+    }                                                         \
     __builtin_amdgcn_sched_barrier(0);                        \
     MDCN_PROF(5);                                             \
   } while (0)

@@ -372,3 +372,29 @@ def test_asm_check_flags_registers_touched_while_an_inline_load_is_in_flight():
     assert asm_check.inflight_violations(head + ds + dwait + mfma + '\ts_endpgm\n') == []
     assert len(asm_check.inflight_violations(head + ds + mfma + dwait + '\ts_endpgm\n')) == 1
     assert len(asm_check.inflight_violations(head + ds + '\ts_waitcnt vmcnt(0)\n' + mfma + '\ts_endpgm\n')) == 1
+
+
+def test_asm_check_follows_role_markers():
+    """A kernel that branches on a wave's role in two places: without markers the scan also
+    follows the paths that take one role's side first and the other's later, and reports them;
+    with `; mdcn-role` markers in the role-specific blocks those paths are dropped."""
+    from mmcv_amd import asm_check
+    load = lambda r: f'\t;;#ASMSTART\n\tglobal_load_dwordx4 v[{r}:{r + 3}], v[8:9], off\n\t;;#ASMEND\n'
+    wait = lambda r: f'\t;;#ASMSTART\n\ts_waitcnt vmcnt(4) ; v[{r}:{r + 3}]\n\t;;#ASMEND\n'
+    mark = lambda name: f'\t;;#ASMSTART\n\t; mdcn-role {name}\n\t;;#ASMEND\n'
+    def kernel(marked):
+        m = mark if marked else (lambda name: '')
+        return ('kern:\n'
+                '\ts_cbranch_scc1 .LBB0_2\n'                       # role test 1
+                + m('early') + load(20) + '\ts_branch .LBB0_3\n'
+                '.LBB0_2:\n' + m('late') + load(30) +
+                '.LBB0_3:\n'
+                '\ts_cbranch_scc1 .LBB0_5\n'                       # role test 2 (same flag)
+                + m('early') + wait(20) + '\tv_mov_b32_e32 v1, v20\n' + load(30) + wait(30) + '\ts_branch .LBB0_6\n'
+                '.LBB0_5:\n' + m('late') + wait(30) + '\tv_mov_b32_e32 v1, v30\n' + load(20) + wait(20) +
+                '.LBB0_6:\n\ts_endpgm\n')
+    assert len(asm_check.inflight_violations(kernel(False))) == 2   # the two mixed paths reissue a locked set
+    assert asm_check.inflight_violations(kernel(True)) == []
+    # a real violation on a consistent path is still found
+    bad = kernel(True).replace(wait(20) + '\tv_mov_b32_e32 v1, v20\n', '\tv_mov_b32_e32 v1, v20\n' + wait(20))
+    assert len(asm_check.inflight_violations(bad)) == 1
