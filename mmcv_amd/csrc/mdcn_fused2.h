@@ -484,16 +484,40 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
   };
   static_assert(kF2WD == 4 || kF2WD == 2, "issue_weights spells out the copies");
 
+  // The blend weights of the blend cursor's step for the lane's two pixels are read from the
+  // table ahead of the block that needs them -- right behind the last MFMA of the MFMA phase in
+  // front of it, which for the late waves is a barrier away -- so that the block does not start
+  // with an LDS round trip (256-channel tiles: 1.5 % off the kernel; with 128-channel tiles, whose
+  // MFMA phase is half as long, it costs as much and is left out).
+  constexpr bool kF2TwAhead = CT == 256;
+  u32x2 tw_pf[2];
+  const uint32_t lds_tw = (uint32_t)(uintptr_t)(lptr_t)(&tws[0][0]) + (uint32_t)pl * 8u;
+  auto prefetch_tw = [&]() {
+    if constexpr (!kF2TwAhead) return;
+    const uint32_t a_ = lds_tw + (uint32_t)(((b_t & 1) ? TBL : 0) + b_tap * PT) * 8u;
+    asm volatile("ds_read_b64 %0, %1" : "=v"(tw_pf[0]) : "v"(a_));
+    asm volatile("ds_read_b64 %0, %1 offset:64" : "=v"(tw_pf[1]) : "v"(a_));
+  };
+
   // One produce block: the weight copies of the step after the blend cursor's,
   // the blend of the cursor's step (gather set SI) into its sample tile, the
   // gather of three steps ahead into the set.
 #define MDCN_F2_BLOCK(SI)                                                               \
   do {                                                                                  \
+    if constexpr (kF2TwAhead)                                                           \
+      asm volatile("s_waitcnt lgkmcnt(0) ; %0 %1" : "+v"(tw_pf[0]), "+v"(tw_pf[1]));    \
     if (b_t < T) {                                                                      \
       issue_weights(true);                                                              \
       next_addresses();                                                                 \
-      const uint2 *tw_ = &tws[b_t & 1][b_tap * PT + pl];                                \
-      const uint2 tw0_ = tw_[0], tw1_ = tw_[8];                                         \
+      uint2 tw0_, tw1_;                                                                 \
+      if constexpr (kF2TwAhead) {                                                       \
+        tw0_ = make_uint2(tw_pf[0].x, tw_pf[0].y);                                      \
+        tw1_ = make_uint2(tw_pf[1].x, tw_pf[1].y);                                      \
+      } else {                                                                          \
+        const uint2 *tw_ = &tws[b_t & 1][b_tap * PT + pl];                              \
+        tw0_ = tw_[0];                                                                  \
+        tw1_ = tw_[8];                                                                  \
+      }                                                                                 \
       const uint32_t xo_ = (b_s & 1) ? kXTile : 0u;                                     \
       {                                                                                 \
         const typename BL::Wt w_ = BL::prep(tw0_, q);                                   \
@@ -610,6 +634,7 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
     MDCN_F2_GATHER(1);
     issue_weights(false);
     MDCN_F2_GATHER(2);
+    prefetch_tw();
     MDCN_F2_BLOCK(0);
   } else {
     MDCN_ROLE("late");
@@ -618,7 +643,9 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
     MDCN_F2_GATHER(0);
     issue_weights(false);
     MDCN_F2_GATHER(1);
+    prefetch_tw();
     MDCN_F2_BLOCK(2);
+    prefetch_tw();
     MDCN_F2_BLOCK(0);
   }
   static_assert(kF2Sets == 3, "the prologue spells out three sets");
@@ -632,6 +659,7 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
 #define MDCN_F2_STEP(K, SI)                                   \
   do {                                                        \
     mfma_step(K);                                             \
+    prefetch_tw();                                            \
     __builtin_amdgcn_sched_barrier(0);                        \
     MDCN_PROF(3);                                             \
     if (late) {                                               \
