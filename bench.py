@@ -38,8 +38,8 @@ PEAK_TFLOPS = {'bf16': 2500.0, 'f16': 2500.0, 'f32': 157.3}
 HBM_PEAK_GBS = 8000.0
 # (workload, dominant kernel) -> (HBM bytes per launch from rocprofv3 counters, the profile they are in)
 TRAFFIC = {
-    ('cfg4', 'fused2_kernel<bf16>'): (421.9e6, 'profiles/fused2_kernel_bf16_cfg4.md (FETCH_SIZE 130 528.9 KiB x 2.00 '
-                                               '+ WRITE_SIZE 150 913.3 KiB x 1.00)'),
+    ('cfg4', 'fused2_kernel<bf16>'): (422.0e6, 'profiles/fused2_kernel_bf16_cfg4.md (FETCH_SIZE 130 554.5 KiB x 2.00 '
+                                               '+ WRITE_SIZE 150 981.9 KiB x 1.00)'),
 }
 
 WORKLOADS = {
