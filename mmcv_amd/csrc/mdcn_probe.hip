@@ -89,16 +89,16 @@ extern "C" int mdcn_mfma_probe(int dtype, int waves_per_simd, int zero_data, voi
                          (float *)scratch, n, zero_data);
   };
   launch(2000);  // warm up (clocks)
-  hipEventRecord(e0, st);
-  launch(iters);
-  hipEventRecord(e1, st);
   int rc = 0;
+  if (hipEventRecord(e0, st) != hipSuccess) rc = -7;
+  launch(iters);
+  if (hipEventRecord(e1, st) != hipSuccess) rc = -7;
   float ms = 0.0f;
   if (hipEventSynchronize(e1) != hipSuccess || hipEventElapsedTime(&ms, e0, e1) != hipSuccess ||
       hipGetLastError() != hipSuccess || ms <= 0.0f)
     rc = -7;
-  hipEventDestroy(e0);
-  hipEventDestroy(e1);
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
   if (rc == 0) *tflops = (float)((double)blocks * 4 * iters * 8 * 32768.0 / ms / 1e9);
   return rc;
 }
