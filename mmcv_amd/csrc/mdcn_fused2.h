@@ -5,10 +5,10 @@
 // Eight wavefronts, all alike.  Per K step (128 bytes of channels of one tap)
 // every wave
 //   * "produces" 16 of the tile's 128 pixels: waits for the gather it issued
-//     three steps earlier (4 corners x 16 bytes of each of two pixels per lane,
+//     two steps earlier (4 corners x 16 bytes of each of two pixels per lane,
 //     held in registers: eight lanes read a pixel's whole 128-byte row),
 //     blends the corners into 2 x 16 bytes of the sample tile, writes them to
-//     LDS and refills the registers with the gather of three steps ahead;
+//     LDS and refills the registers with the gather of two steps ahead;
 //   * issues its share (4 x 1 KiB) of the direct-to-LDS copy of the weight tile
 //     of the next step;
 //   * "consumes": 16 MFMAs (32x32x16) on its 64 pixel x 64 channel part of the
@@ -30,7 +30,7 @@
 // v_permlane32_swap, after which a lane holds 16 bytes of one channel's row).
 //
 // All vector-memory traffic of the K loop is issued from inline assembly and
-// waited for with explicit counts: a wave has 3 x 8 gather loads and the weight
+// waited for with explicit counts: a wave has 2 x 8 gather loads and the weight
 // copies of up to three steps in flight, and the compiler's own bookkeeping
 // would drain them at every use.  Per wave and K step the order of issue is
 // fixed: kWD weight copies, then 8 gather loads (two groups of four, each group
@@ -56,7 +56,13 @@ constexpr int kF2Threads = 512;
 constexpr int kF2CT = 256;             // output channels per tile at most (the template parameter CT: 256 or 128)
 constexpr int kF2Slots = 3;            // ring of weight tiles
 constexpr int kF2GL = 8;               // gather loads per wave and K step
-constexpr int kF2Sets = 3;             // gather register sets: a gather is in flight for kF2Sets steps
+// Gather register sets: a gather is in flight for kF2Sets steps.  Two are enough -- the loaded latency of a
+// gather is well under one step, and three sets measure the same on every shape tried (+-0.5 %) --
+// and leave the 256-channel kernel at 224 instead of 256 vector registers.
+#ifndef MDCN_F2_SETS
+#define MDCN_F2_SETS 2
+#endif
+constexpr int kF2Sets = MDCN_F2_SETS;
 constexpr int kF2Unroll = 6;           // steps per round of the K loop: sets, sample tiles and ring slots are static
 static_assert(kF2Unroll % kF2Sets == 0 && kF2Unroll % 2 == 0 && kF2Unroll % kF2Slots == 0, "static indices");
 
@@ -501,7 +507,7 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
 
   // One produce block: the weight copies of the step after the blend cursor's,
   // the blend of the cursor's step (gather set SI) into its sample tile, the
-  // gather of three steps ahead into the set.
+  // gather of kF2Sets steps ahead into the set.
 #define MDCN_F2_BLOCK(SI)                                                               \
   do {                                                                                  \
     if constexpr (kF2TwAhead)                                                           \
@@ -603,12 +609,12 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
 #endif
 
   // ---- start of the stream: first table, first gathers.  A wave keeps step j of
-  // the stream in set j % 3; the late waves, which run one block ahead, in set
-  // (j + 2) % 3, so that both kinds use the same set at the same place of the K
-  // loop.  The issue order gather, copies, gather, copies, gather is the K
-  // loop's, which keeps the counts of the waits valid from the first block on
-  // (the second group of copies is issued again by the first block: same data,
-  // same slot).
+  // the stream in set j % kF2Sets; the late waves, which run one block ahead, in set
+  // (j - 1) % kF2Sets, so that both kinds use the same set at the same place of the K
+  // loop.  The issue order gather, copies, gather (..., copies, gather with three
+  // sets) is the K loop's, which keeps the counts of the waits valid from the first
+  // block on (with three sets the second group of copies is issued again by the
+  // first block: same data, same slot).
   // bias of this lane's output channels, fetched together with a tile's table (the
   // wait that ends the table's loads covers it, so the epilogue never waits on memory)
   float bv[MB], bv_next[MB];
@@ -627,35 +633,56 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
   build_table(0);
   MDCN_BARRIER_LDS();  // table visible
   __builtin_amdgcn_sched_barrier(0);
-  if (!late) {
-    MDCN_ROLE("early");
-    MDCN_F2_GATHER(0);
-    issue_weights(true);
-    MDCN_F2_GATHER(1);
-    issue_weights(false);
-    MDCN_F2_GATHER(2);
-    prefetch_tw();
-    MDCN_F2_BLOCK(0);
+  if constexpr (kF2Sets == 3) {
+    if (!late) {
+      MDCN_ROLE("early");
+      MDCN_F2_GATHER(0);
+      issue_weights(true);
+      MDCN_F2_GATHER(1);
+      issue_weights(false);
+      MDCN_F2_GATHER(2 % kF2Sets);
+      prefetch_tw();
+      MDCN_F2_BLOCK(0);
+    } else {
+      MDCN_ROLE("late");
+      MDCN_F2_GATHER(2 % kF2Sets);
+      issue_weights(true);
+      MDCN_F2_GATHER(0);
+      issue_weights(false);
+      MDCN_F2_GATHER(1);
+      prefetch_tw();
+      MDCN_F2_BLOCK(2 % kF2Sets);
+      prefetch_tw();
+      MDCN_F2_BLOCK(0);
+    }
   } else {
-    MDCN_ROLE("late");
-    MDCN_F2_GATHER(2);
-    issue_weights(true);
-    MDCN_F2_GATHER(0);
-    issue_weights(false);
-    MDCN_F2_GATHER(1);
-    prefetch_tw();
-    MDCN_F2_BLOCK(2);
-    prefetch_tw();
-    MDCN_F2_BLOCK(0);
+    // two sets: step j in set j % 2 (late waves: (j + 1) % 2)
+    if (!late) {
+      MDCN_ROLE("early");
+      MDCN_F2_GATHER(0);
+      issue_weights(true);
+      MDCN_F2_GATHER(1);
+      prefetch_tw();
+      MDCN_F2_BLOCK(0);
+    } else {
+      MDCN_ROLE("late");
+      MDCN_F2_GATHER(1);
+      issue_weights(true);
+      MDCN_F2_GATHER(0);
+      prefetch_tw();
+      MDCN_F2_BLOCK(1);
+      prefetch_tw();
+      MDCN_F2_BLOCK(0);
+    }
   }
-  static_assert(kF2Sets == 3, "the prologue spells out three sets");
+  static_assert(kF2Sets == 3 || kF2Sets == 2, "the prologue spells out the sets");
   MDCN_PROF(2);
   MDCN_BARRIER(kF2VmBar);  // X[0] and W[0] complete
   __builtin_amdgcn_sched_barrier(0);
   MDCN_PROF(1);
 
   // ---- K loop of a tile: kF2Unroll steps per round; step k runs the produce
-  // block one (late waves: two) steps ahead on set (k + 1) % 3
+  // block one (late waves: two) steps ahead on set (k + 1) % kF2Sets
 #define MDCN_F2_STEP(K, SI)                                   \
   do {                                                        \
     mfma_step(K);                                             \
@@ -698,12 +725,12 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
         __builtin_amdgcn_sched_barrier(0);
         MDCN_PROF(0);
       }
-      MDCN_F2_STEP(k + 0, 1);
-      MDCN_F2_STEP(k + 1, 2);
-      MDCN_F2_STEP(k + 2, 0);
-      MDCN_F2_STEP(k + 3, 1);
-      MDCN_F2_STEP(k + 4, 2);
-      MDCN_F2_STEP(k + 5, 0);
+      MDCN_F2_STEP(k + 0, 1 % kF2Sets);
+      MDCN_F2_STEP(k + 1, 2 % kF2Sets);
+      MDCN_F2_STEP(k + 2, 3 % kF2Sets);
+      MDCN_F2_STEP(k + 3, 4 % kF2Sets);
+      MDCN_F2_STEP(k + 4, 5 % kF2Sets);
+      MDCN_F2_STEP(k + 5, 6 % kF2Sets);
     }
 
     // ---- a part of a tile: the parts meet in memory.  Every part stores its
@@ -878,7 +905,7 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
     MDCN_PROF(6);
   }
   // copies issued past the last step must have landed before the workgroup gives up its LDS
-  MDCN_VMWAIT4(0, gs[0][0][0], gs[0][1][0], gs[1][0][0], gs[2][1][0]);
+  MDCN_VMWAIT4(0, gs[0][0][0], gs[0][1][0], gs[1][0][0], gs[kF2Sets - 1][1][0]);
 #undef MDCN_F2_STEP
 #undef MDCN_F2_IS_PART
 #undef MDCN_F2_UNIT_KB
