@@ -45,10 +45,17 @@ enum mdcn_path {
   MDCN_PATH_AUTO = 0,   /* fused MFMA kernel when the shape allows, else direct */
   MDCN_PATH_FUSED = 1,  /* fused implicit-GEMM MFMA kernel; error if not eligible */
   MDCN_PATH_DIRECT = 2, /* one thread per output element; any shape */
-  MDCN_PATH_FUSED_SPLIT = 3 /* forward only: as MDCN_PATH_FUSED, but always the fused kernel with specialised
+  MDCN_PATH_FUSED_SPLIT = 3, /* forward only: as MDCN_PATH_FUSED, but always the fused kernel with specialised
                                producer / consumer wavefronts (what fp32 tensors, several deformable groups and
                                tiles narrower than 256 channels run anyway), never the eight-wave streaming
                                kernel that 16-bit 256-channel tiles get by default; for comparisons and tests */
+  MDCN_PATH_FUSED_WIDE = 4, /* forward only: as MDCN_PATH_FUSED, and every whole tile of 256 pixels goes to the
+                               kernel with 256-pixel tiles where the shape has one (16-bit tensors, one
+                               deformable group, at most 9 taps, 129..256 output channels per group tile, an even
+                               number of K steps), however unevenly that fills the chip; MDCN_PATH_FUSED and
+                               MDCN_PATH_AUTO give that kernel whole rounds of tiles only and the rest of the
+                               pixels to the 128-pixel kernel.  Error if the shape has no such kernel. */
+  MDCN_PATH_FUSED_NARROW = 5 /* forward only: as MDCN_PATH_FUSED, never the 256-pixel kernel */
 };
 
 enum mdcn_status {

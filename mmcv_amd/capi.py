@@ -10,7 +10,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, 'lib', 'libmdcn_hip.so')
 
 MDCN_F32, MDCN_F16, MDCN_BF16, MDCN_F64 = 0, 1, 2, 3
-PATH_AUTO, PATH_FUSED, PATH_DIRECT, PATH_FUSED_SPLIT = 0, 1, 2, 3
+PATH_AUTO, PATH_FUSED, PATH_DIRECT, PATH_FUSED_SPLIT, PATH_FUSED_WIDE, PATH_FUSED_NARROW = 0, 1, 2, 3, 4, 5
 MDCN_OK = 0
 NOALLOC_SCRATCH_BYTES = 64 << 20
 

@@ -585,7 +585,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("dilation_h"), py::arg("dilation_w"), py::arg("group"),
         py::arg("deformable_group"), py::arg("with_bias"));
   m.def("set_path", [](int path) {
-          TORCH_CHECK(path >= MDCN_PATH_AUTO && path <= MDCN_PATH_FUSED_SPLIT,
+          TORCH_CHECK(path >= MDCN_PATH_AUTO && path <= MDCN_PATH_FUSED_NARROW,
                       "path must be 0 (auto), 1 (fused), 2 (direct) or 3 (fused, specialised-wave kernel only)");
           g_path.store(path);
         }, "choose the device path of forward and backward: 0 auto, 1 fused / matrix-core kernels, 2 direct kernels, "

@@ -18,6 +18,7 @@
 #include "mdcn_backward_gemm.h"
 #include "mdcn_fused.h"
 #include "mdcn_fused2.h"
+#include "mdcn_fused3.h"
 #include "mdcn_oconv.h"
 #include "mdcn_prepass.h"
 
@@ -167,7 +168,13 @@ struct PackExtra {
   void *raw;
 };
 
-// 16-bit tensors, 256-channel tiles, one deformable group, enough K steps: the eight-wave kernel
+inline bool forced_fused(int path) {
+  return path == MDCN_PATH_FUSED || path == MDCN_PATH_FUSED_SPLIT || path == MDCN_PATH_FUSED_WIDE ||
+         path == MDCN_PATH_FUSED_NARROW;
+}
+
+// 16-bit tensors, 256- or 128-channel tiles, one deformable group, enough K steps: the eight-wave
+// kernels (mdcn_fused2.h; mdcn_fused3.h beside it where wide_ok() says so)
 bool uses_fused2(const mdcn_params *p, const Geom &g, const Plan &pl) {
   if ((pl.CT != 256 && pl.CT != 128) || g.taps > kTapsSmall || elem_size(p->dtype) != 2 || g.DG != 1 ||
       p->path == MDCN_PATH_FUSED_SPLIT)
@@ -176,9 +183,56 @@ bool uses_fused2(const mdcn_params *p, const Geom &g, const Plan &pl) {
   return nk_pad >= kF2MinSteps;
 }
 
+// ... and the kernel with 256-pixel tiles for whole tiles of such a call: bordered input copy, an even
+// number of K steps, output planes of whole 16-byte runs (the caller checks the pointer's alignment)
+bool wide_ok(const mdcn_params *p, const Geom &g, const Plan &pl) {
+  if (!pl.fused || !uses_fused2(p, g, pl) || pl.CT != 256 || p->input_nhwc || p->path == MDCN_PATH_FUSED_NARROW)
+    return false;
+  const int nk = pl.slabs * g.taps;
+  const long plane_out = (long)g.Ho * g.Wo;
+  return nk >= kF3MinSteps && nk % 2 == 0 && plane_out % 8 == 0 && plane_out >= 64;
+}
+
+// Rounds of the 128-pixel kernel's schedule for `tiles` tiles of nk K steps, in tile times (its last round's
+// tiles are cut along K when that is allowed).
+double narrow_rounds(long tiles, int nk, bool may_cut) {
+  if (tiles <= 0) return 0.0;
+  const int stride = std::max(1, num_cus() / 8);
+  const long chunk = (tiles + 7) / 8;
+  const long full = chunk / stride, rest = chunk % stride;
+  if (rest == 0) return (double)full;
+  const long steps6 = (nk + kF2Unroll - 1) / kF2Unroll;
+  long parts = 1;
+  if (may_cut) parts = std::max<long>(1, std::min<long>(std::min<long>(stride / rest, kCutMax), steps6));
+  return (double)full + 1.0 / (double)parts;
+}
+
+// How many of a launch's pixel tiles of 256 go to the wide kernel: all of them (`all`), or whole rounds of
+// its one-workgroup-per-CU grid when that and the 128-pixel kernel on the rest come out shorter than the
+// 128-pixel kernel alone.  kWideTileCost: time of a 256-pixel tile in units of a 128-pixel one (measured).
+constexpr double kWideTileCost = 1.65;
+long wide_tiles(long total_px, int n_ctiles_groups, int nk, bool may_cut, bool all) {
+  const long full = total_px / kF3PT;
+  if (all || full == 0) return full;
+  const long grid = std::max(8, num_cus() / 8 * 8);
+  auto cost = [&](long n3) {
+    const long wg_tiles = (n3 * n_ctiles_groups + grid - 1) / grid;  // tiles of the busiest workgroup
+    const long px2 = total_px - n3 * kF3PT;
+    const long tiles2 = (px2 + kPT - 1) / kPT * n_ctiles_groups;
+    return wg_tiles * kWideTileCost + narrow_rounds(tiles2, nk, may_cut) + ((n3 && tiles2) ? 0.05 : 0.0);
+  };
+  const long rounds = full * n_ctiles_groups / grid;
+  const long whole = rounds * grid / n_ctiles_groups;  // pixel tiles of the whole rounds
+  long best = 0;
+  double best_cost = cost(0);
+  for (long n3 : {whole, full})
+    if (n3 > 0 && cost(n3) < best_cost) best = n3, best_cost = cost(n3);
+  return best;
+}
+
 int make_plan(const mdcn_params *p, const Geom &g, Plan *pl) {
   const bool ok = fused_ok(p, g);
-  if ((p->path == MDCN_PATH_FUSED || p->path == MDCN_PATH_FUSED_SPLIT) && !ok) return MDCN_ERR_PATH;
+  if (forced_fused(p->path) && !ok) return MDCN_ERR_PATH;
   if (p->input_nhwc && (!ok || p->path == MDCN_PATH_DIRECT)) return MDCN_ERR_PATH;  // in-place reads: fused kernel only
   pl->fused = ok && p->path != MDCN_PATH_DIRECT;
   pl->CT = pl->KC = pl->n_ctiles = pl->slabs = pl->n_chunk = 0;
@@ -213,6 +267,7 @@ int make_plan(const mdcn_params *p, const Geom &g, Plan *pl) {
     pl->cut_wgs = num_cus() / 8 * 8;
     pl->cut_bytes = align_up((size_t)pl->cut_wgs * kPT * kF2CT * 4) + align_up((size_t)pl->cut_wgs * 4);
   }
+  if (p->path == MDCN_PATH_FUSED_WIDE && !wide_ok(p, g, *pl)) return MDCN_ERR_PATH;
   return MDCN_OK;
 }
 
@@ -233,7 +288,7 @@ int make_pack_plan(const mdcn_pack_params *pp, const Geom &g, Plan *pl) {
   if (pp->offset_weight) {
     if (pl->fused) {
       if (pl->CO_pad > 128) {  // accumulator blocks of the conv_offset kernel
-        if (p->path == MDCN_PATH_FUSED || p->path == MDCN_PATH_FUSED_SPLIT) return MDCN_ERR_PATH;
+        if (forced_fused(p->path)) return MDCN_ERR_PATH;
         pl->fused = false;
         pl->xt_bytes = pl->wp_bytes = pl->cut_bytes = 0;
         pl->cut_wgs = 0;
@@ -311,12 +366,20 @@ hipError_t launch_fused2(const FusedArgs &fa, bool unbordered, hipStream_t st) {
   return hipGetLastError();
 }
 
+// 16-bit tensors, 256-channel tiles, whole tiles of 256 pixels: mdcn_fused3.h
+template <typename E>
+hipError_t launch_fused3(const FusedArgs &fa, hipStream_t st) {
+  const int total_wg = fa.n_ptiles * fa.n_ctiles * fa.g.G;
+  const int per_xcd = std::max(1, std::min((total_wg + 7) / 8, num_cus() / 8));
+  hipLaunchKernelGGL((fused3_kernel<E, 256>), dim3(per_xcd * 8), dim3(kF3Threads), 0, st, fa);
+  return hipGetLastError();
+}
+
 template <typename E, int CT>
-hipError_t launch_fused_tm(const FusedArgs &fa, bool ub, bool split, hipStream_t st) {
+hipError_t launch_fused_tm(const FusedArgs &fa, bool ub, bool eight_wave, hipStream_t st) {
   const bool small = fa.g.taps <= kTapsSmall;
   if constexpr (sizeof(E) == 2 && (CT == 256 || CT == 128)) {
-    const int nk_pad = (fa.slabs * fa.g.taps + kF2Unroll - 1) / kF2Unroll * kF2Unroll;
-    if (!split && small && fa.g.DG == 1 && nk_pad >= kF2MinSteps) return launch_fused2<E, CT>(fa, ub, st);
+    if (eight_wave) return launch_fused2<E, CT>(fa, ub, st);
   }
   if constexpr (CT == 256) {  // (pick_ct never pairs the 256-wide tile with the large table)
     return fa.g.DG > 1 ? launch_fused_ct<E, CT, kTapsSmall, true>(fa, ub, st)
@@ -331,11 +394,11 @@ hipError_t launch_fused_tm(const FusedArgs &fa, bool ub, bool split, hipStream_t
 }
 
 template <typename E>
-hipError_t launch_fused(const FusedArgs &fa, int CT, bool ub, bool split, hipStream_t st) {
+hipError_t launch_fused(const FusedArgs &fa, int CT, bool ub, bool eight_wave, hipStream_t st) {
   switch (CT) {
-    case 64: return launch_fused_tm<E, 64>(fa, ub, split, st);
-    case 128: return launch_fused_tm<E, 128>(fa, ub, split, st);
-    default: return launch_fused_tm<E, 256>(fa, ub, split, st);
+    case 64: return launch_fused_tm<E, 64>(fa, ub, eight_wave, st);
+    case 128: return launch_fused_tm<E, 128>(fa, ub, eight_wave, st);
+    default: return launch_fused_tm<E, 256>(fa, ub, eight_wave, st);
   }
 }
 
@@ -557,8 +620,26 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
       fa.slabs_total = g.Cin / pl.KC;
       fa.plane_px = g.Hp * g.Wp;
       fa.out_vec_ok = (plane_out % (long)(16 / es) == 0) && (((uintptr_t)fa.out % 16) == 0);
+      fa.px0 = 0;
       tic();
-      if (launch_fused<E>(fa, pl.CT, nhwc, p->path == MDCN_PATH_FUSED_SPLIT, st) != hipSuccess) rc = MDCN_ERR_LAUNCH;
+      const bool eight_wave = uses_fused2(p, g, pl);
+      bool rest = true;
+      if constexpr (sizeof(E) == 2) {
+        if (wide_ok(p, g, pl) && fa.out_vec_ok) {
+          // whole tiles of 256 pixels to the wide kernel, what is left to the 128-pixel one
+          const long n3 = wide_tiles(fa.total_px, pl.n_ctiles * g.G, pl.slabs * g.taps, pl.cut_bytes != 0,
+                                     p->path == MDCN_PATH_FUSED_WIDE);
+          if (n3 > 0) {
+            FusedArgs fw = fa;
+            fw.n_ptiles = (int)n3;
+            if (launch_fused3<E>(fw, st) != hipSuccess) rc = MDCN_ERR_LAUNCH;
+            fa.px0 = (int)(n3 * kF3PT);
+            fa.n_ptiles = (int)((fa.total_px - fa.px0 + kPT - 1) / kPT);
+            rest = fa.n_ptiles > 0;
+          }
+        }
+      }
+      if (rest && launch_fused<E>(fa, pl.CT, nhwc, eight_wave, st) != hipSuccess) rc = MDCN_ERR_LAUNCH;
       toc(2);
     }
   }
@@ -690,7 +771,7 @@ void make_bwd_plan(const mdcn_bwd_params *bp, const Geom &g, BwdPlan *pl) {
   pl->P_pad = 0;
   pl->R = pl->sR = -1;
   pl->WH = pl->WW = pl->sWH = pl->sWW = 0;
-  const int path = bp->conv.path == MDCN_PATH_FUSED_SPLIT ? MDCN_PATH_FUSED : bp->conv.path;
+  const int path = forced_fused(bp->conv.path) ? MDCN_PATH_FUSED : bp->conv.path;
   if (path == MDCN_PATH_DIRECT || g.taps > kBwdTapsMax || f64) return;
   const bool forced = path == MDCN_PATH_FUSED;
   const size_t plane_out = (size_t)g.Ho * g.Wo;
@@ -1082,8 +1163,8 @@ int check_bwd(const mdcn_bwd_params *bp, Geom *g, bool need_ptrs) {
   if (data != (bp->grad_offset != nullptr)) return MDCN_ERR_NULL;
   if (p->mask ? (data != (bp->grad_mask != nullptr)) : (bp->grad_mask != nullptr)) return MDCN_ERR_NULL;
   if ((uint64_t)g->N * g->DG * g->taps > 0x7fffffffull) return MDCN_ERR_TOO_LARGE;
-  if (p->dtype == MDCN_F64 && (p->path == MDCN_PATH_FUSED || p->path == MDCN_PATH_FUSED_SPLIT)) return MDCN_ERR_PATH;
-  if (p->path == MDCN_PATH_FUSED || p->path == MDCN_PATH_FUSED_SPLIT) {  // asked for the tiled kernels: the shape must allow them
+  if (p->dtype == MDCN_F64 && forced_fused(p->path)) return MDCN_ERR_PATH;
+  if (forced_fused(p->path)) {  // asked for the tiled kernels: the shape must allow them
     BwdPlan pl;
     make_bwd_plan(bp, *g, &pl);
     if ((data && !pl.tiled && !pl.gemm) || (!data && bp->grad_weight && !pl.wgemm)) return MDCN_ERR_PATH;

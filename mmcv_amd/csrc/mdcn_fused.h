@@ -79,6 +79,9 @@ struct FusedArgs {
   int cut_max;
   void *cut_part;
   void *cut_cnt;
+  // fused2_kernel only: first pixel of its tiles (a multiple of 256; the pixels in front of it belong to
+  // fused3_kernel, which is launched beside it); n_ptiles counts the tiles from there on
+  int px0;
 };
 
 typedef __attribute__((address_space(3))) void *lptr_t;

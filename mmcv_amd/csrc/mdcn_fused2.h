@@ -326,7 +326,7 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
     ctile = L % a.n_ctiles;
     L /= a.n_ctiles;
     grp = L % g.G;
-    p0 = (L / g.G) * PT;
+    p0 = a.px0 + (L / g.G) * PT;
   };
   auto weights_of = [&](int t) __attribute__((always_inline)) {
     int ctile, grp, p0;

@@ -1,0 +1,593 @@
+// Fused DCNv2 forward for gfx950, 16-bit tensors, tiles of 256 pixels x CT (256 or
+// 128) output channels, one deformable group, at most 9 taps, bordered input copy:
+// the implicit GEMM of mdcn_fused.h / mdcn_fused2.h with a tile twice as tall.
+//
+// Why another tile.  Per K step (128 bytes of channels of one tap) a tile of PT
+// pixels x CT channels pulls 4 * PT corner rows and CT weight rows of 128 bytes
+// through the compute unit's vector-memory path for PT * CT * 64 multiply-adds,
+// and that path (64 bytes per clock) is what the 128-pixel kernels are bound by.
+// 256 x 256 moves 160 KiB per 2 048 MFMA clocks where 128 x 256 moves 96 KiB per
+// 1 024: one sixth fewer bytes per FLOP, half the weight-tile copies, a quarter
+// fewer fragment reads, half the barriers.
+//
+// Eight wavefronts.  A wave owns 64 pixels x CT / 2 channels of the tile (128
+// accumulator registers per lane for CT = 256).  Per K step every wave
+//   * "produces" 32 of the tile's pixels: waits for the gather it issued one step
+//     earlier (4 corners x 16 bytes of four pixels per lane: one load instruction
+//     of the wave reads the whole 128-byte rows of 8 pixels), blends the corners
+//     pixel by pixel into the sample tile in LDS and reissues each pixel's four
+//     loads for the next step right behind its blend -- one register set, every
+//     load a whole step in flight;
+//   * "consumes": 8 * CT / 64 MFMAs (32x32x16), fragments read from LDS three
+//     pairs of MFMAs ahead.
+// The two waves of a SIMD do the halves in opposite order between two barriers:
+// waves 0-3 ("early") run their MFMAs first and produce afterwards, waves 4-7
+// ("late") produce first.  The late waves also issue the whole direct-to-LDS copy
+// of the next step's weight tile, right behind the barrier: the ring holds two
+// tiles (LDS: 2 x 32 KiB samples + 2 x 32 KiB weights + the 27 KiB table), so a
+// slot is free only once every wave has passed the barrier that ends its step,
+// and the early waves' MFMA phase, which comes first, is kept free of vector-memory
+// instructions.  One barrier per step.
+//
+// Tile after tile: the (pixel, tap) table exists once, so its next edition is
+// built when the last blend of a tile has read it -- offsets and mask are loaded
+// before the last step's MFMAs and turned into table entries behind them -- and
+// the first gathers of the next tile fly while the accumulators are stored.
+// A tile's K range is never cut here: the host gives this kernel whole rounds of
+// tiles (every workgroup the same number) and the rest of the pixels to the
+// 128-pixel kernel of mdcn_fused2.h.
+//
+// All vector-memory traffic of the K loop is issued from inline assembly and
+// waited for with explicit counts (see mdcn_fused2.h for why); per wave and step
+// the order of issue is fixed -- late waves: WD weight copies; then, both kinds,
+// four groups of four gather loads -- so the number of younger operations at
+// every wait is a constant.
+#pragma once
+
+#include "mdcn_fused2.h"
+
+namespace mdcn {
+
+constexpr int kF3PT = 256;             // pixels per tile
+constexpr int kF3Threads = 512;
+constexpr int kF3Taps = kTapsSmall;    // table capacity (kh * kw)
+constexpr int kF3MinSteps = 4;         // K steps per tile the pipeline needs (and an even number of them)
+constexpr size_t fused3_lds_bytes(int CT) {
+  return (size_t)2 * kF3PT * kRowB + (size_t)2 * CT * kRowB + (size_t)kF3PT * kF3Taps * 12;
+}
+
+// four corners of one pixel: 16 bytes per lane each, from `base` / `base_row`
+// (scalar pointers to the copy and to its next pixel row) + 32-bit byte offset;
+// the right-hand corners are the next 128 bytes.  (s_nop: the compiler may have
+// reloaded the scalar operands with a vector instruction right in front of the
+// statement, and a vector-memory instruction must not read such a register within
+// the next five issue slots.)
+#if MDCN_F2_ABLATE & 1
+#define MDCN_F3_GLOAD4(d, voff, base, base_row) \
+  asm volatile("" : "=&v"(d[0]), "=&v"(d[1]), "=&v"(d[2]), "=&v"(d[3]) : "v"(voff), "s"(base), "s"(base_row))
+#else
+#define MDCN_F3_GLOAD4(d, voff, base, base_row)                                  \
+  asm volatile("s_nop 4\n\t"                                                     \
+               "global_load_dwordx4 %0, %4, %5\n\t"                              \
+               "global_load_dwordx4 %1, %4, %5 offset:128\n\t"                   \
+               "global_load_dwordx4 %2, %4, %6\n\t"                              \
+               "global_load_dwordx4 %3, %4, %6 offset:128"                       \
+               : "=&v"(d[0]), "=&v"(d[1]), "=&v"(d[2]), "=&v"(d[3])              \
+               : "v"(voff), "s"(base), "s"(base_row))
+#endif
+
+template <int N>
+__device__ __forceinline__ void f3_vmwait4(u32x4 &a, u32x4 &b, u32x4 &c, u32x4 &d) {
+  asm volatile("s_waitcnt vmcnt(%4) ; %0 %1 %2 %3" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void f3_lgkmwait4(u32x4 &a, u32x4 &b, u32x4 &c, u32x4 &d) {
+  asm volatile("s_waitcnt lgkmcnt(%4) ; %0 %1 %2 %3" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void f3_lgkmwait3(u32x4 &a, u32x4 &b, u32x4 &c) {
+  asm volatile("s_waitcnt lgkmcnt(%3) ; %0 %1 %2" : "+v"(a), "+v"(b), "+v"(c) : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void f3_lgkmwait1(u32x4 &a) {
+  asm volatile("s_waitcnt lgkmcnt(%1) ; %0" : "+v"(a) : "n"(N));
+}
+
+// The whole kernel as one kind of wave runs it: the two kinds share no code path
+// between the first branch and the end (a register that an asm-issued load is still
+// writing must never meet another copy of itself at a join, where the compiler would
+// be free to move it).
+template <typename E, int CT, bool LATE>
+__device__ __forceinline__ void fused3_role(const FusedArgs &a, const uint32_t lds_x, const uint32_t lds_w,
+                                            uint32_t *tpix, uint2 *tws, const int wave) {
+  using TR = ElemTraits<E>;
+  using BL = Blend2<E>;
+  static_assert(sizeof(E) == 2, "16-bit element types");
+  static_assert(CT == 256 || CT == 128, "a wave owns 64 pixels x CT / 2 channels");
+  constexpr int PT = kF3PT;
+  constexpr int KC = TR::KC;
+  constexpr int TMAX = kF3Taps;
+  constexpr int TBL = PT * TMAX;               // entries of the table
+  constexpr int TPT = (TMAX + 1) / 2;          // table entries per lane and build
+  constexpr int NB = 2, MB = CT / 64;          // 32 x 32 accumulator blocks per wave: pixels x channels
+  constexpr int WCH = CT / 2;                  // output channels per wave
+  constexpr int WD = CT / 32;                  // 1 KiB weight copies per late wave and K step
+  constexpr int NG = 4 * MB;                   // MFMA groups (2 MFMAs each) per K step
+  // vector-memory operations younger than the loads of a pixel when it is blended:
+  // the pixels behind it of the same step and the ones before it of the next (12
+  // loads), for the late waves also the weight copies issued in between
+  constexpr int kVmBlend = LATE ? 12 + WD : 12;
+  // ... younger than the weight copies at the barrier that ends their step (late waves)
+  constexpr int kVmBar = 16;
+  constexpr uint32_t kXTile = PT * kRowB, kWTile = CT * kRowB;
+  static_assert(fused3_lds_bytes(CT) <= 160 * 1024, "LDS of one compute unit");
+
+  const Geom &g = a.g;
+  const int taps = g.taps;
+  const int nk = a.slabs * taps;               // even and >= kF3MinSteps (the host checks)
+  const int plane_out = g.Ho * g.Wo;
+  const int total_px = (int)a.total_px;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  // The code that runs once per tile (table, epilogue) takes the thread index through this: what it
+  // derives from it is then computed there, not once per kernel and kept in -- spilled -- registers
+  // across the K loop.
+  auto tile_tid = [&]() __attribute__((always_inline)) {
+    int v = tid;
+    asm volatile("" : "+v"(v));
+    return v;
+  };
+  // (likewise the divisors of that code: the reciprocals its divisions go through are computed on the
+  // vector ALU, and hoisted out of the tile loop they would each hold a vector register for good)
+  auto tile_s = [](int v) __attribute__((always_inline)) {
+    asm volatile("" : "+s"(v));
+    return v;
+  };
+
+  // ---- produce role: lane serves 16-byte chunk ck of pixels pl + 8 i, i = 0..3
+  const int q = lane & 3;            // row of the lane in its block of four (the matrix-pipe blend)
+  const int ck = lane & 7;
+  const int pl = wave * 32 + (lane >> 3);
+  // where the four chunks go in X[0] (rows 8 apart differ in bit 1 of the swizzle, rows 16 apart in none)
+  const uint32_t xwa = lds_x + (uint32_t)tile_chunk(pl, ck) * 16u;
+  const uint32_t xwb = lds_x + (uint32_t)tile_chunk(pl + 8, ck) * 16u;
+  const unsigned char *xt = uniform_ptr((const unsigned char *)a.xt);
+  const unsigned char *xt_row = uniform_ptr((const unsigned char *)a.xt + a.row_bytes);
+
+  // ---- consume role: 64 pixels x WCH channels
+  const int wave_p = wave & 3, wave_c = wave >> 2;
+  const int frow = lane & 31, fhalf = lane >> 5;
+  const uint32_t xa0 = (uint32_t)tile_chunk(wave_p * 64 + frow, fhalf) * 16u;   // K sub-step s: ^ (s << 5)
+  const uint32_t wa0 = (uint32_t)tile_chunk(wave_c * WCH + frow, fhalf) * 16u;
+
+  // weight copies (late waves): wave 4 + j copies the WD consecutive 1 KiB blocks (8
+  // rows each) from block j * WD on; lane i of a copy writes chunk i of the block and
+  // reads the source chunk the swizzle assigns to it (bits 1, 2 of the row come from
+  // the lane, bit 3 is the block's parity, which flips bit 1 of the chunk number, i.e.
+  // bit 5 of the byte offset, for the odd blocks).
+  const uint32_t wblock0 = (uint32_t)((wave & 3) * WD) * 1024u;
+  const uint32_t wlane = wblock0 + (uint32_t)((lane >> 3) * kRowB + (((lane & 7) ^ swz(lane >> 3)) * 16));
+
+  // XCD-aware persistent schedule: XCD x owns a contiguous run of tiles and hands
+  // them out round robin to its workgroups.
+  const int total_tiles = a.n_ptiles * a.n_ctiles * g.G;
+  const int xcd = (int)(blockIdx.x & 7);
+  const int stride = (int)(gridDim.x >> 3);
+  const int chunk = (total_tiles + 7) >> 3;
+  const int first = xcd * chunk + (int)(blockIdx.x >> 3);
+  const int tile_end = min((xcd + 1) * chunk, total_tiles);
+  if (first >= tile_end) return;  // (a whole workgroup: the barriers below are never short of waves)
+  const int T = (tile_end - first + stride - 1) / stride;
+
+  auto decode = [&](int t, int &ctile, int &grp, int &p0) __attribute__((always_inline)) {
+    int L = first + t * stride;
+    const int nct = tile_s(a.n_ctiles), ng = tile_s(g.G);
+    ctile = L % nct;
+    L /= nct;
+    grp = L % ng;
+    p0 = (L / ng) * PT;
+    // (uniform, and kept in scalar registers: the divisions run on the vector ALU)
+    ctile = __builtin_amdgcn_readfirstlane(ctile);
+    grp = __builtin_amdgcn_readfirstlane(grp);
+    p0 = __builtin_amdgcn_readfirstlane(p0);
+  };
+
+  // ---- (pixel, tap) table of tile t, in two halves: the loads (kept in registers
+  // over the last MFMA phase of the previous tile), then the entries.  Lane serves
+  // pixel tid % 256, taps tid / 256 + 2 i.
+  E rdy[TPT], rdx[TPT], rm[TPT];
+  auto table_load = [&](int t) {
+    const int tt = tile_tid();
+    const int tapq = tt >> 8;
+    int ctile, grp, p0;
+    decode(t, ctile, grp, p0);
+    const int tb_p = p0 + (tt & (PT - 1));
+    const int po = tile_s(plane_out);
+    int tb_n = 0, tb_rem = 0;
+    if (tb_p < total_px) {
+      tb_n = tb_p / po;
+      tb_rem = tb_p - tb_n * po;
+    }
+    const E *off = (const E *)a.om.off + (long)tb_n * a.om.off_n + (long)tb_rem * a.om.off_px;
+    const E *msk = (const E *)a.om.msk + (long)tb_n * a.om.msk_n + (long)tb_rem * a.om.msk_px;
+#pragma unroll
+    for (int i = 0; i < TPT; ++i) {
+      const int tap = min(tapq + 2 * i, taps - 1);
+      rdy[i] = off[(long)(2 * tap) * a.om.off_ch];
+      rdx[i] = off[(long)(2 * tap + 1) * a.om.off_ch];
+      rm[i] = msk[(long)tap * a.om.msk_ch];
+    }
+  };
+  auto table_store = [&](int t) {
+    const int tt = tile_tid();
+    const int tapq = tt >> 8;
+    int ctile, grp, p0;
+    decode(t, ctile, grp, p0);
+    const int tb_pl = tt & (PT - 1);
+    const int tb_p = p0 + tb_pl;
+    const bool tb_valid = tb_p < total_px;
+    const int po = tile_s(plane_out), wo = tile_s(g.Wo), kw = tile_s(g.kw);
+    const int gh = tile_s(g.H), gw = tile_s(g.W);
+    int tb_n = 0, tb_ho = 0, tb_wo = 0;
+    if (tb_valid) {
+      tb_n = tb_p / po;
+      const int tb_rem = tb_p - tb_n * po;
+      tb_ho = tb_rem / wo;
+      tb_wo = tb_rem - tb_ho * wo;
+    }
+#pragma unroll
+    for (int i = 0; i < TPT; ++i) {
+      const int tap = tapq + 2 * i;
+      if (tap < taps) {
+        const int ti = tap / kw, tj = tap - ti * kw;
+        TapSample sm = make_tap_sample(tb_ho * g.sh - g.ph + ti * g.dh, tb_wo * g.sw - g.pw + tj * g.dw,
+                                       to_f32(rdy[i]), to_f32(rdx[i]), mask_value<E>(rm[i], a.om.logit), gh, gw);
+        const uint32_t pix = tb_valid ? (uint32_t)tb_n * a.img_bytes + corner_offset<false>(sm, g, a) : 0u;
+        uint2 w2 = make_uint2(TR::pack2(sm.w00, sm.w01), TR::pack2(sm.w10, sm.w11));
+        if (!tb_valid) w2 = make_uint2(0u, 0u);
+        tpix[tap * PT + tb_pl] = pix;
+        tws[tap * PT + tb_pl] = w2;
+      }
+    }
+    // Retire the loads of table_load with a wait the compiler can see: those of taps
+    // past the last one are never read, and the compiler would otherwise keep their
+    // registers marked as pending and guard later writes to them with full waits.
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), other counters untouched
+  };
+
+  // ---- cursors of the produce side within a tile (uniform): the tap of the step to
+  // blend next; slab and tap of the step to gather next
+  int b_tap = 0, g_tap = 0, g_slab = 0, slab0 = 0;
+  const unsigned char *w_ptr = nullptr;   // packed weights of the tile, step 0
+  auto start_tile = [&](int t) {
+    int ctile, grp, p0;
+    decode(t, ctile, grp, p0);
+    b_tap = g_tap = g_slab = 0;
+    slab0 = __builtin_amdgcn_readfirstlane(grp * g.cin_g / KC);
+    w_ptr = uniform_ptr((const unsigned char *)a.wp + (size_t)(grp * a.n_ctiles + ctile) * nk * (size_t)kWTile);
+  };
+
+  // gather registers: four pixels x four corners
+  u32x4 gs[4][4];
+  // slab part of the gather addresses of the step to gather next; moves the cursor on
+  auto next_slab_offset = [&]() {
+    const uint32_t add_ = (uint32_t)(slab0 + g_slab) * a.slab_bytes + (uint32_t)ck * 16u;
+    if (++g_tap == taps) {
+      g_tap = 0;
+      ++g_slab;
+    }
+    return add_;
+  };
+
+  // weight tile of step kk into ring slot `slot` (late waves)
+  auto issue_weights = [&](int kk, int slot) {
+    const uint32_t voff = (uint32_t)kk * kWTile + wlane;
+    const uint32_t voff_odd = voff ^ 32u;
+    const uint32_t dst = lds_w + (uint32_t)slot * kWTile + wblock0;
+    if (!(MDCN_F2_ABLATE & 2)) {
+      // (the instruction's offset moves the LDS side along with the global one)
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\t"
+                   "global_load_lds_dwordx4 %1, %3\n\t"
+                   "global_load_lds_dwordx4 %2, %3 offset:1024\n\t"
+                   "global_load_lds_dwordx4 %1, %3 offset:2048\n\t"
+                   "global_load_lds_dwordx4 %2, %3 offset:3072"
+                   :
+                   : "s"(dst), "v"(voff), "v"(voff_odd), "s"(w_ptr)
+                   : "memory");
+      if constexpr (WD == 8) {
+        const uint32_t voff2 = voff + 4096u, voff2_odd = voff_odd + 4096u;
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\t"
+                     "global_load_lds_dwordx4 %1, %3\n\t"
+                     "global_load_lds_dwordx4 %2, %3 offset:1024\n\t"
+                     "global_load_lds_dwordx4 %1, %3 offset:2048\n\t"
+                     "global_load_lds_dwordx4 %2, %3 offset:3072"
+                     :
+                     : "s"(dst + 4096u), "v"(voff2), "v"(voff2_odd), "s"(w_ptr)
+                     : "memory");
+      }
+    }
+  };
+  static_assert(WD == 8 || WD == 4, "issue_weights spells out the copies");
+
+  // Blend of the lane's pixel I of the step the blend cursor is on into sample tile
+  // XB, after a wait that leaves VM younger vector-memory operations in flight; with
+  // GATHER the pixel's loads for the step behind it are issued right away.  The
+  // table entries of pixel I + 1 (blend weights; corner offset of the step to
+  // gather) are read one pixel ahead.
+#define MDCN_F3_PIXEL(I, VM, XB, GATHER)                                                         \
+  do {                                                                                           \
+    const uint2 twc_ = tw_;                                                                      \
+    const uint32_t npc_ = np_ + add_;                                                            \
+    if constexpr ((I) < 3) {                                                                     \
+      tw_ = twp_[8 * ((I) + 1)];                                                                 \
+      if constexpr (GATHER) np_ = tp_[8 * ((I) + 1)];                                            \
+    }                                                                                            \
+    const typename BL::Wt w_ = BL::prep(twc_, q);                                                \
+    f3_vmwait4<VM>(gs[I][0], gs[I][1], gs[I][2], gs[I][3]);                                      \
+    const u32x4 o_ = (MDCN_F2_ABLATE & 4) ? (gs[I][0] ^ gs[I][1] ^ gs[I][2] ^ gs[I][3]) : BL::run(gs[I], w_); \
+    *(lds_u32x4_ptr)(uintptr_t)((((I) & 1) ? xwb : xwa) + (uint32_t)(((I) >> 1) * 16 * kRowB) + (XB) * kXTile) = o_; \
+    if constexpr (GATHER) MDCN_F3_GLOAD4(gs[I], npc_, xt, xt_row);                               \
+  } while (0)
+  // One produce block of the K loop: blend a step, gather the one behind it.  VM: see
+  // kVmBlend.  STEADY = false is the block of a tile's last step but one: nothing
+  // is gathered any more, so the loads in flight thin out pixel by pixel.
+#define MDCN_F3_BLOCK(VM, XB, STEADY)                                                            \
+  do {                                                                                           \
+    const uint2 *twp_ = &tws[b_tap * PT + pl];                                                   \
+    const uint32_t *tp_ = &tpix[g_tap * PT + pl];                                                \
+    uint2 tw_ = twp_[0];                                                                         \
+    uint32_t np_ = 0u, add_ = 0u;                                                                \
+    if constexpr (STEADY) {                                                                      \
+      np_ = tp_[0];                                                                              \
+      add_ = next_slab_offset();                                                                 \
+    }                                                                                            \
+    if (++b_tap == taps) b_tap = 0;                                                              \
+    MDCN_F3_PIXEL(0, (STEADY ? (VM) : (VM) - 0), XB, STEADY);                                    \
+    MDCN_F3_PIXEL(1, (STEADY ? (VM) : (VM) - 4), XB, STEADY);                                    \
+    MDCN_F3_PIXEL(2, (STEADY ? (VM) : (VM) - 8), XB, STEADY);                                    \
+    MDCN_F3_PIXEL(3, (STEADY ? (VM) : (VM) - 12), XB, STEADY);                                   \
+  } while (0)
+
+  f32x16 acc[NB][MB];
+
+  // ---- MFMA phase of one step: sample tile and ring slot XB.  The step is a chain
+  // of 4 * MB groups -- K sub-step s = G / MB, channel block mb = G % MB -- of two
+  // MFMAs (both pixel blocks against one channel block); the fragments of a group
+  // (the channel block; with a new sub-step also the two pixel blocks) are read
+  // kF3Ahead groups ahead.
+  u32x4 xf[4][NB], wf[4][MB];
+#define MDCN_F3_NREADS(G) ((G) < NG ? (((G) % MB) == 0 ? 3 : 1) : 0)
+#define MDCN_F3_READS(G)                                                                         \
+  do {                                                                                           \
+    if constexpr ((G) < NG) {                                                                    \
+      constexpr int s_ = (G) / MB, m_ = (G) % MB;                                                \
+      const uint32_t wk_ = wb_ ^ (uint32_t)(s_ << 5);                                            \
+      if constexpr (m_ == 0) {                                                                   \
+        const uint32_t xk_ = xb_ ^ (uint32_t)(s_ << 5);                                          \
+        MDCN_DSREAD(xf[s_][0], xk_, 0);                                                          \
+        MDCN_DSREAD(xf[s_][1], xk_, 4096);                                                       \
+      }                                                                                          \
+      MDCN_DSREAD(wf[s_][m_], wk_, m_ * 4096);                                                   \
+    }                                                                                            \
+  } while (0)
+#define MDCN_F3_GROUP(G)                                                                         \
+  do {                                                                                           \
+    if constexpr ((G) < NG) {                                                                    \
+      constexpr int s_ = (G) / MB, m_ = (G) % MB;                                                \
+      constexpr int after_ = MDCN_F3_NREADS((G) + 1) + MDCN_F3_NREADS((G) + 2) + MDCN_F3_NREADS((G) + 3); \
+      if constexpr (m_ == 0)                                                                     \
+        f3_lgkmwait3<after_>(xf[s_][0], xf[s_][1], wf[s_][0]);                                   \
+      else                                                                                       \
+        f3_lgkmwait1<after_>(wf[s_][m_]);                                                        \
+      _Pragma("unroll") for (int nb_ = 0; nb_ < NB; ++nb_) {                                     \
+        if (!(MDCN_F2_ABLATE & 8))                                                               \
+          TR::mma(acc[nb_][m_], __builtin_bit_cast(uint4, xf[s_][nb_]),                          \
+                  __builtin_bit_cast(uint4, wf[s_][m_]));                                        \
+        else                                                                                     \
+          acc[nb_][m_][s_] += __uint_as_float(xf[s_][nb_].x ^ wf[s_][m_].y);                     \
+      }                                                                                          \
+      MDCN_F3_READS((G) + 4);                                                                    \
+    }                                                                                            \
+  } while (0)
+  // (priority: the arbiter prefers the wave of a SIMD that produces -- a chain of short
+  // dependent steps whose delay moves the barrier -- over the one that streams MFMAs)
+#define MDCN_F3_MFMA(XB)                                                                         \
+  do {                                                                                           \
+    uint32_t xb_ = lds_x + (XB) * kXTile + xa0;                                                  \
+    uint32_t wb_ = lds_w + (XB) * kWTile + wa0;                                                  \
+    /* (opaque: the four sub-step addresses of both tiles would otherwise live in registers across the loop) */ \
+    asm volatile("" : "+v"(xb_), "+v"(wb_));                                                     \
+    __builtin_amdgcn_s_setprio(0);                                                               \
+    MDCN_F3_READS(0); MDCN_F3_READS(1); MDCN_F3_READS(2); MDCN_F3_READS(3);                      \
+    MDCN_F3_GROUP(0); MDCN_F3_GROUP(1); MDCN_F3_GROUP(2); MDCN_F3_GROUP(3);                      \
+    MDCN_F3_GROUP(4); MDCN_F3_GROUP(5); MDCN_F3_GROUP(6); MDCN_F3_GROUP(7);                      \
+    MDCN_F3_GROUP(8); MDCN_F3_GROUP(9); MDCN_F3_GROUP(10); MDCN_F3_GROUP(11);                    \
+    MDCN_F3_GROUP(12); MDCN_F3_GROUP(13); MDCN_F3_GROUP(14); MDCN_F3_GROUP(15);                  \
+    __builtin_amdgcn_s_setprio(2);                                                               \
+  } while (0)
+
+  // One step k of the K loop between two barriers (XB = k % 2): MFMAs on sample tile
+  // and ring slot XB, blend of step k + 1 into the other sample tile, gather of step
+  // k + 2; the late waves first copy the weight tile of step k + 1 into the other slot.
+#define MDCN_F3_STEP(KK, XB, STEADY)                                     \
+  do {                                                                   \
+    if constexpr (LATE) {                                                \
+      issue_weights((KK) + 1, 1 - (XB));                                 \
+      MDCN_F3_BLOCK(kVmBlend, 1 - (XB), STEADY);                         \
+      __builtin_amdgcn_sched_barrier(0);                                 \
+      MDCN_F3_MFMA(XB);                                                  \
+      __builtin_amdgcn_sched_barrier(0);                                 \
+      if constexpr (STEADY) MDCN_BARRIER(kVmBar);                        \
+      else MDCN_BARRIER(0);                                              \
+    } else {                                                             \
+      MDCN_F3_MFMA(XB);                                                  \
+      __builtin_amdgcn_sched_barrier(0);                                 \
+      MDCN_F3_BLOCK(kVmBlend, 1 - (XB), STEADY);                         \
+      MDCN_BARRIER_LDS();                                                \
+    }                                                                    \
+    __builtin_amdgcn_sched_barrier(0);                                   \
+  } while (0)
+
+  // Start of a tile whose table is in LDS: first gathers and weight tile, [the
+  // previous tile's stores, by the caller,] blend of step 0, gather of step 1.
+  auto tile_head_issue = [&]() {
+    const uint32_t *tp_ = &tpix[g_tap * PT + pl];
+    const uint32_t add_ = next_slab_offset();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t o_ = tp_[8 * i] + add_;
+      MDCN_F3_GLOAD4(gs[i], o_, xt, xt_row);
+    }
+    if constexpr (LATE) issue_weights(0, 0);
+  };
+  auto tile_head_blend = [&]() {
+    // everything this wave has in flight -- the sixteen loads, the weight copies, the previous tile's
+    // stores -- has landed
+#pragma unroll
+    for (int i = 0; i < 4; ++i) f3_vmwait4<0>(gs[i][0], gs[i][1], gs[i][2], gs[i][3]);
+    // (... and the compiler is told so: what it still counts as pending -- the stores, the table's loads --
+    // would otherwise reach the K loop's header, and it would guard registers there with full waits)
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), other counters untouched
+    const uint2 *twp_ = &tws[b_tap * PT + pl];
+    if (++b_tap == taps) b_tap = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const typename BL::Wt w_ = BL::prep(twp_[8 * i], q);
+      const u32x4 o_ = (MDCN_F2_ABLATE & 4) ? (gs[i][0] ^ gs[i][1] ^ gs[i][2] ^ gs[i][3]) : BL::run(gs[i], w_);
+      *(lds_u32x4_ptr)(uintptr_t)(((i & 1) ? xwb : xwa) + (uint32_t)((i >> 1) * 16 * kRowB)) = o_;
+    }
+    const uint32_t *tp_ = &tpix[g_tap * PT + pl];
+    const uint32_t add_ = next_slab_offset();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t o_ = tp_[8 * i] + add_;
+      MDCN_F3_GLOAD4(gs[i], o_, xt, xt_row);
+    }
+    MDCN_BARRIER_LDS();  // X[0] complete (W[0] landed before the blend)
+  };
+
+  start_tile(0);
+  table_load(0);
+  table_store(0);
+  MDCN_BARRIER_LDS();  // table visible
+  __builtin_amdgcn_sched_barrier(0);
+  tile_head_issue();
+  tile_head_blend();
+  __builtin_amdgcn_sched_barrier(0);
+
+  // ---- epilogue: bias, one rounding, NCHW store straight from the accumulators.
+  // Accumulator block (A = samples, B = weights): register r of lane l holds
+  //   pixel = (r/4)*8 + (l/32)*4 + r%4,  channel = l%32.
+  // The two halves of the wave exchange packed pixel pairs, after which a lane
+  // holds 8 consecutive pixels = 16 bytes of one channel.  The host gives this
+  // kernel whole tiles only and output planes of whole, aligned 16-byte runs that
+  // are at least 64 pixels long, so every run is one 16-byte store and the wave's 64
+  // pixels cross at most one image boundary, between two runs.
+  auto store_tile = [&](int t) __attribute__((always_inline)) {
+    int ctile, grp, p0;
+    decode(t, ctile, grp, p0);
+    E *out = (E *)a.out;
+    const int tt = tile_tid();
+    const int frow = tt & 31, fhalf = (tt >> 5) & 1;
+    const int pw0 = p0 + wave_p * 64;
+    const int po = tile_s(plane_out);
+    const int n0 = __builtin_amdgcn_readfirstlane(pw0 / po);
+    const int rem0 = pw0 - n0 * po + 8 * fhalf;       // of the lane's first run
+    const long next_image = (long)(g.Cout - 1) * po;  // what a run in the following image adds to the address
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      const int col = ctile * CT + wave_c * WCH + mb * 32 + frow;
+      const bool col_ok = col < g.cout_g;
+      const long cbase = (long)grp * g.cout_g + col;
+      const float bvm = (a.bias && col_ok) ? to_f32(((const E *)a.bias)[cbase]) : 0.0f;
+      E *row = out + ((long)n0 * g.Cout + cbase) * po + rem0;
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+        const f32x16 &c = acc[nb][mb];
+#pragma unroll
+        for (int g2 = 0; g2 < 2; ++g2) {
+          const int ga = 2 * g2, gb = 2 * g2 + 1;
+          const uint32_t a0 = TR::pack2(c[4 * ga + 0] + bvm, c[4 * ga + 1] + bvm);
+          const uint32_t a1 = TR::pack2(c[4 * ga + 2] + bvm, c[4 * ga + 3] + bvm);
+          const uint32_t b0 = TR::pack2(c[4 * gb + 0] + bvm, c[4 * gb + 1] + bvm);
+          const uint32_t b1 = TR::pack2(c[4 * gb + 2] + bvm, c[4 * gb + 3] + bvm);
+          // lower half keeps group ga and receives the upper half's part of it; upper half likewise with gb
+          const auto s0 = __builtin_amdgcn_permlane32_swap(a0, b0, false, false);
+          const auto s1 = __builtin_amdgcn_permlane32_swap(a1, b1, false, false);
+          u32x4 val;
+          val.x = s0[0]; val.y = s1[0]; val.z = s0[1]; val.w = s1[1];
+          const int dp = nb * 32 + 16 * g2;
+          E *dst = row + dp + ((rem0 + dp >= po) ? next_image : 0L);
+          if (col_ok) *(u32x4 *)dst = val;
+        }
+      }
+    }
+  };
+
+  // K loop of a tile up to its last step but one (which still blends the last step; nothing is gathered any more)
+#define MDCN_F3_KLOOP()                                                  \
+  do {                                                                   \
+    _Pragma("unroll") for (int nb = 0; nb < NB; ++nb)                    \
+      _Pragma("unroll") for (int mb = 0; mb < MB; ++mb)                  \
+        _Pragma("unroll") for (int r = 0; r < 16; ++r) acc[nb][mb][r] = 0.0f; \
+    for (int k = 0; k < nk - 2; k += 2) {                                \
+      MDCN_F3_STEP(k, 0, true);                                          \
+      MDCN_F3_STEP(k + 1, 1, true);                                      \
+    }                                                                    \
+    MDCN_F3_STEP(nk - 2, 0, false);                                      \
+  } while (0)
+
+  // All tiles but the last: the head of the next tile is folded into the end of each.  (The last tile has
+  // its own copy of the K loop rather than a way out of this one: a join of "gathers in flight" and "none
+  // in flight" in front of the epilogue would leave the build's scan of the assembly nothing to hold on to.)
+  for (int t = 0; t + 1 < T; ++t) {
+    MDCN_F3_KLOOP();
+    table_load(t + 1);   // (the table was last read by the blend in front of the barrier just passed)
+    __builtin_amdgcn_sched_barrier(0);
+    MDCN_F3_MFMA(1);
+    __builtin_amdgcn_sched_barrier(0);
+    table_store(t + 1);
+    start_tile(t + 1);
+    MDCN_BARRIER_LDS();  // every wave is through with the tile's last MFMAs; the new table is visible
+    __builtin_amdgcn_sched_barrier(0);
+    tile_head_issue();
+    __builtin_amdgcn_sched_barrier(0);
+    store_tile(t);
+    __builtin_amdgcn_sched_barrier(0);
+    tile_head_blend();
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  MDCN_F3_KLOOP();
+  MDCN_F3_MFMA(1);
+  __builtin_amdgcn_sched_barrier(0);
+  store_tile(T - 1);
+#undef MDCN_F3_KLOOP
+#undef MDCN_F3_STEP
+#undef MDCN_F3_MFMA
+#undef MDCN_F3_GROUP
+#undef MDCN_F3_READS
+#undef MDCN_F3_NREADS
+#undef MDCN_F3_BLOCK
+#undef MDCN_F3_PIXEL
+}
+
+template <typename E, int CT>
+__global__ __launch_bounds__(kF3Threads) void fused3_kernel(FusedArgs a) {
+  __shared__ uint4 Xs[2][kF3PT * kRowChunks];      // sample tiles
+  __shared__ uint4 Ws[2][CT * kRowChunks];         // weight tiles
+  __shared__ uint32_t tpix[kF3PT * kF3Taps];       // (pixel, tap) table, [tap][pixel]: corner byte offset
+  __shared__ uint2 tws[kF3PT * kF3Taps];           // ... and the blend weights
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const uint32_t lds_x = (uint32_t)(uintptr_t)(lptr_t)(&Xs[0][0]);
+  const uint32_t lds_w = (uint32_t)(uintptr_t)(lptr_t)(&Ws[0][0]);
+  if (wave >= 4) {
+    MDCN_ROLE("late");
+    fused3_role<E, CT, true>(a, lds_x, lds_w, tpix, tws, wave);
+  } else {
+    MDCN_ROLE("early");
+    fused3_role<E, CT, false>(a, lds_x, lds_w, tpix, tws, wave);
+  }
+}
+
+}  // namespace mdcn
