@@ -184,13 +184,14 @@ bool uses_fused2(const mdcn_params *p, const Geom &g, const Plan &pl) {
 }
 
 // ... and the kernel with 256-pixel tiles for whole tiles of such a call: bordered input copy, an even
-// number of K steps, output planes of whole 16-byte runs (the caller checks the pointer's alignment)
+// number of K steps, output planes of whole 16-byte runs (the caller checks the pointer's alignment), groups of
+// whole channel tiles
 bool wide_ok(const mdcn_params *p, const Geom &g, const Plan &pl) {
   if (!pl.fused || !uses_fused2(p, g, pl) || pl.CT != 256 || p->input_nhwc || p->path == MDCN_PATH_FUSED_NARROW)
     return false;
   const int nk = pl.slabs * g.taps;
   const long plane_out = (long)g.Ho * g.Wo;
-  return nk >= kF3MinSteps && nk % 2 == 0 && plane_out % 8 == 0 && plane_out >= 64;
+  return nk >= kF3MinSteps && nk % 2 == 0 && plane_out % 8 == 0 && plane_out >= 64 && g.cout_g % pl.CT == 0;
 }
 
 // Rounds of the 128-pixel kernel's schedule for `tiles` tiles of nk K steps, in tile times (its last round's
@@ -210,7 +211,8 @@ double narrow_rounds(long tiles, int nk, bool may_cut) {
 // How many of a launch's pixel tiles of 256 go to the wide kernel: all of them (`all`), or whole rounds of
 // its one-workgroup-per-CU grid when that and the 128-pixel kernel on the rest come out shorter than the
 // 128-pixel kernel alone.  kWideTileCost: time of a 256-pixel tile in units of a 128-pixel one (measured).
-constexpr double kWideTileCost = 1.65;
+constexpr double kWideTileCost = 1.71;   // (cfg 4: 79.7 us per round of 256-pixel tiles against 46.6 us)
+constexpr double kSecondKernelCost = 0.45;  // what launching the 128-pixel kernel behind it costs (ramps, table, tail)
 long wide_tiles(long total_px, int n_ctiles_groups, int nk, bool may_cut, bool all) {
   const long full = total_px / kF3PT;
   if (all || full == 0) return full;
@@ -219,7 +221,7 @@ long wide_tiles(long total_px, int n_ctiles_groups, int nk, bool may_cut, bool a
     const long wg_tiles = (n3 * n_ctiles_groups + grid - 1) / grid;  // tiles of the busiest workgroup
     const long px2 = total_px - n3 * kF3PT;
     const long tiles2 = (px2 + kPT - 1) / kPT * n_ctiles_groups;
-    return wg_tiles * kWideTileCost + narrow_rounds(tiles2, nk, may_cut) + ((n3 && tiles2) ? 0.05 : 0.0);
+    return wg_tiles * kWideTileCost + narrow_rounds(tiles2, nk, may_cut) + ((n3 && tiles2) ? kSecondKernelCost : 0.0);
   };
   const long rounds = full * n_ctiles_groups / grid;
   const long whole = rounds * grid / n_ctiles_groups;  // pixel tiles of the whole rounds

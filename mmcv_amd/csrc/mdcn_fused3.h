@@ -250,11 +250,12 @@ __device__ __forceinline__ void fused3_role(const FusedArgs &a, const uint32_t l
         tws[tap * PT + tb_pl] = w2;
       }
     }
-    // Retire the loads of table_load with a wait the compiler can see: those of taps
-    // past the last one are never read, and the compiler would otherwise keep their
-    // registers marked as pending and guard later writes to them with full waits.
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), other counters untouched
   };
+  // Retires the loads of table_load with a wait the compiler can see (those of taps past the last one are
+  // never read, and the compiler would otherwise keep their registers marked as pending and guard later
+  // writes to them -- the assembly loads of the K loop -- with full waits).  Called where nothing else is
+  // in flight, i.e. in front of the stores of a tile, not behind them.
+  auto table_loads_landed = [&]() { __builtin_amdgcn_s_waitcnt(0x0F70); };  // vmcnt(0), other counters untouched
 
   // ---- cursors of the produce side within a tile (uniform): the tap of the step to
   // blend next; slab and tap of the step to gather next
@@ -441,39 +442,36 @@ __device__ __forceinline__ void fused3_role(const FusedArgs &a, const uint32_t l
     }
     if constexpr (LATE) issue_weights(0, 0);
   };
-  auto tile_head_blend = [&]() {
-    // everything this wave has in flight -- the sixteen loads, the weight copies, the previous tile's
-    // stores -- has landed
-#pragma unroll
-    for (int i = 0; i < 4; ++i) f3_vmwait4<0>(gs[i][0], gs[i][1], gs[i][2], gs[i][3]);
-    // (... and the compiler is told so: what it still counts as pending -- the stores, the table's loads --
-    // would otherwise reach the K loop's header, and it would guard registers there with full waits)
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), other counters untouched
-    const uint2 *twp_ = &tws[b_tap * PT + pl];
-    if (++b_tap == taps) b_tap = 0;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const typename BL::Wt w_ = BL::prep(twp_[8 * i], q);
-      const u32x4 o_ = (MDCN_F2_ABLATE & 4) ? (gs[i][0] ^ gs[i][1] ^ gs[i][2] ^ gs[i][3]) : BL::run(gs[i], w_);
-      *(lds_u32x4_ptr)(uintptr_t)(((i & 1) ? xwb : xwa) + (uint32_t)((i >> 1) * 16 * kRowB)) = o_;
-    }
-    const uint32_t *tp_ = &tpix[g_tap * PT + pl];
-    const uint32_t add_ = next_slab_offset();
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const uint32_t o_ = tp_[8 * i] + add_;
-      MDCN_F3_GLOAD4(gs[i], o_, xt, xt_row);
-    }
-    MDCN_BARRIER_LDS();  // X[0] complete (W[0] landed before the blend)
-  };
+  // ... STORES: vector-memory stores this wave has issued behind the gathers (the previous tile's output)
+#define MDCN_F3_HEAD_BLEND(STORES)                                                                        \
+  do {                                                                                                    \
+    /* the sixteen loads and the weight copies have landed; the stores, issued behind them, may still be  \
+       on their way (vector-memory operations complete in the order of issue) */                          \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i) f3_vmwait4<STORES>(gs[i][0], gs[i][1], gs[i][2], gs[i][3]); \
+    const uint2 *twp_ = &tws[b_tap * PT + pl];                                                            \
+    if (++b_tap == taps) b_tap = 0;                                                                       \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                                       \
+      const typename BL::Wt w_ = BL::prep(twp_[8 * i], q);                                                \
+      const u32x4 o_ = (MDCN_F2_ABLATE & 4) ? (gs[i][0] ^ gs[i][1] ^ gs[i][2] ^ gs[i][3]) : BL::run(gs[i], w_); \
+      *(lds_u32x4_ptr)(uintptr_t)(((i & 1) ? xwb : xwa) + (uint32_t)((i >> 1) * 16 * kRowB)) = o_;        \
+    }                                                                                                     \
+    const uint32_t *tp_ = &tpix[g_tap * PT + pl];                                                         \
+    const uint32_t add_ = next_slab_offset();                                                             \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                                       \
+      const uint32_t o_ = tp_[8 * i] + add_;                                                              \
+      MDCN_F3_GLOAD4(gs[i], o_, xt, xt_row);                                                              \
+    }                                                                                                     \
+    MDCN_BARRIER_LDS(); /* X[0] complete (W[0] landed before the blend) */                                \
+  } while (0)
 
   start_tile(0);
   table_load(0);
   table_store(0);
+  table_loads_landed();
   MDCN_BARRIER_LDS();  // table visible
   __builtin_amdgcn_sched_barrier(0);
   tile_head_issue();
-  tile_head_blend();
+  MDCN_F3_HEAD_BLEND(0);
   __builtin_amdgcn_sched_barrier(0);
 
   // ---- epilogue: bias, one rounding, NCHW store straight from the accumulators.
@@ -483,7 +481,8 @@ __device__ __forceinline__ void fused3_role(const FusedArgs &a, const uint32_t l
   // holds 8 consecutive pixels = 16 bytes of one channel.  The host gives this
   // kernel whole tiles only and output planes of whole, aligned 16-byte runs that
   // are at least 64 pixels long, so every run is one 16-byte store and the wave's 64
-  // pixels cross at most one image boundary, between two runs.
+  // pixels cross at most one image boundary, between two runs; and groups of whole
+  // channel tiles (Cout / G a multiple of CT), so no lane is ever without a channel.
   auto store_tile = [&](int t) __attribute__((always_inline)) {
     int ctile, grp, p0;
     decode(t, ctile, grp, p0);
@@ -495,12 +494,20 @@ __device__ __forceinline__ void fused3_role(const FusedArgs &a, const uint32_t l
     const int n0 = __builtin_amdgcn_readfirstlane(pw0 / po);
     const int rem0 = pw0 - n0 * po + 8 * fhalf;       // of the lane's first run
     const long next_image = (long)(g.Cout - 1) * po;  // what a run in the following image adds to the address
+    // (the bias values first: a load behind a store would wait for the store.  Every channel of the tile
+    // exists -- the host gives this kernel groups of whole channel tiles only -- so each lane issues exactly
+    // 4 * MB stores here, which the wait at the head of the next tile counts on.)
+    float bv[MB];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
       const int col = ctile * CT + wave_c * WCH + mb * 32 + frow;
-      const bool col_ok = col < g.cout_g;
+      bv[mb] = a.bias ? to_f32(((const E *)a.bias)[(long)grp * g.cout_g + col]) : 0.0f;
+    }
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      const int col = ctile * CT + wave_c * WCH + mb * 32 + frow;
       const long cbase = (long)grp * g.cout_g + col;
-      const float bvm = (a.bias && col_ok) ? to_f32(((const E *)a.bias)[cbase]) : 0.0f;
+      const float bvm = bv[mb];
       E *row = out + ((long)n0 * g.Cout + cbase) * po + rem0;
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) {
@@ -519,7 +526,7 @@ __device__ __forceinline__ void fused3_role(const FusedArgs &a, const uint32_t l
           val.x = s0[0]; val.y = s1[0]; val.z = s0[1]; val.w = s1[1];
           const int dp = nb * 32 + 16 * g2;
           E *dst = row + dp + ((rem0 + dp >= po) ? next_image : 0L);
-          if (col_ok) *(u32x4 *)dst = val;
+          *(u32x4 *)dst = val;
         }
       }
     }
@@ -548,14 +555,15 @@ __device__ __forceinline__ void fused3_role(const FusedArgs &a, const uint32_t l
     MDCN_F3_MFMA(1);
     __builtin_amdgcn_sched_barrier(0);
     table_store(t + 1);
+    table_loads_landed();
     start_tile(t + 1);
     MDCN_BARRIER_LDS();  // every wave is through with the tile's last MFMAs; the new table is visible
     __builtin_amdgcn_sched_barrier(0);
     tile_head_issue();
     __builtin_amdgcn_sched_barrier(0);
-    store_tile(t);
+    store_tile(t);       // 4 * MB stores per lane, the bias loads in front of them waited for
     __builtin_amdgcn_sched_barrier(0);
-    tile_head_blend();
+    MDCN_F3_HEAD_BLEND(4 * MB);
     __builtin_amdgcn_sched_barrier(0);
   }
   MDCN_F3_KLOOP();
@@ -563,6 +571,7 @@ __device__ __forceinline__ void fused3_role(const FusedArgs &a, const uint32_t l
   __builtin_amdgcn_sched_barrier(0);
   store_tile(T - 1);
 #undef MDCN_F3_KLOOP
+#undef MDCN_F3_HEAD_BLEND
 #undef MDCN_F3_STEP
 #undef MDCN_F3_MFMA
 #undef MDCN_F3_GROUP

@@ -194,6 +194,11 @@ def test_full_size_configs(name):
         y_one = capi_forward(dev, path=capi.PATH_FUSED, unsplit=True)
         y_rev = capi_forward(rev, path=capi.PATH_FUSED, unsplit=True)
         assert torch.equal(y_rev.flip(0), y_one)
+        if name == 'cfg4':
+            # the kernel with 256-pixel tiles and the one with 128-pixel tiles sum every tile in the same order
+            y_wide = capi_forward(dev, path=capi.PATH_FUSED_WIDE, unsplit=True)
+            assert torch.equal(y_wide, capi_forward(dev, path=capi.PATH_FUSED_NARROW, unsplit=True))
+            assert torch.equal(y_wide, y_one)
         # cut tiles: same result on every run, and within an output ulp or so of the uncut sums
         assert torch.equal(capi_forward(dev, path=capi.PATH_FUSED), y)
         diff = (y.float() - y_one.float()).abs()

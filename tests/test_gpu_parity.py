@@ -198,3 +198,52 @@ def test_tiles_cut_along_k(name):
         assert diff <= (1e-5 if dtype == torch.float32 else 8e-3)
         for _ in range(3):
             assert torch.equal(capi_forward(dev, path=capi.PATH_FUSED), y_cut)
+
+
+# Shapes that have the kernel with 256-pixel tiles (16-bit tensors, one deformable group, whole channel
+# tiles of 256, an even number of K steps, planes of whole 16-byte runs): workgroups that walk several
+# tiles, waves whose 64 pixels cross an image boundary, two groups, two channel tiles, stride 2, and a
+# pixel count that leaves a rest for the 128-pixel kernel launched beside it.
+WIDE = {
+    'tiles_and_rest': dict(N=2, Cin=256, Cout=256, H=24, W=24),            # 4 tiles of 256 + 128 pixels
+    'one_tile': dict(N=1, Cin=128, Cout=256, H=16, W=16),                  # 18 K steps, exactly one tile
+    'images_inside_a_wave': dict(N=3, Cin=256, Cout=256, H=20, W=24, sigma=4.0),
+    'two_groups': dict(N=2, Cin=512, Cout=512, H=16, W=24, groups=2),
+    'two_channel_tiles': dict(N=2, Cin=128, Cout=512, H=16, W=16),
+    'stride2': dict(N=2, Cin=128, Cout=256, H=33, W=32, stride=2),
+    'several_tiles_per_workgroup': dict(N=9, Cin=128, Cout=256, H=96, W=88),  # 297 tiles on 256 workgroups
+    'no_bias_k1x3': dict(N=2, Cin=512, Cout=256, H=16, W=24, k=(1, 3), padding=(0, 1), bias=False),  # 24 K steps
+}
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('name', sorted(WIDE))
+def test_wide_tile_kernel(name, dtype):
+    """Every whole tile of 256 pixels through the 256-pixel kernel: against the oracle, and bit for bit
+    against the 128-pixel kernel (the two sum a tile's K range in the same order)."""
+    print(f'case={name} dtype={dtype}', flush=True)
+    case = make_case(777, **WIDE[name])
+    dev = cast_case(case, dtype, 'cuda')
+    ref = oracle_forward(cast_case(case, dtype))
+    y = capi_forward(dev, path=capi.PATH_FUSED_WIDE, unsplit=True)
+    y_narrow = capi_forward(dev, path=capi.PATH_FUSED_NARROW, unsplit=True)
+    assert rel_err(y.float().cpu().numpy(), ref) <= TOL[dtype]
+    assert torch.equal(y, y_narrow)
+    # (... and with the rest's tiles cut along K by the 128-pixel kernel)
+    y_cut = capi_forward(dev, path=capi.PATH_FUSED_WIDE)
+    assert rel_err(y_cut.float().cpu().numpy(), ref) <= TOL[dtype]
+
+
+def test_wide_tile_kernel_needs_its_shape():
+    """MDCN_PATH_FUSED_WIDE is an error where the shape has no 256-pixel kernel (fp32; channel tiles that
+    are not whole; several deformable groups); the default path takes such shapes elsewhere."""
+    import ctypes
+    lib = capi.load()
+    x = torch.zeros(1, device='cuda')
+    for dt, kw in ((capi.MDCN_F32, dict(Cin=256, Cout=256)), (capi.MDCN_BF16, dict(Cin=256, Cout=200)),
+                   (capi.MDCN_BF16, dict(Cin=256, Cout=256, dg=2)), (capi.MDCN_BF16, dict(Cin=64, Cout=256))):
+        p = capi.make_params(dt, 1, kw['Cin'], 16, 16, kw['Cout'], 3, 3, (1, 1), (1, 1), (1, 1), 1, kw.get('dg', 1),
+                             capi.PATH_FUSED_WIDE)
+        p.input = p.offset = p.mask = p.weight = p.output = x.data_ptr()
+        assert lib.mdcn_workspace_bytes(ctypes.byref(p)) == 0
+        assert lib.mdcn_forward(ctypes.byref(p), None) == -5, kw  # MDCN_ERR_PATH
