@@ -191,7 +191,8 @@ bool wide_ok(const mdcn_params *p, const Geom &g, const Plan &pl) {
     return false;
   const int nk = pl.slabs * g.taps;
   const long plane_out = (long)g.Ho * g.Wo;
-  return nk >= kF3MinSteps && nk % 2 == 0 && plane_out % 8 == 0 && plane_out >= 64 && g.cout_g % pl.CT == 0;
+  return nk >= kF3MinSteps && nk % 2 == 0 && g.taps >= kF3MinTaps && plane_out % 8 == 0 && plane_out >= 64 &&
+         g.cout_g % pl.CT == 0 && g.Cout <= kF3MaxBias;
 }
 
 // Rounds of the 128-pixel kernel's schedule for `tiles` tiles of nk K steps, in tile times (its last round's

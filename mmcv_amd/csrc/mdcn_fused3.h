@@ -1,5 +1,5 @@
 // Fused DCNv2 forward for gfx950, 16-bit tensors, tiles of 256 pixels x CT (256 or
-// 128) output channels, one deformable group, at most 9 taps, bordered input copy:
+// 128) output channels, one deformable group, 3 to 9 taps, bordered input copy:
 // the implicit GEMM of mdcn_fused.h / mdcn_fused2.h with a tile twice as tall.
 //
 // Why another tile.  Per K step (128 bytes of channels of one tap) a tile of PT
@@ -24,24 +24,34 @@
 // waves 0-3 ("early") run their MFMAs first and produce afterwards, waves 4-7
 // ("late") produce first.  The late waves also issue the whole direct-to-LDS copy
 // of the next step's weight tile, right behind the barrier: the ring holds two
-// tiles (LDS: 2 x 32 KiB samples + 2 x 32 KiB weights + the 27 KiB table), so a
-// slot is free only once every wave has passed the barrier that ends its step,
-// and the early waves' MFMA phase, which comes first, is kept free of vector-memory
-// instructions.  One barrier per step.
+// tiles (LDS: 2 x 32 KiB samples + 2 x 32 KiB weights + the 27 KiB table + the
+// bias), so a slot is free only once every wave has passed the barrier that ends
+// its step, and the early waves' MFMA phase, which comes first, is kept free of
+// vector-memory instructions.  One barrier per step.
 //
-// Tile after tile: the (pixel, tap) table exists once, so its next edition is
-// built when the last blend of a tile has read it -- offsets and mask are loaded
-// before the last step's MFMAs and turned into table entries behind them -- and
-// the first gathers of the next tile fly while the accumulators are stored.
-// A tile's K range is never cut here: the host gives this kernel whole rounds of
-// tiles (every workgroup the same number) and the rest of the pixels to the
-// 128-pixel kernel of mdcn_fused2.h.
+// The produce side streams across the tiles of a workgroup: its cursors (gather,
+// blend, weight copy) walk one sequence of steps, tile after tile, two, one and
+// one step ahead of the MFMAs, so the memory pipeline never drains between
+// tiles.  The (pixel, tap) table exists once.  K runs slab outer, tap inner, so a
+// tap's row of the table is read for the last time in the tile's last slab; from
+// there on the early waves -- whose produce half is the lighter one -- rewrite
+// it, one row per step, for the next tile: each of them serves its own 32 pixels
+// and those of the late wave four above it, loads offsets and mask one step
+// ahead and writes the row one barrier after its last reader.  A tile's output
+// is stored right behind its last MFMAs; the bias comes from a copy in LDS, so
+// that the K loop holds no load the compiler knows of (it would guard such a
+// load's registers with waits that drain the gathers).
+// A tile's K range is never cut here: the host gives this kernel whole tiles
+// only (and decides how many), the rest of the pixels go to the 128-pixel kernel
+// of mdcn_fused2.h.
 //
-// All vector-memory traffic of the K loop is issued from inline assembly and
+// All vector-memory loads of the K loop are issued from inline assembly and
 // waited for with explicit counts (see mdcn_fused2.h for why); per wave and step
-// the order of issue is fixed -- late waves: WD weight copies; then, both kinds,
-// four groups of four gather loads -- so the number of younger operations at
-// every wait is a constant.
+// the order of issue is fixed -- late waves: WD weight copies; early waves: three
+// loads for the table; then, both kinds, four groups of four gather loads -- so
+// the number of younger loads at every wait is a constant.  (The stores of a
+// tile's output are younger still where they occur; they only make a wait
+// stricter.)
 #pragma once
 
 #include "mdcn_fused2.h"
@@ -52,8 +62,10 @@ constexpr int kF3PT = 256;             // pixels per tile
 constexpr int kF3Threads = 512;
 constexpr int kF3Taps = kTapsSmall;    // table capacity (kh * kw)
 constexpr int kF3MinSteps = 4;         // K steps per tile the pipeline needs (and an even number of them)
+constexpr int kF3MinTaps = 3;          // a row of the table is rewritten at least two steps before its next reader
+constexpr int kF3MaxBias = 2048;       // output channels whose bias the kernel keeps in LDS
 constexpr size_t fused3_lds_bytes(int CT) {
-  return (size_t)2 * kF3PT * kRowB + (size_t)2 * CT * kRowB + (size_t)kF3PT * kF3Taps * 12;
+  return (size_t)2 * kF3PT * kRowB + (size_t)2 * CT * kRowB + (size_t)kF3PT * kF3Taps * 12 + (size_t)kF3MaxBias * 2;
 }
 
 // four corners of one pixel: 16 bytes per lane each, from `base` / `base_row`
@@ -99,7 +111,7 @@ __device__ __forceinline__ void f3_lgkmwait1(u32x4 &a) {
 // be free to move it).
 template <typename E, int CT, bool LATE>
 __device__ __forceinline__ void fused3_role(const FusedArgs &a, const uint32_t lds_x, const uint32_t lds_w,
-                                            uint32_t *tpix, uint2 *tws, const int wave) {
+                                            uint32_t *tpix, uint2 *tws, E *bias_s, const int wave) {
   using TR = ElemTraits<E>;
   using BL = Blend2<E>;
   static_assert(sizeof(E) == 2, "16-bit element types");
@@ -107,39 +119,38 @@ __device__ __forceinline__ void fused3_role(const FusedArgs &a, const uint32_t l
   constexpr int PT = kF3PT;
   constexpr int KC = TR::KC;
   constexpr int TMAX = kF3Taps;
-  constexpr int TBL = PT * TMAX;               // entries of the table
-  constexpr int TPT = (TMAX + 1) / 2;          // table entries per lane and build
+  constexpr int TPT = (TMAX + 1) / 2;          // table entries per lane of the first tile's build
   constexpr int NB = 2, MB = CT / 64;          // 32 x 32 accumulator blocks per wave: pixels x channels
   constexpr int WCH = CT / 2;                  // output channels per wave
   constexpr int WD = CT / 32;                  // 1 KiB weight copies per late wave and K step
   constexpr int NG = 4 * MB;                   // MFMA groups (2 MFMAs each) per K step
-  // vector-memory operations younger than the loads of a pixel when it is blended:
-  // the pixels behind it of the same step and the ones before it of the next (12
-  // loads), for the late waves also the weight copies issued in between
-  constexpr int kVmBlend = LATE ? 12 + WD : 12;
-  // ... younger than the weight copies at the barrier that ends their step (late waves)
-  constexpr int kVmBar = 16;
+  constexpr int TL = LATE ? 0 : 3;             // table loads per early wave and K step
+  // loads younger than those of a pixel when it is blended: the pixels behind it of the same step and the
+  // ones before it of the next (12), and what the wave issues in between (weight copies / table loads)
+  constexpr int kVmBlend = 12 + (LATE ? WD : TL);
+  // ... younger than the weight copies (late waves) at the barrier that ends their step, and than the
+  // table loads (early waves) where the step after theirs uses them: the sixteen gathers
+  constexpr int kVmStep = 16;
   constexpr uint32_t kXTile = PT * kRowB, kWTile = CT * kRowB;
   static_assert(fused3_lds_bytes(CT) <= 160 * 1024, "LDS of one compute unit");
 
   const Geom &g = a.g;
   const int taps = g.taps;
-  const int nk = a.slabs * taps;               // even and >= kF3MinSteps (the host checks)
+  const int slabs = a.slabs;
+  const int nk = slabs * taps;                 // even and >= kF3MinSteps (the host checks)
   const int plane_out = g.Ho * g.Wo;
-  const int total_px = (int)a.total_px;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  // The code that runs once per tile (table, epilogue) takes the thread index through this: what it
-  // derives from it is then computed there, not once per kernel and kept in -- spilled -- registers
-  // across the K loop.
+  // The code that runs once per tile (epilogue) takes the thread index through this: what it derives from
+  // it is then computed there, not once per kernel and kept in -- spilled -- registers across the K loop.
   auto tile_tid = [&]() __attribute__((always_inline)) {
     int v = tid;
     asm volatile("" : "+v"(v));
     return v;
   };
   // (likewise the divisors of that code: the reciprocals its divisions go through are computed on the
-  // vector ALU, and hoisted out of the tile loop they would each hold a vector register for good)
+  // vector ALU, and hoisted out of the loop they would each hold a vector register for good)
   auto tile_s = [](int v) __attribute__((always_inline)) {
     asm volatile("" : "+s"(v));
     return v;
@@ -192,98 +203,74 @@ __device__ __forceinline__ void fused3_role(const FusedArgs &a, const uint32_t l
     grp = __builtin_amdgcn_readfirstlane(grp);
     p0 = __builtin_amdgcn_readfirstlane(p0);
   };
-
-  // ---- (pixel, tap) table of tile t, in two halves: the loads (kept in registers
-  // over the last MFMA phase of the previous tile), then the entries.  Lane serves
-  // pixel tid % 256, taps tid / 256 + 2 i.
-  E rdy[TPT], rdx[TPT], rm[TPT];
-  auto table_load = [&](int t) {
-    const int tt = tile_tid();
-    const int tapq = tt >> 8;
+  auto slab0_of = [&](int t) __attribute__((always_inline)) {
     int ctile, grp, p0;
     decode(t, ctile, grp, p0);
-    const int tb_p = p0 + (tt & (PT - 1));
-    const int po = tile_s(plane_out);
-    int tb_n = 0, tb_rem = 0;
-    if (tb_p < total_px) {
-      tb_n = tb_p / po;
-      tb_rem = tb_p - tb_n * po;
-    }
-    const E *off = (const E *)a.om.off + (long)tb_n * a.om.off_n + (long)tb_rem * a.om.off_px;
-    const E *msk = (const E *)a.om.msk + (long)tb_n * a.om.msk_n + (long)tb_rem * a.om.msk_px;
-#pragma unroll
-    for (int i = 0; i < TPT; ++i) {
-      const int tap = min(tapq + 2 * i, taps - 1);
-      rdy[i] = off[(long)(2 * tap) * a.om.off_ch];
-      rdx[i] = off[(long)(2 * tap + 1) * a.om.off_ch];
-      rm[i] = msk[(long)tap * a.om.msk_ch];
-    }
+    return __builtin_amdgcn_readfirstlane(grp * g.cin_g / KC);
   };
-  auto table_store = [&](int t) {
-    const int tt = tile_tid();
-    const int tapq = tt >> 8;
+  auto weights_of = [&](int t) __attribute__((always_inline)) {
     int ctile, grp, p0;
     decode(t, ctile, grp, p0);
-    const int tb_pl = tt & (PT - 1);
-    const int tb_p = p0 + tb_pl;
-    const bool tb_valid = tb_p < total_px;
+    return uniform_ptr((const unsigned char *)a.wp + (size_t)(grp * a.n_ctiles + ctile) * nk * (size_t)kWTile);
+  };
+
+  // One entry of the (pixel, tap) table: pixel p (of the whole launch; every pixel of this kernel's tiles
+  // exists), tap, its two offsets and its mask value as stored.
+  auto table_entry = [&](int p, int tap, E dy, E dx, E m, int tb_pl) __attribute__((always_inline)) {
     const int po = tile_s(plane_out), wo = tile_s(g.Wo), kw = tile_s(g.kw);
-    const int gh = tile_s(g.H), gw = tile_s(g.W);
-    int tb_n = 0, tb_ho = 0, tb_wo = 0;
-    if (tb_valid) {
-      tb_n = tb_p / po;
-      const int tb_rem = tb_p - tb_n * po;
-      tb_ho = tb_rem / wo;
-      tb_wo = tb_rem - tb_ho * wo;
-    }
-#pragma unroll
-    for (int i = 0; i < TPT; ++i) {
-      const int tap = tapq + 2 * i;
-      if (tap < taps) {
-        const int ti = tap / kw, tj = tap - ti * kw;
-        TapSample sm = make_tap_sample(tb_ho * g.sh - g.ph + ti * g.dh, tb_wo * g.sw - g.pw + tj * g.dw,
-                                       to_f32(rdy[i]), to_f32(rdx[i]), mask_value<E>(rm[i], a.om.logit), gh, gw);
-        const uint32_t pix = tb_valid ? (uint32_t)tb_n * a.img_bytes + corner_offset<false>(sm, g, a) : 0u;
-        uint2 w2 = make_uint2(TR::pack2(sm.w00, sm.w01), TR::pack2(sm.w10, sm.w11));
-        if (!tb_valid) w2 = make_uint2(0u, 0u);
-        tpix[tap * PT + tb_pl] = pix;
-        tws[tap * PT + tb_pl] = w2;
-      }
-    }
+    const int tb_n = p / po;
+    const int tb_rem = p - tb_n * po;
+    const int tb_ho = tb_rem / wo;
+    const int tb_wo = tb_rem - tb_ho * wo;
+    const int ti = tap / kw, tj = tap - ti * kw;
+    TapSample sm = make_tap_sample(tb_ho * g.sh - g.ph + ti * g.dh, tb_wo * g.sw - g.pw + tj * g.dw, to_f32(dy),
+                                   to_f32(dx), mask_value<E>(m, a.om.logit), g.H, g.W);
+    tpix[tap * PT + tb_pl] = (uint32_t)tb_n * a.img_bytes + corner_offset<false>(sm, g, a);
+    tws[tap * PT + tb_pl] = make_uint2(TR::pack2(sm.w00, sm.w01), TR::pack2(sm.w10, sm.w11));
   };
-  // Retires the loads of table_load with a wait the compiler can see (those of taps past the last one are
-  // never read, and the compiler would otherwise keep their registers marked as pending and guard later
-  // writes to them -- the assembly loads of the K loop -- with full waits).  Called where nothing else is
-  // in flight, i.e. in front of the stores of a tile, not behind them.
-  auto table_loads_landed = [&]() { __builtin_amdgcn_s_waitcnt(0x0F70); };  // vmcnt(0), other counters untouched
+  // where the offsets and the mask of pixel p live (tap 0)
+  auto offsets_of = [&](int p, const E *&off, const E *&msk) __attribute__((always_inline)) {
+    const int po = tile_s(plane_out);
+    const int tb_n = p / po;
+    const int tb_rem = p - tb_n * po;
+    off = (const E *)a.om.off + (long)tb_n * a.om.off_n + (long)tb_rem * a.om.off_px;
+    msk = (const E *)a.om.msk + (long)tb_n * a.om.msk_n + (long)tb_rem * a.om.msk_px;
+  };
 
-  // ---- cursors of the produce side within a tile (uniform): the tap of the step to
-  // blend next; slab and tap of the step to gather next
-  int b_tap = 0, g_tap = 0, g_slab = 0, slab0 = 0;
-  const unsigned char *w_ptr = nullptr;   // packed weights of the tile, step 0
-  auto start_tile = [&](int t) {
-    int ctile, grp, p0;
-    decode(t, ctile, grp, p0);
-    b_tap = g_tap = g_slab = 0;
-    slab0 = __builtin_amdgcn_readfirstlane(grp * g.cin_g / KC);
-    w_ptr = uniform_ptr((const unsigned char *)a.wp + (size_t)(grp * a.n_ctiles + ctile) * nk * (size_t)kWTile);
-  };
+  // ---- cursors of the stream (all uniform).  Steps are counted through the tiles of the workgroup; in
+  // the interval between two barriers in which the MFMAs of step (c_t, c_s) run, the blend cursor is one
+  // step ahead of it, the gather cursor two, the weight-copy cursor one.  Past the last step of the last
+  // tile the gather and weight cursors stay on it (loads nobody uses, which keep the wait counts constant).
+  int c_t = 0, c_s = 0;                                     // MFMAs: tile, step
+  int b_tap = 0;                                            // blend: tap (the table's row; the tile follows from the rewriting)
+  int g_t = 0, g_tap = 0, g_slab = 0, g_slab0 = slab0_of(0);  // gather
+  int w_t = 0, w_s = 0;                                     // weight copies
+  const unsigned char *w_ptr = weights_of(0);               // ... packed weights of tile w_t, step 0
 
   // gather registers: four pixels x four corners
   u32x4 gs[4][4];
-  // slab part of the gather addresses of the step to gather next; moves the cursor on
+  // slab part of the gather addresses of the step the gather cursor is on; moves the cursor on
   auto next_slab_offset = [&]() {
-    const uint32_t add_ = (uint32_t)(slab0 + g_slab) * a.slab_bytes + (uint32_t)ck * 16u;
+    const uint32_t add_ = (uint32_t)(g_slab0 + g_slab) * a.slab_bytes + (uint32_t)ck * 16u;
     if (++g_tap == taps) {
       g_tap = 0;
-      ++g_slab;
+      if (++g_slab == slabs) {
+        if (g_t + 1 < T) {
+          ++g_t;
+          g_slab = 0;
+          g_slab0 = slab0_of(g_t);
+        } else {
+          g_tap = taps - 1;
+          g_slab = slabs - 1;
+        }
+      }
     }
     return add_;
   };
 
-  // weight tile of step kk into ring slot `slot` (late waves)
-  auto issue_weights = [&](int kk, int slot) {
-    const uint32_t voff = (uint32_t)kk * kWTile + wlane;
+  // weight tile of the step the weight cursor is on into ring slot `slot` (late waves); moves the cursor on
+  auto issue_weights = [&](int slot) {
+    const uint32_t voff = (uint32_t)w_s * kWTile + wlane;
     const uint32_t voff_odd = voff ^ 32u;
     const uint32_t dst = lds_w + (uint32_t)slot * kWTile + wblock0;
     if (!(MDCN_F2_ABLATE & 2)) {
@@ -308,46 +295,101 @@ __device__ __forceinline__ void fused3_role(const FusedArgs &a, const uint32_t l
                      : "memory");
       }
     }
+    if (++w_s == nk) {
+      if (w_t + 1 < T) {
+        ++w_t;
+        w_s = 0;
+        w_ptr = weights_of(w_t);
+      } else {
+        w_s = nk - 1;
+      }
+    }
   };
   static_assert(WD == 8 || WD == 4, "issue_weights spells out the copies");
 
+  // ---- the table's next edition (early waves).  In the interval of step (t, s) with s in the tile's last
+  // slab, row s - (nk - taps) is written for tile t + 1: its last readers were the blends of the interval
+  // before, a barrier ago.  Lane l of wave w serves pixel w * 32 + l % 32 + 128 * (l / 32): its own wave's
+  // and those of the late wave four above.  The row's offsets and mask are loaded in the interval before;
+  // with row 0 the lane works out where its pixel of the new tile lies (image, row, column) and keeps that
+  // for the tile's rows.
+  uint32_t tl_dy = 0, tl_dx = 0, tl_m = 0;   // what the interval before loaded (16 bits each)
+  int tb_n = 0, tb_ho = 0, tb_wo = 0;        // the lane's pixel of the tile whose table is being written
+  const int tb_pl = (wave & 3) * 32 + (lane & 31) + ((lane >> 5) << 7);
+  // row that the interval of step (t, s) writes (for tile t + 1); < 0: none
+  auto table_row = [&](int t, int s) __attribute__((always_inline)) { return t + 1 < T ? s - (nk - taps) : -1; };
+  auto table_issue = [&](int t, int s) {  // loads for what the interval of step (t, s) will write
+    const int row = table_row(t, s);
+    const E *pdy = (const E *)a.om.off, *pdx = pdy, *pm = (const E *)a.om.msk;  // (nothing due: any valid address)
+    if (row >= 0) {
+      if (row == 0) {
+        int ctile, grp, p0;
+        decode(t + 1, ctile, grp, p0);
+        const int po = tile_s(plane_out), wo = tile_s(g.Wo);
+        const int p = p0 + tb_pl;
+        tb_n = p / po;
+        const int rem = p - tb_n * po;
+        tb_ho = rem / wo;
+        tb_wo = rem - tb_ho * wo;
+      }
+      const long rem = (long)(tb_ho * g.Wo + tb_wo);
+      const E *off = (const E *)a.om.off + (long)tb_n * a.om.off_n + rem * a.om.off_px;
+      pdy = off + (long)(2 * row) * a.om.off_ch;
+      pdx = pdy + a.om.off_ch;
+      pm = (const E *)a.om.msk + (long)tb_n * a.om.msk_n + rem * a.om.msk_px + (long)row * a.om.msk_ch;
+    }
+    asm volatile("global_load_ushort %0, %3, off\n\t"
+                 "global_load_ushort %1, %4, off\n\t"
+                 "global_load_ushort %2, %5, off"
+                 : "=&v"(tl_dy), "=&v"(tl_dx), "=&v"(tl_m)
+                 : "v"(pdy), "v"(pdx), "v"(pm));
+  };
+  auto table_write = [&](int t, int s) {  // with what table_issue(t, s) loaded, kVmStep loads ago
+    asm volatile("s_waitcnt vmcnt(%3) ; %0 %1 %2" : "+v"(tl_dy), "+v"(tl_dx), "+v"(tl_m) : "n"(kVmStep));
+    const int row = table_row(t, s);
+    if (row >= 0) {
+      const uint16_t by = (uint16_t)tl_dy, bx = (uint16_t)tl_dx, bm = (uint16_t)tl_m;
+      const int kw = tile_s(g.kw);
+      const int ti = __builtin_amdgcn_readfirstlane(row / kw), tj = row - ti * kw;
+      TapSample sm = make_tap_sample(tb_ho * g.sh - g.ph + ti * g.dh, tb_wo * g.sw - g.pw + tj * g.dw,
+                                     to_f32(__builtin_bit_cast(E, by)), to_f32(__builtin_bit_cast(E, bx)),
+                                     mask_value<E>(__builtin_bit_cast(E, bm), a.om.logit), g.H, g.W);
+      tpix[row * PT + tb_pl] = (uint32_t)tb_n * a.img_bytes + corner_offset<false>(sm, g, a);
+      tws[row * PT + tb_pl] = make_uint2(TR::pack2(sm.w00, sm.w01), TR::pack2(sm.w10, sm.w11));
+    }
+  };
+
   // Blend of the lane's pixel I of the step the blend cursor is on into sample tile
-  // XB, after a wait that leaves VM younger vector-memory operations in flight; with
-  // GATHER the pixel's loads for the step behind it are issued right away.  The
-  // table entries of pixel I + 1 (blend weights; corner offset of the step to
-  // gather) are read one pixel ahead.
-#define MDCN_F3_PIXEL(I, VM, XB, GATHER)                                                         \
+  // XB, after a wait that leaves VM younger loads in flight; the pixel's loads for the
+  // step behind it are issued right away.  The table entries of pixel I + 1 (blend
+  // weights; corner offset of the step to gather) are read one pixel ahead.
+#define MDCN_F3_PIXEL(I, VM, XB)                                                                 \
   do {                                                                                           \
     const uint2 twc_ = tw_;                                                                      \
     const uint32_t npc_ = np_ + add_;                                                            \
     if constexpr ((I) < 3) {                                                                     \
       tw_ = twp_[8 * ((I) + 1)];                                                                 \
-      if constexpr (GATHER) np_ = tp_[8 * ((I) + 1)];                                            \
+      np_ = tp_[8 * ((I) + 1)];                                                                  \
     }                                                                                            \
     const typename BL::Wt w_ = BL::prep(twc_, q);                                                \
     f3_vmwait4<VM>(gs[I][0], gs[I][1], gs[I][2], gs[I][3]);                                      \
     const u32x4 o_ = (MDCN_F2_ABLATE & 4) ? (gs[I][0] ^ gs[I][1] ^ gs[I][2] ^ gs[I][3]) : BL::run(gs[I], w_); \
     *(lds_u32x4_ptr)(uintptr_t)((((I) & 1) ? xwb : xwa) + (uint32_t)(((I) >> 1) * 16 * kRowB) + (XB) * kXTile) = o_; \
-    if constexpr (GATHER) MDCN_F3_GLOAD4(gs[I], npc_, xt, xt_row);                               \
+    MDCN_F3_GLOAD4(gs[I], npc_, xt, xt_row);                                                     \
   } while (0)
-  // One produce block of the K loop: blend a step, gather the one behind it.  VM: see
-  // kVmBlend.  STEADY = false is the block of a tile's last step but one: nothing
-  // is gathered any more, so the loads in flight thin out pixel by pixel.
-#define MDCN_F3_BLOCK(VM, XB, STEADY)                                                            \
+  // One produce block: blend the blend cursor's step, gather the gather cursor's.
+#define MDCN_F3_BLOCK(XB)                                                                        \
   do {                                                                                           \
     const uint2 *twp_ = &tws[b_tap * PT + pl];                                                   \
     const uint32_t *tp_ = &tpix[g_tap * PT + pl];                                                \
     uint2 tw_ = twp_[0];                                                                         \
-    uint32_t np_ = 0u, add_ = 0u;                                                                \
-    if constexpr (STEADY) {                                                                      \
-      np_ = tp_[0];                                                                              \
-      add_ = next_slab_offset();                                                                 \
-    }                                                                                            \
+    uint32_t np_ = tp_[0];                                                                       \
+    const uint32_t add_ = next_slab_offset();                                                    \
     if (++b_tap == taps) b_tap = 0;                                                              \
-    MDCN_F3_PIXEL(0, (STEADY ? (VM) : (VM) - 0), XB, STEADY);                                    \
-    MDCN_F3_PIXEL(1, (STEADY ? (VM) : (VM) - 4), XB, STEADY);                                    \
-    MDCN_F3_PIXEL(2, (STEADY ? (VM) : (VM) - 8), XB, STEADY);                                    \
-    MDCN_F3_PIXEL(3, (STEADY ? (VM) : (VM) - 12), XB, STEADY);                                   \
+    MDCN_F3_PIXEL(0, kVmBlend, XB);                                                              \
+    MDCN_F3_PIXEL(1, kVmBlend, XB);                                                              \
+    MDCN_F3_PIXEL(2, kVmBlend, XB);                                                              \
+    MDCN_F3_PIXEL(3, kVmBlend, XB);                                                              \
   } while (0)
 
   f32x16 acc[NB][MB];
@@ -356,7 +398,7 @@ __device__ __forceinline__ void fused3_role(const FusedArgs &a, const uint32_t l
   // of 4 * MB groups -- K sub-step s = G / MB, channel block mb = G % MB -- of two
   // MFMAs (both pixel blocks against one channel block); the fragments of a group
   // (the channel block; with a new sub-step also the two pixel blocks) are read
-  // kF3Ahead groups ahead.
+  // three groups ahead.
   u32x4 xf[4][NB], wf[4][MB];
 #define MDCN_F3_NREADS(G) ((G) < NG ? (((G) % MB) == 0 ? 3 : 1) : 0)
 #define MDCN_F3_READS(G)                                                                         \
@@ -408,106 +450,31 @@ __device__ __forceinline__ void fused3_role(const FusedArgs &a, const uint32_t l
     __builtin_amdgcn_s_setprio(2);                                                               \
   } while (0)
 
-  // One step k of the K loop between two barriers (XB = k % 2): MFMAs on sample tile
-  // and ring slot XB, blend of step k + 1 into the other sample tile, gather of step
-  // k + 2; the late waves first copy the weight tile of step k + 1 into the other slot.
-#define MDCN_F3_STEP(KK, XB, STEADY)                                     \
-  do {                                                                   \
-    if constexpr (LATE) {                                                \
-      issue_weights((KK) + 1, 1 - (XB));                                 \
-      MDCN_F3_BLOCK(kVmBlend, 1 - (XB), STEADY);                         \
-      __builtin_amdgcn_sched_barrier(0);                                 \
-      MDCN_F3_MFMA(XB);                                                  \
-      __builtin_amdgcn_sched_barrier(0);                                 \
-      if constexpr (STEADY) MDCN_BARRIER(kVmBar);                        \
-      else MDCN_BARRIER(0);                                              \
-    } else {                                                             \
-      MDCN_F3_MFMA(XB);                                                  \
-      __builtin_amdgcn_sched_barrier(0);                                 \
-      MDCN_F3_BLOCK(kVmBlend, 1 - (XB), STEADY);                         \
-      MDCN_BARRIER_LDS();                                                \
-    }                                                                    \
-    __builtin_amdgcn_sched_barrier(0);                                   \
-  } while (0)
-
-  // Start of a tile whose table is in LDS: first gathers and weight tile, [the
-  // previous tile's stores, by the caller,] blend of step 0, gather of step 1.
-  auto tile_head_issue = [&]() {
-    const uint32_t *tp_ = &tpix[g_tap * PT + pl];
-    const uint32_t add_ = next_slab_offset();
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const uint32_t o_ = tp_[8 * i] + add_;
-      MDCN_F3_GLOAD4(gs[i], o_, xt, xt_row);
-    }
-    if constexpr (LATE) issue_weights(0, 0);
-  };
-  // ... STORES: vector-memory stores this wave has issued behind the gathers (the previous tile's output)
-#define MDCN_F3_HEAD_BLEND(STORES)                                                                        \
-  do {                                                                                                    \
-    /* the sixteen loads and the weight copies have landed; the stores, issued behind them, may still be  \
-       on their way (vector-memory operations complete in the order of issue) */                          \
-    _Pragma("unroll") for (int i = 0; i < 4; ++i) f3_vmwait4<STORES>(gs[i][0], gs[i][1], gs[i][2], gs[i][3]); \
-    const uint2 *twp_ = &tws[b_tap * PT + pl];                                                            \
-    if (++b_tap == taps) b_tap = 0;                                                                       \
-    _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                                       \
-      const typename BL::Wt w_ = BL::prep(twp_[8 * i], q);                                                \
-      const u32x4 o_ = (MDCN_F2_ABLATE & 4) ? (gs[i][0] ^ gs[i][1] ^ gs[i][2] ^ gs[i][3]) : BL::run(gs[i], w_); \
-      *(lds_u32x4_ptr)(uintptr_t)(((i & 1) ? xwb : xwa) + (uint32_t)((i >> 1) * 16 * kRowB)) = o_;        \
-    }                                                                                                     \
-    const uint32_t *tp_ = &tpix[g_tap * PT + pl];                                                         \
-    const uint32_t add_ = next_slab_offset();                                                             \
-    _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                                       \
-      const uint32_t o_ = tp_[8 * i] + add_;                                                              \
-      MDCN_F3_GLOAD4(gs[i], o_, xt, xt_row);                                                              \
-    }                                                                                                     \
-    MDCN_BARRIER_LDS(); /* X[0] complete (W[0] landed before the blend) */                                \
-  } while (0)
-
-  start_tile(0);
-  table_load(0);
-  table_store(0);
-  table_loads_landed();
-  MDCN_BARRIER_LDS();  // table visible
-  __builtin_amdgcn_sched_barrier(0);
-  tile_head_issue();
-  MDCN_F3_HEAD_BLEND(0);
-  __builtin_amdgcn_sched_barrier(0);
-
-  // ---- epilogue: bias, one rounding, NCHW store straight from the accumulators.
+  // ---- a tile's output: bias, one rounding, NCHW store straight from the accumulators.
   // Accumulator block (A = samples, B = weights): register r of lane l holds
   //   pixel = (r/4)*8 + (l/32)*4 + r%4,  channel = l%32.
   // The two halves of the wave exchange packed pixel pairs, after which a lane
   // holds 8 consecutive pixels = 16 bytes of one channel.  The host gives this
-  // kernel whole tiles only and output planes of whole, aligned 16-byte runs that
-  // are at least 64 pixels long, so every run is one 16-byte store and the wave's 64
-  // pixels cross at most one image boundary, between two runs; and groups of whole
+  // kernel whole tiles only, output planes of whole, aligned 16-byte runs that are
+  // at least 64 pixels long -- so every run is one 16-byte store and the wave's 64
+  // pixels cross at most one image boundary, between two runs -- and groups of whole
   // channel tiles (Cout / G a multiple of CT), so no lane is ever without a channel.
   auto store_tile = [&](int t) __attribute__((always_inline)) {
     int ctile, grp, p0;
     decode(t, ctile, grp, p0);
     E *out = (E *)a.out;
     const int tt = tile_tid();
-    const int frow = tt & 31, fhalf = (tt >> 5) & 1;
+    const int frow_ = tt & 31, fhalf_ = (tt >> 5) & 1;
     const int pw0 = p0 + wave_p * 64;
     const int po = tile_s(plane_out);
     const int n0 = __builtin_amdgcn_readfirstlane(pw0 / po);
-    const int rem0 = pw0 - n0 * po + 8 * fhalf;       // of the lane's first run
+    const int rem0 = pw0 - n0 * po + 8 * fhalf_;      // of the lane's first run
     const long next_image = (long)(g.Cout - 1) * po;  // what a run in the following image adds to the address
-    // (the bias values first: a load behind a store would wait for the store.  Every channel of the tile
-    // exists -- the host gives this kernel groups of whole channel tiles only -- so each lane issues exactly
-    // 4 * MB stores here, which the wait at the head of the next tile counts on.)
-    float bv[MB];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
-      const int col = ctile * CT + wave_c * WCH + mb * 32 + frow;
-      bv[mb] = a.bias ? to_f32(((const E *)a.bias)[(long)grp * g.cout_g + col]) : 0.0f;
-    }
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-      const int col = ctile * CT + wave_c * WCH + mb * 32 + frow;
+      const int col = ctile * CT + wave_c * WCH + mb * 32 + frow_;
       const long cbase = (long)grp * g.cout_g + col;
-      const float bvm = bv[mb];
+      const float bvm = to_f32(bias_s[cbase]);
       E *row = out + ((long)n0 * g.Cout + cbase) * po + rem0;
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) {
@@ -531,48 +498,133 @@ __device__ __forceinline__ void fused3_role(const FusedArgs &a, const uint32_t l
       }
     }
   };
-
-  // K loop of a tile up to its last step but one (which still blends the last step; nothing is gathered any more)
-#define MDCN_F3_KLOOP()                                                  \
+  // behind the MFMAs of a step: the tile's output and fresh accumulators when it was the tile's last;
+  // the MFMA cursor moves on
+#define MDCN_F3_STEP_DONE(MAY_END)                                       \
   do {                                                                   \
-    _Pragma("unroll") for (int nb = 0; nb < NB; ++nb)                    \
-      _Pragma("unroll") for (int mb = 0; mb < MB; ++mb)                  \
-        _Pragma("unroll") for (int r = 0; r < 16; ++r) acc[nb][mb][r] = 0.0f; \
-    for (int k = 0; k < nk - 2; k += 2) {                                \
-      MDCN_F3_STEP(k, 0, true);                                          \
-      MDCN_F3_STEP(k + 1, 1, true);                                      \
+    if (MAY_END && c_s == nk - 1) {                                      \
+      store_tile(c_t);                                                   \
+      _Pragma("unroll") for (int nb = 0; nb < NB; ++nb)                  \
+        _Pragma("unroll") for (int mb = 0; mb < MB; ++mb)                \
+          _Pragma("unroll") for (int r = 0; r < 16; ++r) acc[nb][mb][r] = 0.0f; \
+      ++c_t;                                                             \
+      c_s = 0;                                                           \
+    } else {                                                             \
+      ++c_s;                                                             \
     }                                                                    \
-    MDCN_F3_STEP(nk - 2, 0, false);                                      \
   } while (0)
 
-  // All tiles but the last: the head of the next tile is folded into the end of each.  (The last tile has
-  // its own copy of the K loop rather than a way out of this one: a join of "gathers in flight" and "none
-  // in flight" in front of the epilogue would leave the build's scan of the assembly nothing to hold on to.)
-  for (int t = 0; t + 1 < T; ++t) {
-    MDCN_F3_KLOOP();
-    table_load(t + 1);   // (the table was last read by the blend in front of the barrier just passed)
-    __builtin_amdgcn_sched_barrier(0);
-    MDCN_F3_MFMA(1);
-    __builtin_amdgcn_sched_barrier(0);
-    table_store(t + 1);
-    table_loads_landed();
-    start_tile(t + 1);
-    MDCN_BARRIER_LDS();  // every wave is through with the tile's last MFMAs; the new table is visible
-    __builtin_amdgcn_sched_barrier(0);
-    tile_head_issue();
-    __builtin_amdgcn_sched_barrier(0);
-    store_tile(t);       // 4 * MB stores per lane, the bias loads in front of them waited for
-    __builtin_amdgcn_sched_barrier(0);
-    MDCN_F3_HEAD_BLEND(4 * MB);
-    __builtin_amdgcn_sched_barrier(0);
+  // One step of the stream between two barriers (XB = parity of the step; a tile has an even number of
+  // steps, so its last one has XB = 1): MFMAs on sample tile and ring slot XB, blend of the next step into
+  // the other sample tile, gather of the step after that; the late waves first copy the next step's weight
+  // tile into the other slot, the early waves tend the table.
+#define MDCN_F3_STEP(XB)                                                 \
+  do {                                                                   \
+    if constexpr (LATE) {                                                \
+      issue_weights(1 - (XB));                                           \
+      MDCN_F3_BLOCK(1 - (XB));                                           \
+      __builtin_amdgcn_sched_barrier(0);                                 \
+      MDCN_F3_MFMA(XB);                                                  \
+      __builtin_amdgcn_sched_barrier(0);                                 \
+      MDCN_F3_STEP_DONE((XB) == 1);                                      \
+      MDCN_BARRIER(kVmStep);                                             \
+    } else {                                                             \
+      MDCN_F3_MFMA(XB);                                                  \
+      __builtin_amdgcn_sched_barrier(0);                                 \
+      const int it_ = c_t, is_ = c_s;                                    \
+      MDCN_F3_STEP_DONE((XB) == 1);                                      \
+      table_write(it_, is_);                                             \
+      table_issue(c_t, c_s);                                             \
+      MDCN_F3_BLOCK(1 - (XB));                                           \
+      MDCN_BARRIER_LDS();                                                \
+    }                                                                    \
+    __builtin_amdgcn_sched_barrier(0);                                   \
+  } while (0)
+
+  // ---- start of the stream: the bias and the first tile's table (every lane: pixel tid % 256, taps
+  // tid / 256 + 2 i), the gather of step 0 and its weight tile, its blend, the gather of step 1
+  for (int i = tid; i < g.Cout; i += kF3Threads)
+    bias_s[i] = a.bias ? ((const E *)a.bias)[i] : from_f32<E>(0.0f);
+  {
+    int ctile, grp, p0;
+    decode(0, ctile, grp, p0);
+    const int tapq = tid >> 8, px = tid & (PT - 1);
+    const E *off, *msk;
+    offsets_of(p0 + px, off, msk);
+    E rdy[TPT], rdx[TPT], rm[TPT];
+#pragma unroll
+    for (int i = 0; i < TPT; ++i) {
+      const int tap = min(tapq + 2 * i, taps - 1);
+      rdy[i] = off[(long)(2 * tap) * a.om.off_ch];
+      rdx[i] = off[(long)(2 * tap + 1) * a.om.off_ch];
+      rm[i] = msk[(long)tap * a.om.msk_ch];
+    }
+#pragma unroll
+    for (int i = 0; i < TPT; ++i) {
+      const int tap = tapq + 2 * i;
+      if (tap < taps) table_entry(p0 + px, tap, rdy[i], rdx[i], rm[i], px);
+    }
+    // (retire the loads with a wait the compiler can see: those of taps past the last one are never read,
+    // and it would otherwise keep their registers marked as pending and guard the K loop's assembly loads
+    // into them with full waits)
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), other counters untouched
   }
-  MDCN_F3_KLOOP();
-  MDCN_F3_MFMA(1);
+  MDCN_BARRIER_LDS();  // table and bias visible
   __builtin_amdgcn_sched_barrier(0);
-  store_tile(T - 1);
-#undef MDCN_F3_KLOOP
-#undef MDCN_F3_HEAD_BLEND
+  {
+    const uint32_t *tp_ = &tpix[g_tap * PT + pl];
+    const uint32_t add_ = next_slab_offset();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t o_ = tp_[8 * i] + add_;
+      MDCN_F3_GLOAD4(gs[i], o_, xt, xt_row);
+    }
+  }
+  if constexpr (LATE) issue_weights(0);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) f3_vmwait4<0>(gs[i][0], gs[i][1], gs[i][2], gs[i][3]);
+  {
+    const uint2 *twp_ = &tws[b_tap * PT + pl];
+    if (++b_tap == taps) b_tap = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const typename BL::Wt w_ = BL::prep(twp_[8 * i], q);
+      const u32x4 o_ = (MDCN_F2_ABLATE & 4) ? (gs[i][0] ^ gs[i][1] ^ gs[i][2] ^ gs[i][3]) : BL::run(gs[i], w_);
+      *(lds_u32x4_ptr)(uintptr_t)(((i & 1) ? xwb : xwa) + (uint32_t)((i >> 1) * 16 * kRowB)) = o_;
+    }
+  }
+  if constexpr (!LATE) table_issue(0, 0);
+  {
+    const uint32_t *tp_ = &tpix[g_tap * PT + pl];
+    const uint32_t add_ = next_slab_offset();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t o_ = tp_[8 * i] + add_;
+      MDCN_F3_GLOAD4(gs[i], o_, xt, xt_row);
+    }
+  }
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[nb][mb][r] = 0.0f;
+  MDCN_BARRIER_LDS();  // X[0] complete (W[0] landed before the blend)
+  __builtin_amdgcn_sched_barrier(0);
+
+  // ---- the stream: T tiles of nk steps, two steps per round
+  const int rounds = T * (nk >> 1);
+  for (int r = 0; r < rounds; ++r) {
+    MDCN_F3_STEP(0);
+    MDCN_F3_STEP(1);
+  }
+  // what the cursors issued past the last step has landed before the registers (and the workgroup's LDS)
+  // are given up
+#pragma unroll
+  for (int i = 0; i < 4; ++i) f3_vmwait4<0>(gs[i][0], gs[i][1], gs[i][2], gs[i][3]);
+  asm volatile("s_waitcnt vmcnt(0) ; %0 %1 %2" : "+v"(tl_dy), "+v"(tl_dx), "+v"(tl_m));
 #undef MDCN_F3_STEP
+#undef MDCN_F3_STEP_DONE
 #undef MDCN_F3_MFMA
 #undef MDCN_F3_GROUP
 #undef MDCN_F3_READS
@@ -587,15 +639,16 @@ __global__ __launch_bounds__(kF3Threads) void fused3_kernel(FusedArgs a) {
   __shared__ uint4 Ws[2][CT * kRowChunks];         // weight tiles
   __shared__ uint32_t tpix[kF3PT * kF3Taps];       // (pixel, tap) table, [tap][pixel]: corner byte offset
   __shared__ uint2 tws[kF3PT * kF3Taps];           // ... and the blend weights
+  __shared__ E bias_s[kF3MaxBias];                 // the bias of every output channel (zeros without one)
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const uint32_t lds_x = (uint32_t)(uintptr_t)(lptr_t)(&Xs[0][0]);
   const uint32_t lds_w = (uint32_t)(uintptr_t)(lptr_t)(&Ws[0][0]);
   if (wave >= 4) {
     MDCN_ROLE("late");
-    fused3_role<E, CT, true>(a, lds_x, lds_w, tpix, tws, wave);
+    fused3_role<E, CT, true>(a, lds_x, lds_w, tpix, tws, bias_s, wave);
   } else {
     MDCN_ROLE("early");
-    fused3_role<E, CT, false>(a, lds_x, lds_w, tpix, tws, wave);
+    fused3_role<E, CT, false>(a, lds_x, lds_w, tpix, tws, bias_s, wave);
   }
 }
 
