@@ -1,11 +1,11 @@
 // Bench-only probe, not part of the product library: what the matrix cores of the
 // current device sustain on back-to-back MFMAs (the clock, and with it the rate,
 // depends on how much the operands toggle), for bench.py to print beside the
-// published peak.  Built into lib/libmdcn_probe.so.
+// published peak.  Built into bench_probe/libmfma_probe.so (bench_probe/build.py).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
-#include "mdcn_fused.h"
+#include "../mmcv_amd/csrc/mdcn_fused.h"
 
 namespace mdcn {
 

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define MDCN_ABI_VERSION 4
+#define MDCN_ABI_VERSION 5
 
 /* Element type of every tensor of a call (the Python wrapper unifies them to
  * offset's dtype, mmcv/ops/modulated_deform_conv.py:136-139). */
@@ -144,6 +144,13 @@ int mdcn_output_size(const mdcn_params *p, int32_t *Ho, int32_t *Wo);
  * channels-last input is read in place, so it must be 16-byte aligned -- set it
  * before this query and before mdcn_workspace_bytes(). */
 int mdcn_fused_eligible(const mdcn_params *p);
+
+/* Which device kernels mdcn_forward() launches for the main stage of the call described by *p (shape,
+ * dtype, path, no_k_split; of the pointers only `input` and `output` are looked at, for their alignment):
+ * a static string such as "fused3_kernel", "fused3_kernel+fused2_kernel", "fused2_kernel", "fused_kernel",
+ * "direct_kernel", "f64_forward_kernel"; "" for an invalid *p.  The first name is the kernel that does
+ * most of the work.  For reports and tests (no counterpart in the reference). */
+const char *mdcn_forward_kernels(const mdcn_params *p);
 
 /* Bytes of device scratch mdcn_forward() asks for (of the pointer fields only
  * `input` is looked at, see mdcn_fused_eligible()).  The fused path keeps a

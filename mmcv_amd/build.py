@@ -2,7 +2,6 @@
 
 ``libmdcn_hip.so``  hand-written HIP for gfx950 behind the C ABI of include/mdcn.h
                     (hipcc cross-compiles it without a GPU),
-``libmdcn_probe.so`` the bench's MFMA-rate probe (not part of the product ABI),
 ``_ext*.so``        the PyTorch-ROCm extension module ``mmcv_amd._ext`` (host
                     compiler only) that mmcv's Python op layer binds to.
 
@@ -18,7 +17,6 @@ ROOT = os.path.dirname(PKG)
 CSRC = os.path.join(PKG, 'csrc')
 LIBDIR = os.path.join(PKG, 'lib')
 HIP_LIB = os.path.join(LIBDIR, 'libmdcn_hip.so')
-PROBE_LIB = os.path.join(LIBDIR, 'libmdcn_probe.so')
 EXT_LIB = os.path.join(PKG, '_ext' + sysconfig.get_config_var('EXT_SUFFIX'))
 ROCM = os.environ.get('ROCM_PATH', '/opt/rocm')
 
@@ -69,14 +67,6 @@ def build_hip(extra=(), check=True):
     return HIP_LIB
 
 
-def build_probe():
-    """The bench's MFMA-rate probe: its own library, not part of the product ABI."""
-    hipcc = os.path.join(ROCM, 'bin', 'hipcc')
-    _run([hipcc, *HIPCC_FLAGS, '-I', os.path.join(ROOT, 'include'),
-          '-o', PROBE_LIB, os.path.join(CSRC, 'mdcn_probe.hip')])
-    return PROBE_LIB
-
-
 def build_ext():
     import torch
     tdir = os.path.dirname(torch.__file__)
@@ -103,7 +93,6 @@ def build_ext():
 
 def build_all():
     build_hip()
-    build_probe()
     build_ext()
 
 

@@ -15,7 +15,7 @@ MDCN_OK = 0
 NOALLOC_SCRATCH_BYTES = 64 << 20
 
 EXPORTS = ('mdcn_abi_version', 'mdcn_set_pass_limits', 'mdcn_status_string', 'mdcn_output_size',
-           'mdcn_fused_eligible', 'mdcn_workspace_bytes', 'mdcn_forward', 'mdcn_forward_noalloc',
+           'mdcn_fused_eligible', 'mdcn_forward_kernels', 'mdcn_workspace_bytes', 'mdcn_forward', 'mdcn_forward_noalloc',
            'mdcn_forward_timed', 'mdcn_pack_workspace_bytes', 'mdcn_pack_forward',
            'mdcn_pack_forward_timed', 'mdcn_backward_workspace_bytes', 'mdcn_backward')
 
@@ -62,6 +62,8 @@ def load():
                                          ctypes.POINTER(ctypes.c_int32)]
         lib.mdcn_fused_eligible.restype = ctypes.c_int
         lib.mdcn_fused_eligible.argtypes = [P]
+        lib.mdcn_forward_kernels.restype = ctypes.c_char_p
+        lib.mdcn_forward_kernels.argtypes = [P]
         lib.mdcn_workspace_bytes.restype = ctypes.c_size_t
         lib.mdcn_workspace_bytes.argtypes = [P]
         lib.mdcn_forward.restype = ctypes.c_int

@@ -305,6 +305,12 @@ int make_pack_plan(const mdcn_pack_params *pp, const Geom &g, Plan *pl) {
   return MDCN_OK;
 }
 
+// ... for a launch of total_px pixels of the call *p
+long wide_tiles_of_call(const mdcn_params *p, const Geom &g, const Plan &pl, long total_px, bool out_vec_ok) {
+  if (!wide_ok(p, g, pl) || !out_vec_ok) return 0;
+  return wide_tiles(total_px, pl.n_ctiles * g.G, pl.slabs * g.taps, pl.cut_bytes != 0, p->path == MDCN_PATH_FUSED_WIDE);
+}
+
 // conv_offset of one batch chunk: the tiled kernel when its input patch and one
 // slab of weights fit an LDS budget, else the gather variant.
 template <typename E, int COF>
@@ -592,28 +598,9 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
         fa.om = dense_view((const E *)p->offset + (size_t)n0 * g.DG * 2 * g.taps * plane_out,
                            p->mask ? (const E *)p->mask + (size_t)n0 * g.DG * g.taps * plane_out : nullptr, g);
       }
-      fa.prof = nullptr;
       fa.cut_max = pl.cut_bytes ? kCutMax : 0;
       fa.cut_part = cut_part;
       fa.cut_cnt = cut_cnt;
-#if defined(MDCN_F2_PROFILE) && MDCN_F2_PROFILE
-      {  // profiling build: phase sums land behind the packed weights (the workspace is over-allocated by the harness)
-        static void *prof_buf = nullptr;
-        if (!prof_buf) (void)hipMalloc(&prof_buf, 4096);
-        fa.prof = prof_buf;
-        static bool once = (atexit([]() {
-          long long h[128];
-          if (hipMemcpy(h, prof_buf, sizeof(h), hipMemcpyDeviceToHost) == hipSuccess)
-            for (int b = 0; b < 2; ++b)
-              for (int w = 0; w < 8; ++w) {
-                printf("prof block %d wave %d:", b, w);
-                for (int i = 0; i < 8; ++i) printf(" %lld", h[(b * 8 + w) * 8 + i]);
-                printf("\n");
-              }
-        }), true);
-        (void)once;
-      }
-#endif
       fa.bias = p->bias;
       fa.out = (E *)p->output + (size_t)n0 * g.Cout * plane_out;
       fa.total_px = (long)gc.N * plane_out;
@@ -628,10 +615,9 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
       const bool eight_wave = uses_fused2(p, g, pl);
       bool rest = true;
       if constexpr (sizeof(E) == 2) {
-        if (wide_ok(p, g, pl) && fa.out_vec_ok) {
+        {
           // whole tiles of 256 pixels to the wide kernel, what is left to the 128-pixel one
-          const long n3 = wide_tiles(fa.total_px, pl.n_ctiles * g.G, pl.slabs * g.taps, pl.cut_bytes != 0,
-                                     p->path == MDCN_PATH_FUSED_WIDE);
+          const long n3 = wide_tiles_of_call(p, g, pl, fa.total_px, fa.out_vec_ok != 0);
           if (n3 > 0) {
             FusedArgs fw = fa;
             fw.n_ptiles = (int)n3;
@@ -1214,6 +1200,23 @@ int mdcn_fused_eligible(const mdcn_params *p) {
   Geom g;
   if (check_params(p, &g, false) != MDCN_OK) return 0;
   return fused_ok(p, g) ? 1 : 0;
+}
+
+const char *mdcn_forward_kernels(const mdcn_params *p) {
+  Geom g;
+  if (check_params(p, &g, false) != MDCN_OK) return "";
+  Plan pl;
+  if (make_plan(p, g, &pl) != MDCN_OK) return "";
+  if (p->dtype == MDCN_F64) return "f64_forward_kernel";
+  if (!pl.fused) return "direct_kernel";
+  if (!uses_fused2(p, g, pl)) return "fused_kernel";
+  const size_t es = elem_size(p->dtype);
+  const long plane_out = (long)g.Ho * g.Wo;
+  const bool out_vec_ok = (plane_out % (long)(16 / es) == 0) && (((uintptr_t)p->output % 16) == 0);
+  const long total_px = (long)std::min(pl.n_chunk, g.N) * plane_out;
+  const long n3 = wide_tiles_of_call(p, g, pl, total_px, out_vec_ok);
+  if (n3 == 0) return "fused2_kernel";
+  return total_px - n3 * kF3PT > 0 ? "fused3_kernel+fused2_kernel" : "fused3_kernel";
 }
 
 size_t mdcn_workspace_bytes(const mdcn_params *p) {

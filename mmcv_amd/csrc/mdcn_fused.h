@@ -72,7 +72,6 @@ struct FusedArgs {
   uint32_t px_bytes;   // bytes between horizontally adjacent pixels: kRowB (copy) or Cin * sizeof(E)
   uint32_t slab_bytes; // bytes between channel slabs of one pixel: plane_px * kRowB (copy) or kRowB
   uint32_t img_bytes;  // bytes between images
-  void *prof;          // per-phase clock sums of a profiling build, else unused
   // fused2_kernel only: tiles of the last, partial round of the schedule are cut along K into up to
   // cut_max parts (0 or 1: never) that meet in cut_part, gridDim.x buffers of kPT x 256 floats,
   // counted in cut_cnt, gridDim.x words that are zero when the kernel starts

@@ -37,10 +37,6 @@
 // issued right after the blend that frees its registers), which makes the
 // number of younger operations at every wait a constant.
 //
-// Build-time switches for measurements (all 0 in the product): MDCN_F2_ABLATE
-// (bit 0 no gathers, 1 no weight copies, 2 no blend, 3 no MFMA), MDCN_F2_PROFILE
-// (per-phase clock sums of two workgroups), MDCN_F2_BLEND 0 (bf16 blend on the
-// vector ALU instead of the matrix pipe).
 #pragma once
 
 #include "mdcn_fused.h"
@@ -73,23 +69,8 @@ constexpr size_t fused2_lds_bytes(int CT) {
 }
 
 // 16 bytes per lane from `base` (two SGPRs) + 32-bit byte offset + immediate
-#ifndef MDCN_F2_ABLATE
-#define MDCN_F2_ABLATE 0
-#endif
-#ifndef MDCN_F2_PROFILE
-#define MDCN_F2_PROFILE 0
-#endif
-#if MDCN_F2_PROFILE
-#define MDCN_PROF(slot) do { const long long t_ = clock64(); prof_acc[slot] += t_ - prof_t; prof_t = t_; } while (0)
-#else
-#define MDCN_PROF(slot) do { } while (0)
-#endif
-#if MDCN_F2_ABLATE & 1
-#define MDCN_GLOAD(dst, voff, base, imm) asm volatile("" : "=v"(dst) : "v"(voff), "s"(base), "n"(imm))
-#else
 #define MDCN_GLOAD(dst, voff, base, imm) \
   asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3" : "=v"(dst) : "v"(voff), "s"(base), "n"(imm))
-#endif
 #define MDCN_DSREAD(dst, addr, imm) \
   asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(imm))
 // wait until at most N vector-memory (LDS) operations of this wave are outstanding;
@@ -113,10 +94,6 @@ typedef __attribute__((address_space(3))) u32x4 *lds_u32x4_ptr;
 template <typename E>
 struct Blend2;
 
-#ifndef MDCN_F2_BLEND
-#define MDCN_F2_BLEND 1
-#endif
-#if MDCN_F2_BLEND == 1
 // bf16 on the matrix pipe: one v_mfma_f32_4x4x4 (16 blocks of 4x4x4) takes the four
 // lanes that serve one pixel as one block, a lane's 4 channels (two words) as a
 // column of B and (corner weight) x identity as A -- lane q of the block holds row
@@ -159,36 +136,6 @@ struct Blend2<bf16_t> {
     return o;
   }
 };
-#else
-// bf16 on the vector ALU: a 32-bit word holds two channels; shifting / masking
-// turns each into an fp32 value exactly, the four corners are summed with fp32
-// FMAs and the pair is rounded to bf16 once.
-template <>
-struct Blend2<bf16_t> {
-  struct Wt { float w[4]; };
-  static __device__ __forceinline__ Wt prep(const uint2 &tw, int) {
-    Wt w;
-    w.w[0] = __uint_as_float(tw.x << 16); w.w[1] = __uint_as_float(tw.x & 0xffff0000u);
-    w.w[2] = __uint_as_float(tw.y << 16); w.w[3] = __uint_as_float(tw.y & 0xffff0000u);
-    return w;
-  }
-  static __device__ __forceinline__ u32x4 run(const u32x4 (&v)[4], const Wt &w) {
-    u32x4 o;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      float lo = w.w[0] * __uint_as_float(v[0][j] << 16);
-      float hi = w.w[0] * __uint_as_float(v[0][j] & 0xffff0000u);
-#pragma unroll
-      for (int c = 1; c < 4; ++c) {
-        lo = __builtin_fmaf(w.w[c], __uint_as_float(v[c][j] << 16), lo);
-        hi = __builtin_fmaf(w.w[c], __uint_as_float(v[c][j] & 0xffff0000u), hi);
-      }
-      o[j] = ElemTraits<bf16_t>::pack2(lo, hi);
-    }
-    return o;
-  }
-};
-#endif
 
 // fp16 has packed arithmetic: every corner weight in both halves of a word, one
 // v_pk_mul_f16 and three v_pk_fma_f16 per two channels (the blend then rounds to
@@ -454,7 +401,7 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
     const uint32_t voff = (uint32_t)kk * kWTile + wlane;
     const uint32_t voff_odd = voff ^ 32u;
     const uint32_t dst = lds_w + (uint32_t)islot * kWTile + (uint32_t)(wave * kF2WD) * 1024u;
-    if (!(MDCN_F2_ABLATE & 2)) {
+    {
       // (the instruction's offset moves the LDS side along with the global one; the five idle slots
       // cover a reload of the spilled base pointer right in front of the statement)
       if constexpr (kF2WD == 4)
@@ -528,16 +475,14 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
       {                                                                                 \
         const typename BL::Wt w_ = BL::prep(tw0_, q);                                   \
         MDCN_VMWAIT4(kF2VmBlend, gs[SI][0][0], gs[SI][0][1], gs[SI][0][2], gs[SI][0][3]); \
-        const u32x4 o_ = (MDCN_F2_ABLATE & 4) ? (gs[SI][0][0] ^ gs[SI][0][1] ^ gs[SI][0][2] ^ gs[SI][0][3]) \
-                                              : BL::run(gs[SI][0], w_);                 \
+        const u32x4 o_ = BL::run(gs[SI][0], w_);                                        \
         *(lds_u32x4_ptr)(uintptr_t)(xw0 + xo_) = o_;                                    \
       }                                                                                 \
       MDCN_F2_GATHER_HALF(gs[SI], 0);                                                   \
       {                                                                                 \
         const typename BL::Wt w_ = BL::prep(tw1_, q);                                   \
         MDCN_VMWAIT4(kF2VmBlend, gs[SI][1][0], gs[SI][1][1], gs[SI][1][2], gs[SI][1][3]); \
-        const u32x4 o_ = (MDCN_F2_ABLATE & 4) ? (gs[SI][1][0] ^ gs[SI][1][1] ^ gs[SI][1][2] ^ gs[SI][1][3]) \
-                                              : BL::run(gs[SI][1], w_);                 \
+        const u32x4 o_ = BL::run(gs[SI][1], w_);                                        \
         *(lds_u32x4_ptr)(uintptr_t)(xw1 + xo_) = o_;                                    \
       }                                                                                 \
       MDCN_F2_GATHER_HALF(gs[SI], 1);                                                   \
@@ -591,8 +536,7 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
       for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
-          if (!(MDCN_F2_ABLATE & 8)) TR::mma(acc[nb][mb], __builtin_bit_cast(uint4, xf[s][nb]), __builtin_bit_cast(uint4, wf[s][mb]));
-          else acc[nb][mb][s] += __uint_as_float(xf[s][nb].x ^ wf[s][mb].y);
+          TR::mma(acc[nb][mb], __builtin_bit_cast(uint4, xf[s][nb]), __builtin_bit_cast(uint4, wf[s][mb]));
       if (s + 2 < 4) {
         const uint32_t xk = xb ^ (uint32_t)((s + 2) << 5), wk = wb ^ (uint32_t)((s + 2) << 5);
         MDCN_DSREAD(xf[s + 2][0], xk, 0); MDCN_DSREAD(xf[s + 2][1], xk, 4096);
@@ -603,10 +547,6 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
     __builtin_amdgcn_s_setprio(2);
   };
 
-#if MDCN_F2_PROFILE
-  long long prof_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-  long long prof_t = clock64();
-#endif
 
   // ---- start of the stream: first table, first gathers.  A wave keeps step j of
   // the stream in set j % kF2Sets; the late waves, which run one block ahead, in set
@@ -676,10 +616,8 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
     }
   }
   static_assert(kF2Sets == 3 || kF2Sets == 2, "the prologue spells out the sets");
-  MDCN_PROF(2);
   MDCN_BARRIER(kF2VmBar);  // X[0] and W[0] complete
   __builtin_amdgcn_sched_barrier(0);
-  MDCN_PROF(1);
 
   // ---- K loop of a tile: kF2Unroll steps per round; step k runs the produce
   // block one (late waves: two) steps ahead on set (k + 1) % kF2Sets
@@ -688,22 +626,18 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
     mfma_step(K);                                             \
     prefetch_tw();                                            \
     __builtin_amdgcn_sched_barrier(0);                        \
-    MDCN_PROF(3);                                             \
     if (late) {                                               \
       MDCN_ROLE("late");                                      \
       MDCN_BARRIER(kF2VmBar);                                 \
     }                                                         \
     __builtin_amdgcn_sched_barrier(0);                        \
-    MDCN_PROF(5);                                             \
     MDCN_F2_BLOCK(SI);                                        \
     __builtin_amdgcn_sched_barrier(0);                        \
-    MDCN_PROF(4);                                             \
     if (!late) {                                              \
       MDCN_ROLE("early");                                     \
       MDCN_BARRIER(kF2VmBar);                                 \
     }                                                         \
     __builtin_amdgcn_sched_barrier(0);                        \
-    MDCN_PROF(5);                                             \
   } while (0)
 
   for (int t = 0; t < T; ++t) {
@@ -723,7 +657,6 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
         load_bias(t + 1, bv_next);
         build_table(t + 1);
         __builtin_amdgcn_sched_barrier(0);
-        MDCN_PROF(0);
       }
       MDCN_F2_STEP(k + 0, 1 % kF2Sets);
       MDCN_F2_STEP(k + 1, 2 % kF2Sets);
@@ -902,7 +835,6 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) bv[mb] = bv_next[mb];
     __builtin_amdgcn_sched_barrier(0);
-    MDCN_PROF(6);
   }
   // copies issued past the last step must have landed before the workgroup gives up its LDS
   MDCN_VMWAIT4(0, gs[0][0][0], gs[0][1][0], gs[1][0][0], gs[kF2Sets - 1][1][0]);
@@ -914,12 +846,6 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
 #undef MDCN_F2_BLOCK
 #undef MDCN_F2_GATHER
 #undef MDCN_F2_GATHER_HALF
-#if MDCN_F2_PROFILE
-  // slots: 0 next tile's table, 1 barrier before the K loop, 2 first blocks, 3 MFMA steps,
-  //        4 produce blocks, 5 step barriers, 6 epilogue
-  if (a.prof && lane == 0 && (blockIdx.x == 0 || blockIdx.x == 101))
-    for (int i = 0; i < 8; ++i) ((long long *)a.prof)[((blockIdx.x ? 1 : 0) * 8 + wave) * 8 + i] = prof_acc[i];
-#endif
 }
 
 }  // namespace mdcn

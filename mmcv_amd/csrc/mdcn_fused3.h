@@ -74,10 +74,6 @@ constexpr size_t fused3_lds_bytes(int CT) {
 // reloaded the scalar operands with a vector instruction right in front of the
 // statement, and a vector-memory instruction must not read such a register within
 // the next five issue slots.)
-#if MDCN_F2_ABLATE & 1
-#define MDCN_F3_GLOAD4(d, voff, base, base_row) \
-  asm volatile("" : "=&v"(d[0]), "=&v"(d[1]), "=&v"(d[2]), "=&v"(d[3]) : "v"(voff), "s"(base), "s"(base_row))
-#else
 #define MDCN_F3_GLOAD4(d, voff, base, base_row)                                  \
   asm volatile("s_nop 4\n\t"                                                     \
                "global_load_dwordx4 %0, %4, %5\n\t"                              \
@@ -86,7 +82,6 @@ constexpr size_t fused3_lds_bytes(int CT) {
                "global_load_dwordx4 %3, %4, %6 offset:128"                       \
                : "=&v"(d[0]), "=&v"(d[1]), "=&v"(d[2]), "=&v"(d[3])              \
                : "v"(voff), "s"(base), "s"(base_row))
-#endif
 
 template <int N>
 __device__ __forceinline__ void f3_vmwait4(u32x4 &a, u32x4 &b, u32x4 &c, u32x4 &d) {
@@ -273,7 +268,7 @@ __device__ __forceinline__ void fused3_role(const FusedArgs &a, const uint32_t l
     const uint32_t voff = (uint32_t)w_s * kWTile + wlane;
     const uint32_t voff_odd = voff ^ 32u;
     const uint32_t dst = lds_w + (uint32_t)slot * kWTile + wblock0;
-    if (!(MDCN_F2_ABLATE & 2)) {
+    {
       // (the instruction's offset moves the LDS side along with the global one)
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\t"
                    "global_load_lds_dwordx4 %1, %3\n\t"
@@ -373,7 +368,7 @@ __device__ __forceinline__ void fused3_role(const FusedArgs &a, const uint32_t l
     }                                                                                            \
     const typename BL::Wt w_ = BL::prep(twc_, q);                                                \
     f3_vmwait4<VM>(gs[I][0], gs[I][1], gs[I][2], gs[I][3]);                                      \
-    const u32x4 o_ = (MDCN_F2_ABLATE & 4) ? (gs[I][0] ^ gs[I][1] ^ gs[I][2] ^ gs[I][3]) : BL::run(gs[I], w_); \
+    const u32x4 o_ = BL::run(gs[I], w_);                                                         \
     *(lds_u32x4_ptr)(uintptr_t)((((I) & 1) ? xwb : xwa) + (uint32_t)(((I) >> 1) * 16 * kRowB) + (XB) * kXTile) = o_; \
     MDCN_F3_GLOAD4(gs[I], npc_, xt, xt_row);                                                     \
   } while (0)
@@ -423,13 +418,8 @@ __device__ __forceinline__ void fused3_role(const FusedArgs &a, const uint32_t l
         f3_lgkmwait3<after_>(xf[s_][0], xf[s_][1], wf[s_][0]);                                   \
       else                                                                                       \
         f3_lgkmwait1<after_>(wf[s_][m_]);                                                        \
-      _Pragma("unroll") for (int nb_ = 0; nb_ < NB; ++nb_) {                                     \
-        if (!(MDCN_F2_ABLATE & 8))                                                               \
-          TR::mma(acc[nb_][m_], __builtin_bit_cast(uint4, xf[s_][nb_]),                          \
-                  __builtin_bit_cast(uint4, wf[s_][m_]));                                        \
-        else                                                                                     \
-          acc[nb_][m_][s_] += __uint_as_float(xf[s_][nb_].x ^ wf[s_][m_].y);                     \
-      }                                                                                          \
+      _Pragma("unroll") for (int nb_ = 0; nb_ < NB; ++nb_)                                       \
+        TR::mma(acc[nb_][m_], __builtin_bit_cast(uint4, xf[s_][nb_]), __builtin_bit_cast(uint4, wf[s_][m_])); \
       MDCN_F3_READS((G) + 4);                                                                    \
     }                                                                                            \
   } while (0)
@@ -589,7 +579,7 @@ __device__ __forceinline__ void fused3_role(const FusedArgs &a, const uint32_t l
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const typename BL::Wt w_ = BL::prep(twp_[8 * i], q);
-      const u32x4 o_ = (MDCN_F2_ABLATE & 4) ? (gs[i][0] ^ gs[i][1] ^ gs[i][2] ^ gs[i][3]) : BL::run(gs[i], w_);
+      const u32x4 o_ = BL::run(gs[i], w_);
       *(lds_u32x4_ptr)(uintptr_t)(((i & 1) ? xwb : xwa) + (uint32_t)((i >> 1) * 16 * kRowB)) = o_;
     }
   }

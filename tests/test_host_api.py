@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
     assert sorted(names) == sorted(capi.EXPORTS)
     for n in names:
         assert hasattr(lib, n), n
-    assert lib.mdcn_abi_version() == 4
+    assert lib.mdcn_abi_version() == 5
     assert capi.status_string(0) == 'ok'
     assert 'workspace' in capi.status_string(-4)
 
@@ -108,7 +108,7 @@ def test_ext_module_exports():
     from mmcv_amd.utils import ext_loader
     ext = ext_loader.load_ext('_ext', ['modulated_deform_conv_forward',
                                        'modulated_deform_conv_backward'])
-    assert ext.abi_version() == 4
+    assert ext.abi_version() == 5
     with pytest.raises(AssertionError):
         ext_loader.load_ext('_ext', ['no_such_op'])
     with pytest.raises(ImportError):
