@@ -62,6 +62,9 @@ def build_hip(extra=(), check=True):
                                '(see above and asm_check.py)')
         print(f'asm_check: {len(asm)} device assembly file(s) clean', flush=True)
         shutil.move(out, HIP_LIB)
+        # the assembly the library was built from stays beside it (git-ignored): tests scan it again
+        for f in asm:
+            shutil.copy(f, os.path.join(LIBDIR, 'libmdcn_hip.s' if len(asm) == 1 else os.path.basename(f)))
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
     return HIP_LIB

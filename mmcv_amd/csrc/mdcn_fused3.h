@@ -83,6 +83,12 @@ constexpr size_t fused3_lds_bytes(int CT) {
                : "=&v"(d[0]), "=&v"(d[1]), "=&v"(d[2]), "=&v"(d[3])              \
                : "v"(voff), "s"(base), "s"(base_row))
 
+// Barrier of a step for the waves that copy weight tiles: all but N of the wave's loads have landed -- the
+// youngest direct-to-LDS copies among them, which the comment tells the build's scan of the assembly
+// (asm_check.py) -- and its own LDS operations are done.
+#define MDCN_F3_BARRIER_COPIES(N) \
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0) ; lds-copies\n\ts_barrier" ::"n"(N) : "memory")
+
 template <int N>
 __device__ __forceinline__ void f3_vmwait4(u32x4 &a, u32x4 &b, u32x4 &c, u32x4 &d) {
   asm volatile("s_waitcnt vmcnt(%4) ; %0 %1 %2 %3" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) : "n"(N));
@@ -517,7 +523,7 @@ __device__ __forceinline__ void fused3_role(const FusedArgs &a, const uint32_t l
       MDCN_F3_MFMA(XB);                                                  \
       __builtin_amdgcn_sched_barrier(0);                                 \
       MDCN_F3_STEP_DONE((XB) == 1);                                      \
-      MDCN_BARRIER(kVmStep);                                             \
+      MDCN_F3_BARRIER_COPIES(kVmStep);                                   \
     } else {                                                             \
       MDCN_F3_MFMA(XB);                                                  \
       __builtin_amdgcn_sched_barrier(0);                                 \
@@ -630,6 +636,9 @@ __global__ __launch_bounds__(kF3Threads) void fused3_kernel(FusedArgs a) {
   __shared__ uint32_t tpix[kF3PT * kF3Taps];       // (pixel, tap) table, [tap][pixel]: corner byte offset
   __shared__ uint2 tws[kF3PT * kF3Taps];           // ... and the blend weights
   __shared__ E bias_s[kF3MaxBias];                 // the bias of every output channel (zeros without one)
+  // (for the build's scan of the assembly: every count-based wait of this kernel is to be checked against
+  // the loads issued behind the registers it names)
+  asm volatile("; mdcn-counted-waits");
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const uint32_t lds_x = (uint32_t)(uintptr_t)(lptr_t)(&Xs[0][0]);
   const uint32_t lds_w = (uint32_t)(uintptr_t)(lptr_t)(&Ws[0][0]);

@@ -398,3 +398,88 @@ def test_asm_check_follows_role_markers():
     # a real violation on a consistent path is still found
     bad = kernel(True).replace(wait(20) + '\tv_mov_b32_e32 v1, v20\n', '\tv_mov_b32_e32 v1, v20\n' + wait(20))
     assert len(asm_check.inflight_violations(bad)) == 1
+
+
+def test_asm_check_counts_wait_states_along_branches():
+    """A reload of a scalar at the end of a block reaches an inline-asm memory instruction at a
+    branch target as well: the scan counts wait states along every edge into the instruction,
+    not only along the text in front of it."""
+    from mmcv_amd import asm_check
+    load = '\t;;#ASMSTART\n\tglobal_load_dwordx4 v[2:5], v1, s[6:7]\n\t;;#ASMEND\n'
+    # loop whose latch reloads s7 right in front of the back edge; the loop header starts with the load
+    loop = ('kern:\n\ts_mov_b32 s1, 0\n\tv_mov_b32_e32 v9, v8\n' * 1 + '\tv_mov_b32_e32 v9, v8\n' * 5 +
+            '.LBB0_1:\n' + load + '\tv_mov_b32_e32 v9, v8\n' * 6 +
+            '\tv_readlane_b32 s7, v253, 57\n\ts_cbranch_scc1 .LBB0_1\n\ts_endpgm\n')
+    hits = asm_check.violations(loop)
+    assert len(hits) == 1 and hits[0][2] == [7] and hits[0][3] == 1   # (the branch itself is one slot)
+    # far enough from the back edge, or an s_nop at the head of the asm statement: fine
+    assert asm_check.violations(loop.replace('\tv_readlane_b32 s7, v253, 57\n', '\tv_readlane_b32 s7, v253, 57\n' +
+                                             '\tv_mov_b32_e32 v9, v8\n' * 4)) == []
+    assert asm_check.violations(loop.replace('\tglobal_load_dwordx4 v[2:5]', '\ts_nop 4\n\tglobal_load_dwordx4 v[2:5]')) == []
+    # a forward branch over harmless code into the statement
+    fwd = ('kern:\n\tv_readlane_b32 s6, v253, 3\n\ts_cbranch_scc1 .LBB0_2\n' + '\tv_mov_b32_e32 v9, v8\n' * 8 +
+           '.LBB0_2:\n' + load + '\ts_endpgm\n')
+    assert len(asm_check.violations(fwd)) == 1
+
+
+def test_asm_check_verifies_wait_counts():
+    """Third scan of mmcv_amd/asm_check.py: a wait that names a register must not allow more
+    loads in flight than were issued behind that register's load."""
+    from mmcv_amd import asm_check
+    head = 'kern:\n\t;;#ASMSTART\n\t; mdcn-counted-waits\n\t;;#ASMEND\n'
+    load = lambda r: f'\t;;#ASMSTART\n\tglobal_load_dwordx4 v[{r}:{r + 3}], v[8:9], off\n\t;;#ASMEND\n'
+    wait = lambda n, r: f'\t;;#ASMSTART\n\ts_waitcnt vmcnt({n}) ; v[{r}:{r + 3}]\n\t;;#ASMEND\n'
+    tail = '\ts_endpgm\n'
+    notes = []
+    ok = head + load(20) + load(30) + load(40) + wait(2, 20) + wait(1, 30) + wait(0, 40) + tail
+    assert asm_check.wait_count_findings(ok, notes) == []
+    assert sorted(n[2:] for n in notes) == [(0, 0), (1, 0), (2, 0)]          # every count exactly right
+    bad = asm_check.wait_count_findings(head + load(20) + load(30) + load(40) + wait(3, 20) + tail)
+    assert len(bad) == 4 and bad[0][4] == 2                                  # v20..v23, two loads behind them
+    # stores and compiler loads in between: stores do not count, loads do
+    mixed = head + load(20) + '\tglobal_store_dwordx4 v[8:9], v[50:53], off\n' + load(30) + wait(2, 20) + tail
+    assert len(asm_check.wait_count_findings(mixed)) == 4
+    assert asm_check.wait_count_findings(mixed.replace('global_store_dwordx4 v[8:9], v[50:53], off',
+                                                       'global_load_dword v60, v[8:9], off')) == []
+    # a loop: the count must hold on the shortest way round
+    loop = (head + load(20) + '.LBB0_1:\n' + load(30) + wait(1, 20) + load(20) + wait(1, 30) +
+            '\ts_cbranch_scc1 .LBB0_1\n' + wait(0, 20) + tail)
+    assert asm_check.wait_count_findings(loop) == []
+    assert len(asm_check.wait_count_findings(loop.replace(wait(1, 30), wait(2, 30)))) == 4
+    # direct-to-LDS copies: a wait marked `lds-copies` is about the youngest of them
+    copy = '\t;;#ASMSTART\n\tglobal_load_lds_dwordx4 v7, s[2:3] offset:1024\n\t;;#ASMEND\n'
+    bar = lambda n: f'\t;;#ASMSTART\n\ts_waitcnt vmcnt({n}) lgkmcnt(0) ; lds-copies\n\ts_barrier\n\t;;#ASMEND\n'
+    assert asm_check.wait_count_findings(head + copy + copy + load(20) + load(30) + bar(2) + wait(0, 20) + tail) == []
+    assert len(asm_check.wait_count_findings(head + copy + copy + load(20) + load(30) + bar(3) + tail)) == 1
+    # kernels that do not ask for the check are left alone
+    assert asm_check.wait_count_findings('kern:\n' + load(20) + wait(5, 20) + tail) == []
+
+
+def test_built_library_passes_the_assembly_scans():
+    """The device assembly the library in mmcv_amd/lib was built from (kept beside it by
+    mmcv_amd.build.build_hip) passes all three scans, every count-based wait of the 256-pixel
+    kernel is exactly right on its shortest path, and a count shifted by one is found."""
+    import os
+    import re
+    import pytest
+    from mmcv_amd import asm_check, build
+    path = os.path.join(build.LIBDIR, 'libmdcn_hip.s')
+    if not os.path.exists(path) or os.path.getmtime(path) + 5 < os.path.getmtime(build.HIP_LIB):
+        pytest.skip('no device assembly beside the built library (mmcv_amd/lib/libmdcn_hip.s): built elsewhere '
+                    'or by a build without the scans')
+    text = open(path).read()
+    assert asm_check.violations(text) == []
+    assert asm_check.inflight_violations(text) == []
+    notes = []
+    assert asm_check.wait_count_findings(text, notes) == []
+    eight_wave = [n for n in notes if 'fused3_kernel' in n[0]]
+    assert len(eight_wave) >= 40
+    # waits for a count above zero are tight; waits for zero may have any number of loads behind them
+    assert all(slack == 0 for _, _, count, slack in eight_wave if count > 0), \
+        [n for n in eight_wave if n[2] > 0 and n[3] != 0][:5]
+    # shift one count of the 256-pixel kernel up by one: found
+    k0 = text.index('fused3_kernel')
+    m = re.compile(r's_waitcnt vmcnt\((\d+)\) ; v\[').search(text, k0)
+    assert m and int(m.group(1)) > 0
+    shifted = text[:m.start(1)] + str(int(m.group(1)) + 1) + text[m.end(1):]
+    assert len(asm_check.wait_count_findings(shifted)) >= 1
