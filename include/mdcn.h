@@ -155,12 +155,12 @@ const char *mdcn_forward_kernels(const mdcn_params *p);
 /* Bytes of device scratch mdcn_forward() asks for (of the pointer fields only
  * `input` is looked at, see mdcn_fused_eligible()).  The fused path keeps a
  * zero-bordered channels-last copy of the input and the repacked weights there;
- * the direct path and MDCN_F64 need none.  For 16-bit tensors with 256-channel
- * output tiles the figure ends with an optional region (one 128 x 256 fp32 tile
- * and a counter per workgroup, 32 MiB on a 256-CU device) through which
- * workgroups that would otherwise idle in the last round of the schedule share
- * the K range of a tile: a workspace that is smaller by that region is accepted
- * too and only runs that last round unshared.  Returns 0 for an invalid *p
+ * the direct path and MDCN_F64 need none.  Where the schedule of a launch ends in a
+ * round that fills at most half of an XCD's workgroups (see no_k_split), the figure
+ * ends with an optional region (one 128 x 256 fp32 tile and a counter per workgroup,
+ * 32 MiB on a 256-CU device) through which the workgroups that would otherwise idle
+ * share the K range of that round's tiles: a workspace that is smaller by that region
+ * is accepted too and only runs that last round unshared.  Returns 0 for an invalid *p
  * (mdcn_forward then reports the error). */
 size_t mdcn_workspace_bytes(const mdcn_params *p);
 
@@ -180,7 +180,9 @@ int mdcn_forward(const mdcn_params *p, void *hip_stream);
  * ends).  Calls whose mdcn_workspace_bytes() exceeds that size return
  * MDCN_ERR_SCRATCH_LIMIT and enqueue nothing (the optional region at the end
  * of the workspace is used when it fits as well and left out otherwise).  The call allocates and frees
- * nothing, on the host or on the device.  All calls on one device share the
+ * nothing, on the host or on the device -- from the second call on a device on: the
+ * first one asks the runtime for the buffer's address and the device's CU count, so
+ * make one call outside a graph capture before capturing.  All calls on one device share the
  * buffer: calls that overlap in time on one device (different streams or
  * threads) race; calls on one stream are ordered by the stream.  Nothing in the
  * buffer has to survive between calls: each call rewrites every byte it reads. */

@@ -233,6 +233,12 @@ long wide_tiles(long total_px, int n_ctiles_groups, int nk, bool may_cut, bool a
   return best;
 }
 
+// ... for a launch of total_px pixels of the call *p
+long wide_tiles_of_call(const mdcn_params *p, const Geom &g, const Plan &pl, long total_px, bool out_vec_ok) {
+  if (!wide_ok(p, g, pl) || !out_vec_ok) return 0;
+  return wide_tiles(total_px, pl.n_ctiles * g.G, pl.slabs * g.taps, pl.cut_bytes != 0, p->path == MDCN_PATH_FUSED_WIDE);
+}
+
 int make_plan(const mdcn_params *p, const Geom &g, Plan *pl) {
   const bool ok = fused_ok(p, g);
   if (forced_fused(p->path) && !ok) return MDCN_ERR_PATH;
@@ -266,9 +272,37 @@ int make_plan(const mdcn_params *p, const Geom &g, Plan *pl) {
   pl->n_ctiles = (g.cout_g + pl->CT - 1) / pl->CT;
   pl->xt_bytes = p->input_nhwc ? 0 : align_up((size_t)img * pl->n_chunk);
   pl->wp_bytes = align_up((size_t)g.G * pl->n_ctiles * pl->slabs * g.taps * pl->CT * pl->KC * es);
-  if (!p->no_k_split) {  // one 128 x 256 fp32 tile and a counter per workgroup of the persistent grid
-    pl->cut_wgs = num_cus() / 8 * 8;
-    pl->cut_bytes = align_up((size_t)pl->cut_wgs * kPT * kF2CT * 4) + align_up((size_t)pl->cut_wgs * 4);
+  // Tiles of the 128-pixel kernels' last round are cut along K where workgroups would otherwise idle: one
+  // 128 x 256 fp32 tile and a counter per workgroup of the persistent grid -- asked for only when a launch
+  // of this call has such a round (the 256-pixel kernel never cuts; what it leaves to the 128-pixel one may)
+  if (!p->no_k_split) {
+    const int stride = std::max(1, num_cus() / 8);
+    auto may_cut = [&](long tiles) {  // an XCD's run of tiles ends in a round that fills at most half of its workgroups
+      if (tiles <= 0) return false;
+      const long chunk = (tiles + 7) / 8;
+      for (long run : {chunk, tiles - 7 * chunk}) {
+        const long rest = run > 0 ? run % stride : 0;
+        if (rest > 0 && stride / rest >= 2) return true;
+      }
+      return false;
+    };
+    const long plane_out = (long)g.Ho * g.Wo;
+    bool cuts = false;
+    for (int n0 = 0; n0 < g.N && !cuts; n0 += pl->n_chunk) {
+      const long total_px = (long)std::min(pl->n_chunk, g.N - n0) * plane_out;
+      long px = total_px;
+      if (wide_ok(p, g, *pl)) {
+        // (the split itself looks at whether cutting is allowed: take the answer for "allowed")
+        pl->cut_bytes = 1;
+        px -= wide_tiles_of_call(p, g, *pl, total_px, plane_out % 8 == 0) * kF3PT;
+        pl->cut_bytes = 0;
+      }
+      cuts = may_cut((px + kPT - 1) / kPT * pl->n_ctiles * g.G);
+    }
+    if (cuts) {
+      pl->cut_wgs = num_cus() / 8 * 8;
+      pl->cut_bytes = align_up((size_t)pl->cut_wgs * kPT * kF2CT * 4) + align_up((size_t)pl->cut_wgs * 4);
+    }
   }
   if (p->path == MDCN_PATH_FUSED_WIDE && !wide_ok(p, g, *pl)) return MDCN_ERR_PATH;
   return MDCN_OK;
@@ -303,12 +337,6 @@ int make_pack_plan(const mdcn_pack_params *pp, const Geom &g, Plan *pl) {
     if (!pl->fused && !pp->raw) pl->raw_bytes = align_up((size_t)g.N * pl->CO * plane * es);
   }
   return MDCN_OK;
-}
-
-// ... for a launch of total_px pixels of the call *p
-long wide_tiles_of_call(const mdcn_params *p, const Geom &g, const Plan &pl, long total_px, bool out_vec_ok) {
-  if (!wide_ok(p, g, pl) || !out_vec_ok) return 0;
-  return wide_tiles(total_px, pl.n_ctiles * g.G, pl.slabs * g.taps, pl.cut_bytes != 0, p->path == MDCN_PATH_FUSED_WIDE);
 }
 
 // conv_offset of one batch chunk: the tiled kernel when its input patch and one

@@ -66,3 +66,52 @@ def test_direct_path_shapes_need_no_scratch():
     rc, out, need, _ = noalloc_forward(case)
     assert rc == 0 and need == 0
     assert torch.equal(out, capi_forward(case))
+
+
+def _free_device_bytes():
+    hip = ctypes.CDLL('libamdhip64.so')
+    free, total = ctypes.c_size_t(), ctypes.c_size_t()
+    assert hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+    return free.value
+
+
+def test_in_a_captured_graph_after_one_warm_up_call():
+    """After one ordinary call on the device (which resolves the scratch address and the CU count)
+    the entry point only enqueues kernels: it can be captured into a HIP graph, replays match
+    mdcn_forward() on new contents of the captured tensors, and the device's free memory does
+    not move over the calls."""
+    lib = capi.load()
+    dev = torch.device('cuda:0')
+    kw = dict(N=2, Cin=128, Cout=256, H=24, W=32, sigma=2.0)
+    cases = [cast_case(make_case(60 + i, **kw), torch.bfloat16, dev) for i in range(3)]
+    static = {k: cases[0][k].clone().contiguous() for k in ('input', 'offset', 'mask', 'weight', 'bias')}
+    N, Cin, H, W = static['input'].shape
+    Cout = static['weight'].shape[0]
+    p = capi.make_params(capi.MDCN_BF16, N, Cin, H, W, Cout, 3, 3, (1, 1), (1, 1), (1, 1), 1, 1)
+    out = torch.zeros(N, Cout, H, W, dtype=torch.bfloat16, device=dev)
+    p.input, p.offset, p.mask, p.weight, p.bias = (static[k].data_ptr() for k in ('input', 'offset', 'mask', 'weight', 'bias'))
+    p.output = out.data_ptr()
+    side = torch.cuda.Stream()
+    call = lambda: lib.mdcn_forward_noalloc(ctypes.byref(p), ctypes.c_void_p(side.cuda_stream))
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        assert call() == 0          # the warm-up call, outside any capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        assert call() == 0
+    for i in (1, 2, 0):
+        for k in static:
+            static[k].copy_(cases[i][k])
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        ref = capi_forward(cases[i])    # (eager work and a synchronisation between the replays)
+        assert torch.equal(got, ref), i
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        free1 = _free_device_bytes()
+        assert call() == 0
+        side.synchronize()
+        assert _free_device_bytes() == free1   # an eager call allocates nothing on the device either
