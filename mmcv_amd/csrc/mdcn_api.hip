@@ -187,7 +187,7 @@ bool uses_fused2(const mdcn_params *p, const Geom &g, const Plan &pl) {
 // number of K steps, output planes of whole 16-byte runs (the caller checks the pointer's alignment), groups of
 // whole channel tiles
 bool wide_ok(const mdcn_params *p, const Geom &g, const Plan &pl) {
-  if (!pl.fused || !uses_fused2(p, g, pl) || pl.CT != 256 || p->input_nhwc || p->path == MDCN_PATH_FUSED_NARROW)
+  if (!pl.fused || !uses_fused2(p, g, pl) || p->input_nhwc || p->path == MDCN_PATH_FUSED_NARROW)
     return false;
   const int nk = pl.slabs * g.taps;
   const long plane_out = (long)g.Ho * g.Wo;
@@ -211,10 +211,14 @@ double narrow_rounds(long tiles, int nk, bool may_cut) {
 
 // How many of a launch's pixel tiles of 256 go to the wide kernel: all of them (`all`), or whole rounds of
 // its one-workgroup-per-CU grid when that and the 128-pixel kernel on the rest come out shorter than the
-// 128-pixel kernel alone.  kWideTileCost: time of a 256-pixel tile in units of a 128-pixel one (measured).
-constexpr double kWideTileCost = 1.71;   // (cfg 4: 79.7 us per round of 256-pixel tiles against 46.6 us)
+// 128-pixel kernel alone.  wide_cost: time of a 256-pixel tile in units of a 128-pixel one (measured).
+// 256 channels, stride 1 (N=16, 100x152): 79.7 us per round of 256-pixel tiles against 46.6 us.
+// 128 channels, stride 1 (N=16, 100x168): 29.4 us against 19.4 us.
+// Stride 2 (128 channels, 200x336 input): the wide kernel's main stage takes as long as the narrow one's;
+// neighbouring pixels share no input rows there and the time goes with the rows the L2 delivers.
+inline double wide_tile_cost(int CT, bool unit_stride) { return !unit_stride ? 2.0 : CT == 256 ? 1.71 : 1.52; }
 constexpr double kSecondKernelCost = 0.45;  // what launching the 128-pixel kernel behind it costs (ramps, table, tail)
-long wide_tiles(long total_px, int n_ctiles_groups, int nk, bool may_cut, bool all) {
+long wide_tiles(long total_px, int n_ctiles_groups, int nk, bool may_cut, bool all, double wide_cost) {
   const long full = total_px / kF3PT;
   if (all || full == 0) return full;
   const long grid = std::max(8, num_cus() / 8 * 8);
@@ -222,7 +226,7 @@ long wide_tiles(long total_px, int n_ctiles_groups, int nk, bool may_cut, bool a
     const long wg_tiles = (n3 * n_ctiles_groups + grid - 1) / grid;  // tiles of the busiest workgroup
     const long px2 = total_px - n3 * kF3PT;
     const long tiles2 = (px2 + kPT - 1) / kPT * n_ctiles_groups;
-    return wg_tiles * kWideTileCost + narrow_rounds(tiles2, nk, may_cut) + ((n3 && tiles2) ? kSecondKernelCost : 0.0);
+    return wg_tiles * wide_cost + narrow_rounds(tiles2, nk, may_cut) + ((n3 && tiles2) ? kSecondKernelCost : 0.0);
   };
   const long rounds = full * n_ctiles_groups / grid;
   const long whole = rounds * grid / n_ctiles_groups;  // pixel tiles of the whole rounds
@@ -236,7 +240,8 @@ long wide_tiles(long total_px, int n_ctiles_groups, int nk, bool may_cut, bool a
 // ... for a launch of total_px pixels of the call *p
 long wide_tiles_of_call(const mdcn_params *p, const Geom &g, const Plan &pl, long total_px, bool out_vec_ok) {
   if (!wide_ok(p, g, pl) || !out_vec_ok) return 0;
-  return wide_tiles(total_px, pl.n_ctiles * g.G, pl.slabs * g.taps, pl.cut_bytes != 0, p->path == MDCN_PATH_FUSED_WIDE);
+  return wide_tiles(total_px, pl.n_ctiles * g.G, pl.slabs * g.taps, pl.cut_bytes != 0, p->path == MDCN_PATH_FUSED_WIDE,
+                    wide_tile_cost(pl.CT, g.sh == 1 && g.sw == 1));
 }
 
 int make_plan(const mdcn_params *p, const Geom &g, Plan *pl) {
@@ -403,12 +408,15 @@ hipError_t launch_fused2(const FusedArgs &fa, bool unbordered, hipStream_t st) {
   return hipGetLastError();
 }
 
-// 16-bit tensors, 256-channel tiles, whole tiles of 256 pixels: mdcn_fused3.h
+// 16-bit tensors, 256- or 128-channel tiles, whole tiles of 256 pixels: mdcn_fused3.h
 template <typename E>
-hipError_t launch_fused3(const FusedArgs &fa, hipStream_t st) {
+hipError_t launch_fused3(const FusedArgs &fa, int CT, hipStream_t st) {
   const int total_wg = fa.n_ptiles * fa.n_ctiles * fa.g.G;
   const int per_xcd = std::max(1, std::min((total_wg + 7) / 8, num_cus() / 8));
-  hipLaunchKernelGGL((fused3_kernel<E, 256>), dim3(per_xcd * 8), dim3(kF3Threads), 0, st, fa);
+  if (CT == 256)
+    hipLaunchKernelGGL((fused3_kernel<E, 256>), dim3(per_xcd * 8), dim3(kF3Threads), 0, st, fa);
+  else
+    hipLaunchKernelGGL((fused3_kernel<E, 128>), dim3(per_xcd * 8), dim3(kF3Threads), 0, st, fa);
   return hipGetLastError();
 }
 
@@ -649,7 +657,7 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
           if (n3 > 0) {
             FusedArgs fw = fa;
             fw.n_ptiles = (int)n3;
-            if (launch_fused3<E>(fw, st) != hipSuccess) rc = MDCN_ERR_LAUNCH;
+            if (launch_fused3<E>(fw, pl.CT, st) != hipSuccess) rc = MDCN_ERR_LAUNCH;
             fa.px0 = (int)(n3 * kF3PT);
             fa.n_ptiles = (int)((fa.total_px - fa.px0 + kPT - 1) / kPT);
             rest = fa.n_ptiles > 0;

@@ -212,6 +212,9 @@ WIDE = {
     'two_channel_tiles': dict(N=2, Cin=128, Cout=512, H=16, W=16),
     'stride2': dict(N=2, Cin=128, Cout=256, H=33, W=32, stride=2),
     'several_tiles_per_workgroup': dict(N=9, Cin=128, Cout=256, H=96, W=88),  # 297 tiles on 256 workgroups
+    'channel_tile_128': dict(N=2, Cin=128, Cout=128, H=24, W=24),           # the 128-channel variant of the tile
+    'channel_tile_128_two_groups': dict(N=3, Cin=256, Cout=256, H=16, W=24, groups=2, sigma=3.0),
+    'channel_tile_128_stride2': dict(N=2, Cin=256, Cout=128, H=31, W=32, stride=2, bias=False),
     'no_bias_k1x3': dict(N=2, Cin=512, Cout=256, H=16, W=24, k=(1, 3), padding=(0, 1), bias=False),  # 24 K steps
 }
 
