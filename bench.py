@@ -43,6 +43,8 @@ PEAK_TFLOPS = {'bf16': 2500.0, 'f16': 2500.0, 'f32': 157.3}
 HBM_PEAK_GBS = 8000.0
 # (workload, dominant kernel) -> (HBM bytes per launch from rocprofv3 counters, the profile they are in)
 TRAFFIC = {
+    ('cfg4', 'fused3_kernel<bf16>'): (335.0e6, 'profiles/fused3_kernel_bf16_cfg4.md (FETCH_SIZE 102 497.9 KiB x 2.00 '
+                                               '+ WRITE_SIZE 122 151.7 KiB x 1.00)'),
     ('cfg4', 'fused2_kernel<bf16>'): (422.0e6, 'profiles/fused2_kernel_bf16_cfg4.md (FETCH_SIZE 130 554.5 KiB x 2.00 '
                                                '+ WRITE_SIZE 150 981.9 KiB x 1.00)'),
 }
@@ -273,6 +275,9 @@ def main():
     ap.add_argument('--steps', type=int, default=200)
     ap.add_argument('--warmup', type=int, default=20)
     ap.add_argument('--workload', default='cfg4', choices=sorted(WORKLOADS) + ['cfg5'])
+    ap.add_argument('--path', default='auto', choices=['auto', 'narrow', 'wide'],
+                    help="forward kernels of the 16-bit fused path: the library's choice, the 128-pixel "
+                         'kernel only, or the 256-pixel kernel on every whole tile')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     ap.add_argument('--no-configs', action='store_true',
                     help='skip the short runs of the other benchmark configurations')
@@ -318,6 +323,7 @@ def main():
 
     assert torch.cuda.is_available(), 'bench.py needs a GPU'
     torch.cuda.set_device(0)
+    ext_module.set_path({'auto': 0, 'narrow': 5, 'wide': 4}[a.path])  # (MDCN_PATH_AUTO / _FUSED_NARROW / _FUSED_WIDE)
     wl = dict(WORKLOADS[a.workload])
     dname = wl.pop('dtype')
     dtype = {'bf16': torch.bfloat16, 'f16': torch.float16, 'f32': torch.float32}[dname]
@@ -412,9 +418,9 @@ def main():
     cp = capi.make_params({'f32': 0, 'f16': 1, 'bf16': 2}[dname], N, Cin, H, W, Cout, kh, kw, (sh, sw), (ph, pw),
                           (dh, dw), case['groups'], case['deform_groups'])
     cp.input, cp.offset, cp.mask, cp.weight, cp.bias, cp.output = (t.data_ptr() for t in (x, off, msk, w, b, out))
+    cp.path = ext_module.get_path()
     cws = torch.empty(lib.mdcn_workspace_bytes(ctypes.byref(cp)), dtype=torch.uint8, device='cuda')
     cp.workspace, cp.workspace_bytes = cws.data_ptr(), cws.numel()
-    cp.path = ext_module.get_path()
     kernels = lib.mdcn_forward_kernels(ctypes.byref(cp)).decode()  # what the library launches for this call
     cstream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
@@ -506,6 +512,7 @@ def main():
                          f'{H}x{W} k{kh}x{kw} s{sh} p{ph} d{dh} groups={case["groups"]} '
                          f'deform_groups={case["deform_groups"]}, offsets N(0,{wl["sigma"]}) px'),
             'entry': 'mmcv_amd._ext.modulated_deform_conv_forward',
+            'path': a.path,
             'flops_per_step': flops,
             'algorithmic_bytes_per_step': alg_bytes,
         },

@@ -586,10 +586,12 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("deformable_group"), py::arg("with_bias"));
   m.def("set_path", [](int path) {
           TORCH_CHECK(path >= MDCN_PATH_AUTO && path <= MDCN_PATH_FUSED_NARROW,
-                      "path must be 0 (auto), 1 (fused), 2 (direct) or 3 (fused, specialised-wave kernel only)");
+                      "path must be 0 (auto), 1 (fused), 2 (direct), 3 (fused, specialised-wave kernel only), "
+                      "4 (fused, 256-pixel kernel on every whole tile) or 5 (fused, without the 256-pixel kernel)");
           g_path.store(path);
         }, "choose the device path of forward and backward: 0 auto, 1 fused / matrix-core kernels, 2 direct kernels, "
-           "3 fused with the specialised-wave forward kernel", py::arg("path"));
+           "3 fused with the specialised-wave forward kernel, 4 fused with the 256-pixel forward kernel on every "
+           "whole tile, 5 fused without that kernel", py::arg("path"));
   m.def("get_path", []() { return g_path.load(); });
   m.def("set_k_split", [](bool on) { g_no_k_split.store(on ? 0 : 1); },
         "true (default): idle workgroups of the fused forward kernel's last round take parts of the K range of its "
