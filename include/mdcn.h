@@ -51,10 +51,13 @@ enum mdcn_path {
                                kernel that 16-bit 256-channel tiles get by default; for comparisons and tests */
   MDCN_PATH_FUSED_WIDE = 4, /* forward only: as MDCN_PATH_FUSED, and every whole tile of 256 pixels goes to the
                                kernel with 256-pixel tiles where the shape has one (16-bit tensors, one
-                               deformable group, 3 to 9 taps, 128 or a multiple of 256 output channels per group (2048 at most in all), an even
-                               number of K steps, output planes of a multiple of 8 and at least 64 pixels), however unevenly that fills the chip; MDCN_PATH_FUSED and
-                               MDCN_PATH_AUTO give that kernel whole rounds of tiles only and the rest of the
-                               pixels to the 128-pixel kernel.  Error if the shape has no such kernel. */
+                               deformable group, 3 to 9 taps, 128 or a multiple of 256 output channels per
+                               group (2048 at most in all), an even number of K steps, output planes of a
+                               multiple of 8 and at least 64 pixels; input dense or channels-last), however
+                               unevenly that fills the chip; MDCN_PATH_FUSED and MDCN_PATH_AUTO give that
+                               kernel all tiles or whole rounds of tiles, whichever its measured tile cost
+                               says is shorter, and the rest of the pixels to the 128-pixel kernel.  Error if
+                               the shape has no such kernel. */
   MDCN_PATH_FUSED_NARROW = 5 /* forward only: as MDCN_PATH_FUSED, never the 256-pixel kernel */
 };
 

@@ -183,11 +183,11 @@ bool uses_fused2(const mdcn_params *p, const Geom &g, const Plan &pl) {
   return nk_pad >= kF2MinSteps;
 }
 
-// ... and the kernel with 256-pixel tiles for whole tiles of such a call: bordered input copy, an even
+// ... and the kernel with 256-pixel tiles for whole tiles of such a call: an even
 // number of K steps, output planes of whole 16-byte runs (the caller checks the pointer's alignment), groups of
 // whole channel tiles
 bool wide_ok(const mdcn_params *p, const Geom &g, const Plan &pl) {
-  if (!pl.fused || !uses_fused2(p, g, pl) || p->input_nhwc || p->path == MDCN_PATH_FUSED_NARROW)
+  if (!pl.fused || !uses_fused2(p, g, pl) || p->path == MDCN_PATH_FUSED_NARROW)
     return false;
   const int nk = pl.slabs * g.taps;
   const long plane_out = (long)g.Ho * g.Wo;
@@ -410,13 +410,21 @@ hipError_t launch_fused2(const FusedArgs &fa, bool unbordered, hipStream_t st) {
 
 // 16-bit tensors, 256- or 128-channel tiles, whole tiles of 256 pixels: mdcn_fused3.h
 template <typename E>
-hipError_t launch_fused3(const FusedArgs &fa, int CT, hipStream_t st) {
+hipError_t launch_fused3(const FusedArgs &fa, int CT, bool nhwc, hipStream_t st) {
   const int total_wg = fa.n_ptiles * fa.n_ctiles * fa.g.G;
   const int per_xcd = std::max(1, std::min((total_wg + 7) / 8, num_cus() / 8));
-  if (CT == 256)
-    hipLaunchKernelGGL((fused3_kernel<E, 256>), dim3(per_xcd * 8), dim3(kF3Threads), 0, st, fa);
-  else
-    hipLaunchKernelGGL((fused3_kernel<E, 128>), dim3(per_xcd * 8), dim3(kF3Threads), 0, st, fa);
+  const dim3 grid(per_xcd * 8), block(kF3Threads);
+  if (CT == 256) {
+    if (nhwc)
+      hipLaunchKernelGGL((fused3_kernel<E, 256, true>), grid, block, 0, st, fa);
+    else
+      hipLaunchKernelGGL((fused3_kernel<E, 256, false>), grid, block, 0, st, fa);
+  } else {
+    if (nhwc)
+      hipLaunchKernelGGL((fused3_kernel<E, 128, true>), grid, block, 0, st, fa);
+    else
+      hipLaunchKernelGGL((fused3_kernel<E, 128, false>), grid, block, 0, st, fa);
+  }
   return hipGetLastError();
 }
 
@@ -657,7 +665,7 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
           if (n3 > 0) {
             FusedArgs fw = fa;
             fw.n_ptiles = (int)n3;
-            if (launch_fused3<E>(fw, pl.CT, st) != hipSuccess) rc = MDCN_ERR_LAUNCH;
+            if (launch_fused3<E>(fw, pl.CT, nhwc, st) != hipSuccess) rc = MDCN_ERR_LAUNCH;
             fa.px0 = (int)(n3 * kF3PT);
             fa.n_ptiles = (int)((fa.total_px - fa.px0 + kPT - 1) / kPT);
             rest = fa.n_ptiles > 0;

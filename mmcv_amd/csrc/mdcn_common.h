@@ -75,16 +75,18 @@ __device__ __forceinline__ TapSample make_tap_sample(int base_y, int base_x,
 // place in the block.  Positions outside (-1,H)x(-1,W) already have zero weights
 // and y0 = x0 = 0.
 __device__ __forceinline__ void clamp_to_image(TapSample &s, int H, int W) {
-  if (s.x0 < 0) {            // only the right column (x0 + 1 == 0) is inside: it becomes the left one
-    s.w00 = s.w01; s.w10 = s.w11; s.w01 = 0.0f; s.w11 = 0.0f; s.x0 = 0;
-  } else if (s.x0 > W - 2) { // only the left column (x0 == W - 1) is inside: it becomes the right one
-    s.w01 = s.w00; s.w11 = s.w10; s.w00 = 0.0f; s.w10 = 0.0f; s.x0 = W - 2;
-  }
-  if (s.y0 < 0) {
-    s.w00 = s.w10; s.w01 = s.w11; s.w10 = 0.0f; s.w11 = 0.0f; s.y0 = 0;
-  } else if (s.y0 > H - 2) {
-    s.w10 = s.w00; s.w11 = s.w01; s.w00 = 0.0f; s.w01 = 0.0f; s.y0 = H - 2;
-  }
+  // (selects on values, not conditional stores into the struct, which the compiler parks in scratch memory)
+  const bool xl = s.x0 < 0;        // only the right column (x0 + 1 == 0) is inside: it becomes the left one
+  const bool xr = s.x0 > W - 2;    // only the left column (x0 == W - 1) is inside: it becomes the right one
+  const float a00 = xl ? s.w01 : (xr ? 0.0f : s.w00), a01 = xl ? 0.0f : (xr ? s.w00 : s.w01);
+  const float a10 = xl ? s.w11 : (xr ? 0.0f : s.w10), a11 = xl ? 0.0f : (xr ? s.w10 : s.w11);
+  const int x0 = xl ? 0 : (xr ? W - 2 : s.x0);
+  const bool yu = s.y0 < 0, yd = s.y0 > H - 2;   // likewise the rows
+  const float b00 = yu ? a10 : (yd ? 0.0f : a00), b01 = yu ? a11 : (yd ? 0.0f : a01);
+  const float b10 = yu ? 0.0f : (yd ? a00 : a10), b11 = yu ? 0.0f : (yd ? a01 : a11);
+  const int y0 = yu ? 0 : (yd ? H - 2 : s.y0);
+  s.w00 = b00; s.w01 = b01; s.w10 = b10; s.w11 = b11;
+  s.x0 = x0; s.y0 = y0;
 }
 
 // Where the offsets and the mask of one output pixel live, in elements: image n,

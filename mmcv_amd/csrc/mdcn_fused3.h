@@ -1,5 +1,6 @@
 // Fused DCNv2 forward for gfx950, 16-bit tensors, tiles of 256 pixels x CT (256 or
-// 128) output channels, one deformable group, 3 to 9 taps, bordered input copy:
+// 128) output channels, one deformable group, 3 to 9 taps, bordered input copy
+// or a channels-last tensor read in place:
 // the implicit GEMM of mdcn_fused.h / mdcn_fused2.h with a tile twice as tall.
 //
 // Why another tile.  Per K step (128 bytes of channels of one tap) a tile of PT
@@ -82,6 +83,16 @@ constexpr size_t fused3_lds_bytes(int CT) {
                "global_load_dwordx4 %3, %4, %6 offset:128"                       \
                : "=&v"(d[0]), "=&v"(d[1]), "=&v"(d[2]), "=&v"(d[3])              \
                : "v"(voff), "s"(base), "s"(base_row))
+// ... from a channels-last tensor read in place: the right-hand corners are a whole pixel (all channels)
+// further on, at `base_r` / `base_row_r`
+#define MDCN_F3_GLOAD4_NHWC(d, voff, base, base_r, base_row, base_row_r)         \
+  asm volatile("s_nop 4\n\t"                                                     \
+               "global_load_dwordx4 %0, %4, %5\n\t"                              \
+               "global_load_dwordx4 %1, %4, %6\n\t"                              \
+               "global_load_dwordx4 %2, %4, %7\n\t"                              \
+               "global_load_dwordx4 %3, %4, %8"                                  \
+               : "=&v"(d[0]), "=&v"(d[1]), "=&v"(d[2]), "=&v"(d[3])              \
+               : "v"(voff), "s"(base), "s"(base_r), "s"(base_row), "s"(base_row_r))
 
 // Barrier of a step for the waves that copy weight tiles: all but N of the wave's loads have landed -- the
 // youngest direct-to-LDS copies among them, which the comment tells the build's scan of the assembly
@@ -110,7 +121,7 @@ __device__ __forceinline__ void f3_lgkmwait1(u32x4 &a) {
 // between the first branch and the end (a register that an asm-issued load is still
 // writing must never meet another copy of itself at a join, where the compiler would
 // be free to move it).
-template <typename E, int CT, bool LATE>
+template <typename E, int CT, bool LATE, bool UNBORDERED>
 __device__ __forceinline__ void fused3_role(const FusedArgs &a, const uint32_t lds_x, const uint32_t lds_w,
                                             uint32_t *tpix, uint2 *tws, E *bias_s, const int wave) {
   using TR = ElemTraits<E>;
@@ -166,6 +177,17 @@ __device__ __forceinline__ void fused3_role(const FusedArgs &a, const uint32_t l
   const uint32_t xwb = lds_x + (uint32_t)tile_chunk(pl + 8, ck) * 16u;
   const unsigned char *xt = uniform_ptr((const unsigned char *)a.xt);
   const unsigned char *xt_row = uniform_ptr((const unsigned char *)a.xt + a.row_bytes);
+  // (channels-last input read in place: the pixel to the right is a.px_bytes away, not 128 bytes)
+  const unsigned char *xt_r = uniform_ptr((const unsigned char *)a.xt + a.px_bytes);
+  const unsigned char *xt_row_r = uniform_ptr((const unsigned char *)a.xt + a.row_bytes + a.px_bytes);
+  // the four loads of one pixel
+#define MDCN_F3_GATHER(d, voff)                                                  \
+  do {                                                                           \
+    if constexpr (UNBORDERED)                                                    \
+      MDCN_F3_GLOAD4_NHWC(d, voff, xt, xt_r, xt_row, xt_row_r);                  \
+    else                                                                         \
+      MDCN_F3_GLOAD4(d, voff, xt, xt_row);                                       \
+  } while (0)
 
   // ---- consume role: 64 pixels x WCH channels
   const int wave_p = wave & 3, wave_c = wave >> 2;
@@ -226,7 +248,7 @@ __device__ __forceinline__ void fused3_role(const FusedArgs &a, const uint32_t l
     const int ti = tap / kw, tj = tap - ti * kw;
     TapSample sm = make_tap_sample(tb_ho * g.sh - g.ph + ti * g.dh, tb_wo * g.sw - g.pw + tj * g.dw, to_f32(dy),
                                    to_f32(dx), mask_value<E>(m, a.om.logit), g.H, g.W);
-    tpix[tap * PT + tb_pl] = (uint32_t)tb_n * a.img_bytes + corner_offset<false>(sm, g, a);
+    tpix[tap * PT + tb_pl] = (uint32_t)tb_n * a.img_bytes + corner_offset<UNBORDERED>(sm, g, a);
     tws[tap * PT + tb_pl] = make_uint2(TR::pack2(sm.w00, sm.w01), TR::pack2(sm.w10, sm.w11));
   };
   // where the offsets and the mask of pixel p live (tap 0)
@@ -355,7 +377,7 @@ __device__ __forceinline__ void fused3_role(const FusedArgs &a, const uint32_t l
       TapSample sm = make_tap_sample(tb_ho * g.sh - g.ph + ti * g.dh, tb_wo * g.sw - g.pw + tj * g.dw,
                                      to_f32(__builtin_bit_cast(E, by)), to_f32(__builtin_bit_cast(E, bx)),
                                      mask_value<E>(__builtin_bit_cast(E, bm), a.om.logit), g.H, g.W);
-      tpix[row * PT + tb_pl] = (uint32_t)tb_n * a.img_bytes + corner_offset<false>(sm, g, a);
+      tpix[row * PT + tb_pl] = (uint32_t)tb_n * a.img_bytes + corner_offset<UNBORDERED>(sm, g, a);
       tws[row * PT + tb_pl] = make_uint2(TR::pack2(sm.w00, sm.w01), TR::pack2(sm.w10, sm.w11));
     }
   };
@@ -376,7 +398,7 @@ __device__ __forceinline__ void fused3_role(const FusedArgs &a, const uint32_t l
     f3_vmwait4<VM>(gs[I][0], gs[I][1], gs[I][2], gs[I][3]);                                      \
     const u32x4 o_ = BL::run(gs[I], w_);                                                         \
     *(lds_u32x4_ptr)(uintptr_t)((((I) & 1) ? xwb : xwa) + (uint32_t)(((I) >> 1) * 16 * kRowB) + (XB) * kXTile) = o_; \
-    MDCN_F3_GLOAD4(gs[I], npc_, xt, xt_row);                                                     \
+    MDCN_F3_GATHER(gs[I], npc_);                                                                 \
   } while (0)
   // One produce block: blend the blend cursor's step, gather the gather cursor's.
 #define MDCN_F3_BLOCK(XB)                                                                        \
@@ -573,7 +595,7 @@ __device__ __forceinline__ void fused3_role(const FusedArgs &a, const uint32_t l
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const uint32_t o_ = tp_[8 * i] + add_;
-      MDCN_F3_GLOAD4(gs[i], o_, xt, xt_row);
+      MDCN_F3_GATHER(gs[i], o_);
     }
   }
   if constexpr (LATE) issue_weights(0);
@@ -596,7 +618,7 @@ __device__ __forceinline__ void fused3_role(const FusedArgs &a, const uint32_t l
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const uint32_t o_ = tp_[8 * i] + add_;
-      MDCN_F3_GLOAD4(gs[i], o_, xt, xt_row);
+      MDCN_F3_GATHER(gs[i], o_);
     }
   }
 #pragma unroll
@@ -627,9 +649,10 @@ __device__ __forceinline__ void fused3_role(const FusedArgs &a, const uint32_t l
 #undef MDCN_F3_NREADS
 #undef MDCN_F3_BLOCK
 #undef MDCN_F3_PIXEL
+#undef MDCN_F3_GATHER
 }
 
-template <typename E, int CT>
+template <typename E, int CT, bool UNBORDERED>
 __global__ __launch_bounds__(kF3Threads) void fused3_kernel(FusedArgs a) {
   __shared__ uint4 Xs[2][kF3PT * kRowChunks];      // sample tiles
   __shared__ uint4 Ws[2][CT * kRowChunks];         // weight tiles
@@ -644,10 +667,10 @@ __global__ __launch_bounds__(kF3Threads) void fused3_kernel(FusedArgs a) {
   const uint32_t lds_w = (uint32_t)(uintptr_t)(lptr_t)(&Ws[0][0]);
   if (wave >= 4) {
     MDCN_ROLE("late");
-    fused3_role<E, CT, true>(a, lds_x, lds_w, tpix, tws, bias_s, wave);
+    fused3_role<E, CT, true, UNBORDERED>(a, lds_x, lds_w, tpix, tws, bias_s, wave);
   } else {
     MDCN_ROLE("early");
-    fused3_role<E, CT, false>(a, lds_x, lds_w, tpix, tws, bias_s, wave);
+    fused3_role<E, CT, false, UNBORDERED>(a, lds_x, lds_w, tpix, tws, bias_s, wave);
   }
 }
 

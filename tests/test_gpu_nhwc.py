@@ -15,6 +15,10 @@ CASES = [
     ('c64_g2_dil2', dict(N=1, Cin=128, Cout=64, H=16, W=18, padding=2, dilation=2, groups=2, sigma=2.0)),
     ('c64_2x2_image', dict(N=3, Cin=64, Cout=32, H=2, W=2, sigma=1.0)),
     ('c256_5x5', dict(N=1, Cin=256, Cout=48, H=12, W=12, k=5, padding=2, sigma=2.0)),
+    # shapes with whole tiles of 256 pixels: the 256-pixel kernel reads the tensor in place as well
+    ('wide_c256', dict(N=2, Cin=256, Cout=256, H=24, W=24, sigma=3.0)),
+    ('wide_c128_far_offsets', dict(N=3, Cin=128, Cout=128, H=16, W=16, sigma=6.0)),
+    ('wide_s2_g2', dict(N=2, Cin=256, Cout=512, H=33, W=32, stride=2, groups=2, sigma=2.0)),
 ]
 DTYPES = [torch.float32, torch.bfloat16, torch.float16]
 
@@ -36,6 +40,18 @@ def test_in_place_channels_last_against_oracle(name, kw, dtype):
     print(f'  {name} {dtype}: vs oracle {err:.2e}, vs bordered-copy path {both:.2e}', flush=True)
     assert err <= TOL[dtype]
     assert both <= TOL[dtype] * 0.1
+    if name.startswith('wide') and dtype != torch.float32:
+        import ctypes
+        N, Cin, H, W = case['input'].shape
+        Cout, _, kh, kw = case['weight'].shape
+        p = capi.make_params(capi.MDCN_BF16, N, Cin, H, W, Cout, kh, kw, case['stride'], case['padding'],
+                             case['dilation'], case['groups'], case['deform_groups'], capi.PATH_FUSED_WIDE)
+        p.input_nhwc = 1
+        p.input = dev['input'].data_ptr()
+        assert capi.load().mdcn_forward_kernels(ctypes.byref(p)).decode().startswith('fused3_kernel')
+        y_wide = capi_forward(dict(dev, input_nhwc=True), path=capi.PATH_FUSED_WIDE, unsplit=True)
+        y_narrow = capi_forward(dict(dev, input_nhwc=True), path=capi.PATH_FUSED_NARROW, unsplit=True)
+        assert torch.equal(y_wide, y_narrow)   # the two kernels sum a tile's K range in the same order
 
 
 def test_extension_takes_channels_last_tensors_in_place():
