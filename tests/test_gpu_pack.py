@@ -25,6 +25,9 @@ CASES = [
     ('c64_5x5_d3_s2_big_patch', dict(N=1, Cin=64, Cout=32, H=30, W=41, k=5, padding=6, dilation=3, stride=2)),
     ('c16_direct', dict(N=2, Cin=16, Cout=24, H=9, W=10)),
     ('c20_direct_dg2_s2', dict(N=1, Cin=20, Cout=10, H=12, W=9, stride=2, deform_groups=2)),
+    # whole tiles of 256 pixels: the 256-pixel kernel reads offsets and mask logits from the raw tensor
+    ('c128_wide_tiles', dict(N=2, Cin=128, Cout=128, H=24, W=24)),
+    ('c256_wide_tiles', dict(N=1, Cin=256, Cout=256, H=16, W=32)),
 ]
 DTYPES = [torch.float32, torch.bfloat16, torch.float16]
 
