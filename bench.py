@@ -145,6 +145,29 @@ CFG5_STAGES = [('c3', 128, 4, (200, 336), (100, 168)),
                ('c5', 512, 3, (50, 84), (25, 42))]
 
 
+SETTLE_CALLS = 100   # calls between the first timed loop of a configuration and its second one
+
+
+def time_calls(fn, warmup, steps, settle=0):
+    """ms per call of `steps` calls after `warmup` untimed ones; with `settle`, also of `steps` more calls
+    after that many further untimed ones (a card that idled a moment ago -- a CPU leg, tensor set-up -- runs
+    its first tens of calls at lower clocks): (first, settled or None)."""
+    import torch
+    res = []
+    for pre in ([warmup] if not settle else [warmup, settle]):
+        for _ in range(pre):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        res.append(e0.elapsed_time(e1) / steps)
+    return res[0], (res[1] if settle else None)
+
+
 def cfg5_layers():
     """The 13 deformable 3x3 convs: (name, C, (Hin, Win), stride)."""
     layers = []
@@ -187,20 +210,15 @@ def run_cfg5(a):
             pack = lambda: layer(x)   # one extension call: conv_offset + split + sigmoid + DCN
             t = []
             for fn in (producer, dcn, pack):
-                for _ in range(a.warmup):
-                    fn()
-                torch.cuda.synchronize()
-                e0, e1 = ev(), ev()
-                e0.record()
-                for _ in range(a.steps):
-                    fn()
-                e1.record()
-                torch.cuda.synchronize()
-                t.append(e0.elapsed_time(e1) / a.steps)
+                first, settled = time_calls(fn, a.warmup, a.steps, SETTLE_CALLS if fn is dcn else 0)
+                t.append(first)
+                if fn is dcn:
+                    dcn_settled = settled
         flops = 2.0 * N * Ho * Wo * C * C * 9
         rows.append({'layer': name, 'C': C, 'in': [H, W], 'stride': stride,
                      'producer_ms': round(t[0], 4), 'dcn_ms': round(t[1], 4),
-                     'dcn_TFLOPs': round(flops / t[1] / 1e9, 1), 'pack_fused_ms': round(t[2], 4)})
+                     'dcn_TFLOPs': round(flops / t[1] / 1e9, 1), 'dcn_ms_settled': round(dcn_settled, 4),
+                     'pack_fused_ms': round(t[2], 4)})
         if getattr(a, 'parity', False) and name.endswith('.1'):
             # one layer per stage: first and last sample of the op's output against the CPU path
             dcn()
@@ -244,20 +262,17 @@ def quick_config(name, steps, warmup, parity=False):
                   dilation_h=dh, dilation_w=dw, group=case['groups'],
                   deformable_group=case['deform_groups'], with_bias=True)
     fn = lambda: ext_module.modulated_deform_conv_forward(x, w, b, empty, off, msk, out, empty, **kwargs)
-    for _ in range(warmup):
-        fn()
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(steps):
-        fn()
-    e1.record()
-    torch.cuda.synchronize()
-    ms = e0.elapsed_time(e1) / steps
+    ms, ms_settled = time_calls(fn, warmup, steps, SETTLE_CALLS)
     flops = 2.0 * N * Ho * Wo * Cout * cin_g * kh * kw
     tf = flops / ms / 1e9
+    tf_settled = flops / ms_settled / 1e9
     rec = {'dtype': dname, 'ms_per_layer': round(ms, 4), 'TFLOPs': round(tf, 2),
-           'pct_matrix_peak': round(100.0 * tf / PEAK_TFLOPS[dname], 2), 'steps': steps, 'warmup': warmup}
+           'pct_matrix_peak': round(100.0 * tf / PEAK_TFLOPS[dname], 2), 'steps': steps, 'warmup': warmup,
+           # the same loop again after SETTLE_CALLS more calls: the configuration's tensors were set up on
+           # the host a moment ago, and the first loop runs on a card that is still raising its clocks
+           'settled': {'ms_per_layer': round(ms_settled, 4), 'TFLOPs': round(tf_settled, 2),
+                       'pct_matrix_peak': round(100.0 * tf_settled / PEAK_TFLOPS[dname], 2),
+                       'after_calls': warmup + steps + SETTLE_CALLS}}
     if parity:
         seen = dict(case)
         for k in ('input', 'offset', 'mask', 'weight', 'bias'):
@@ -316,6 +331,7 @@ def main():
             'pct_mfma_peak': round(100.0 * tot_flops / tot_dcn / 1e9 / PEAK_TFLOPS['bf16'], 2),
             'offset_mask_producer_ms': round(tot_prod, 4),
             'summed_ms_with_producer': round(tot_dcn + tot_prod, 4),
+            'summed_ms_settled': round(sum(r['dcn_ms_settled'] for r in rows), 4),
             'summed_ms_pack_fused': round(tot_pack, 4), 'layers': rows}), flush=True)
         return
     from common import make_case, cast_case
@@ -396,6 +412,11 @@ def main():
                           'pct_matrix_peak': round(100.0 * tot_flops / tot_dcn / 1e9 / PEAK_TFLOPS['bf16'], 2),
                           'summed_ms_pack_fused': round(tot_pack, 4), 'steps': a5.steps, 'warmup': a5.warmup,
                           'per_layer_ms': {r['layer']: r['dcn_ms'] for r in rows},
+                          # each layer's loop again after SETTLE_CALLS more calls (see quick_config)
+                          'settled': {'summed_ms': round(sum(r['dcn_ms_settled'] for r in rows), 4),
+                                      'pct_matrix_peak': round(100.0 * tot_flops / sum(r['dcn_ms_settled'] for r in rows)
+                                                               / 1e9 / PEAK_TFLOPS['bf16'], 2),
+                                      'per_layer_ms': {r['layer']: r['dcn_ms_settled'] for r in rows}},
                           'parity': {r['layer']: r['parity'] for r in rows if 'parity' in r}}
 
     # ---- 4. the same call on four rotating sets of buffers and through the bare C ABI (these legs also keep
