@@ -528,10 +528,10 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
     uint32_t *cut_cnt = (uint32_t *)((unsigned char *)cut_part + align_up((size_t)pl.cut_wgs * kPT * kF2CT * 4));
     if (!pl.cut_bytes) cut_part = nullptr, cut_cnt = nullptr;
 
-    // weights: once per call -- inside the launch that re-lays the first batch chunk when the
-    // input allows the vector re-layout (whole 16-byte runs per channel row), else on their own
+    // weights: once per call -- inside the launch that re-lays the first batch chunk; on their own when
+    // there is no such launch (channels-last input read in place)
     constexpr int EPV = 16 / (int)sizeof(E);
-    const bool vec_relayout = !p->input_nhwc && ((g.H * g.W) % EPV == 0) && (((uintptr_t)p->input % 16) == 0);
+    const bool vec_relayout = !p->input_nhwc;
     const long wtotal = (long)g.G * pl.n_ctiles * pl.slabs * g.taps * pl.CT * pl.KC;
     bool packed = false;
     {
@@ -572,17 +572,6 @@ int run_typed(const mdcn_params *p, const Geom &g, const Plan &pl, hipStream_t s
           hipLaunchKernelGGL((relayout_vec_kernel<E, true>), dim3((unsigned)blocks), dim3(256), 0, st, gc, in, xt,
                              n_pchunks);
         }
-        if (hipGetLastError() != hipSuccess) rc = MDCN_ERR_LAUNCH;
-        toc(0);
-      } else if (!nhwc) {
-        // runs of 128 pixels of the image plane
-        const int n_pchunks = (gc.H * gc.W + 127) / 128;
-        const long blocks = (long)gc.N * (gc.Cin / pl.KC) * n_pchunks;
-        // 16-bit pixels are read two at a time when every channel plane starts word aligned
-        const int words_ok = ((gc.H * gc.W) % 2 == 0) && (((uintptr_t)in % 4) == 0);
-        tic();
-        hipLaunchKernelGGL(relayout_kernel<E>, dim3((unsigned)blocks), dim3(256), 0, st, gc, in,
-                           xt, n_pchunks, words_ok);
         if (hipGetLastError() != hipSuccess) rc = MDCN_ERR_LAUNCH;
         toc(0);
       }

@@ -767,7 +767,10 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
       int ctile, grp, p0;
       decode(t, ctile, grp, p0);
       E *out = (E *)a.out;
-      const bool vec_ok = a.out_vec_ok != 0;
+      // A run of 8 pixels of one channel is one 16-byte store wherever it lies in one image; planes that are
+      // not whole 16-byte runs (25 x 42 pixels, say) make such a store start at any even or odd pixel, which
+      // global memory takes (unaligned access mode).  Only runs across the end of an image go pixel by pixel.
+      typedef u32x4 u32x4_any __attribute__((aligned(2)));
       const int pw0 = p0 + wave_p * 64;
       // image and pixel-in-image of the wave's first pixel; the runs below step on from there
       const int n0 = pw0 / plane_out;
@@ -781,8 +784,8 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
           ++n;
         }
         E *dst = out + ((long)n * g.Cout + cbase) * plane_out + rem;
-        if (vec_ok && p + 8 <= total_px) {  // (rows of 8 never straddle images then)
-          *(u32x4 *)dst = val;
+        if (p + 8 <= total_px && rem + 8 <= plane_out) {
+          *(u32x4_any *)dst = val;
         } else {
 #pragma unroll
           for (int i = 0; i < 8; ++i) {
@@ -800,7 +803,7 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
         }
       };
       // the common case: the wave's 64 pixels lie in one image and every run is one 16-byte store
-      const bool plain = vec_ok && pw0 + 64 <= total_px && rem0 + 64 <= plane_out;
+      const bool plain = pw0 + 64 <= total_px && rem0 + 64 <= plane_out;
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
         const int col = ctile * CT + wave_c * WCH + mb * 32 + frow;
@@ -824,7 +827,7 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
             u32x4 val;
             val.x = s0[0]; val.y = s1[0]; val.z = s0[1]; val.w = s1[1];
             if (plain) {
-              if (col_ok) *(u32x4 *)(row + nb * 32 + 16 * g2) = val;
+              if (col_ok) *(u32x4_any *)(row + nb * 32 + 16 * g2) = val;
             } else if (col_ok) {
               store_run(cbase, nb * 32 + 8 * (fhalf ? gb : ga), val);
             }

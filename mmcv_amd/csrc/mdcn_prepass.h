@@ -103,9 +103,11 @@ __global__ __launch_bounds__(256) void relayout_kernel(Geom g, const E *__restri
       *(uint4 *)(dst_slab + ((long)(g.Hp - 1) * g.Wp) * 128 + (long)i * 16) = zero;
 }
 
-// The same re-layout without LDS, for planes whose channel rows can be read 16
-// bytes at a time (H * W a multiple of 16 / sizeof(E) and a 16-byte aligned
-// tensor).  A thread owns EPV = 16 / sizeof(E) consecutive pixels x EPV
+// The same re-layout without LDS: channel rows are read 16 bytes at a time, at
+// whatever alignment the plane size and the tensor give them (global memory takes
+// unaligned accesses; only the last, partial run of a plane whose size is not a
+// multiple of the run is read element by element, so that nothing past the
+// tensor is touched).  A thread owns EPV = 16 / sizeof(E) consecutive pixels x EPV
 // consecutive channels: EPV loads of 16 bytes (one channel each), a transpose in
 // registers (16-bit elements: one v_perm_b32 per output word; fp32: none, the
 // words only change names) and EPV stores of 16 bytes (one pixel each).  Eight
@@ -131,11 +133,23 @@ __device__ __forceinline__ void relayout_vec_block(const Geom &g, const E *__res
   unsigned char *dst_slab =
       (unsigned char *)xt + (((long)n * slabs_total + slab) * (BORDER ? (long)g.Hp * g.Wp : (long)plane)) * 128;
   const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
-  if (p0 < plane) {  // (plane is a multiple of EPV: the whole run is inside)
+  if (p0 < plane) {
+    const int np = min(EPV, plane - p0);  // pixels of the run that exist
     const E *src = in + ((long)n * g.Cin + slab * KC + cg * EPV) * plane + p0;
+    typedef uint4 uint4_any __attribute__((aligned(2)));  // (2: the smallest element)
     uint4 r[EPV];
+    if (np == EPV) {
 #pragma unroll
-    for (int j = 0; j < EPV; ++j) r[j] = *(const uint4 *)(src + (long)j * plane);
+      for (int j = 0; j < EPV; ++j) r[j] = *(const uint4_any *)(src + (long)j * plane);
+    } else {
+#pragma unroll
+      for (int j = 0; j < EPV; ++j) {
+        E e[EPV];
+#pragma unroll
+        for (int i = 0; i < EPV; ++i) e[i] = i < np ? src[(long)j * plane + i] : from_f32<E>(0.0f);
+        __builtin_memcpy(&r[j], e, 16);
+      }
+    }
     uint4 o[EPV];
     if constexpr (sizeof(E) == 2) {
       // r[j] = 8 pixels of channel j; o[i] = 8 channels of pixel i
@@ -161,6 +175,7 @@ __device__ __forceinline__ void relayout_vec_block(const Geom &g, const E *__res
     int x = p0 - y * g.W;
 #pragma unroll
     for (int i = 0; i < EPV; ++i) {
+      if (i >= np) break;
       unsigned char *d = dst_slab + (BORDER ? (long)(y + 1) * g.Wp + (x + 1) : (long)(p0 + i)) * 128 + cg * 16;
       *(uint4 *)d = o[i];
       if (BORDER && x == g.W - 1) {
@@ -197,11 +212,15 @@ __device__ __forceinline__ void pack_weight_elems(const Geom &g, const E *__rest
                                                   int KC, int n_ctiles, int slabs, long total, long first,
                                                   long stride, uint32_t *__restrict__ zero_ptr, int zero_n) {
   for (long i = first; i < zero_n; i += stride) zero_ptr[i] = 0u;
+  // one 16-byte run of a row (EPV consecutive input channels of one output channel and tap) per step: the
+  // index arithmetic is paid once per run and the store is whole
+  constexpr int EPV = 16 / (int)sizeof(E);
   const int nk = slabs * g.taps;
-  for (long idx = first; idx < total; idx += stride) {
+  const int runs = KC / EPV;
+  for (long idx = first; idx < total / EPV; idx += stride) {
     long r = idx;
-    const int kc = (int)(r % KC);
-    r /= KC;
+    const int kc = (int)(r % runs) * EPV;
+    r /= runs;
     const int row = (int)(r % CT);
     r /= CT;
     const int ks = (int)(r % nk);
@@ -210,13 +229,19 @@ __device__ __forceinline__ void pack_weight_elems(const Geom &g, const E *__rest
     const int grp = (int)(r / n_ctiles);
     const int slab = ks / g.taps, tap = ks % g.taps;
     const int col = ctile * CT + row;  // output channel within the group
-    E v = from_f32<E>(0.0f);
+    E v[EPV];
     if (col < g.cout_g) {
       const int co = grp * g.cout_g + col;
-      const int cl = slab * KC + kc;
-      v = w[((long)co * g.cin_g + cl) * g.taps + tap];
+      const E *src = w + ((long)co * g.cin_g + slab * KC + kc) * g.taps + tap;
+#pragma unroll
+      for (int i = 0; i < EPV; ++i) v[i] = src[(long)i * g.taps];
+    } else {
+#pragma unroll
+      for (int i = 0; i < EPV; ++i) v[i] = from_f32<E>(0.0f);
     }
-    wp[idx] = v;
+    uint4 o;
+    __builtin_memcpy(&o, v, 16);
+    *(uint4 *)(wp + idx * EPV) = o;
   }
 }
 
