@@ -903,11 +903,11 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
   }
 
   if (gemm || wgemm) {
-    {  // zero-bordered pixel-major copy of the input
-      const int n_pchunks = (g.H * g.W + 127) / 128;
-      const int words_ok = ((g.H * g.W) % 2 == 0) && (((uintptr_t)p->input % 4) == 0);
-      hipLaunchKernelGGL(relayout_kernel<E>, dim3((unsigned)((long)g.N * (g.Cin / KC) * n_pchunks)),
-                         dim3(256), 0, st, g, (const E *)p->input, (E *)xt, n_pchunks, words_ok);
+    {  // zero-bordered copy of the input in 32-byte records (what the scatter kernel reads per corner)
+      constexpr int EPV = 16 / (int)sizeof(E);
+      const int n_pchunks = (g.H * g.W + 32 * EPV - 1) / (32 * EPV);
+      hipLaunchKernelGGL((relayout_vec_kernel<E, true, 32>), dim3((unsigned)((long)g.N * (g.Cin / KC) * n_pchunks)),
+                         dim3(256), 0, st, g, (const E *)p->input, (E *)xt, n_pchunks);
       check();
     }
     if (gemm) {  // pixel-major grad_output, transposed weights

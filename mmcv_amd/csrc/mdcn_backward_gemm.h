@@ -288,7 +288,7 @@ constexpr int kScTW = 32;
 
 struct BwdScatterArgs {
   Geom g;
-  const void *xt;  // zero-bordered pixel-major input copy [N][Cin / KC][H + 2][W + 2][KC]
+  const void *xt;  // zero-bordered input copy in 32-byte records [N][Cin / RC][H + 2][W + 2][RC], RC = 32 bytes of channels
   OffMaskView om;
   const void *D;   // column gradient of the pass, layout of ColGradArgs::D; null: columns only
   float *gin32;
@@ -338,7 +338,8 @@ __global__ __launch_bounds__(256) void combine_parts_kernel(const float *__restr
 // weight-gradient product; with a.D == null that is all it does.
 template <typename E, int CH, typename WT>
 __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
-  constexpr int KC = 128 / (int)sizeof(E);
+  constexpr int RC = 32 / (int)sizeof(E);   // channels per record of the input copy
+  static_assert(CH <= RC && RC % CH == 0, "a pass reads a record or a whole fraction of one");
   constexpr bool kFixed = sizeof(WT) == 4;
   static_assert(kScTH * kScTW == 256, "one thread per pixel of the tile");
   static_assert(kScTH * kScTW * kBwdTapsMax <= kScMaxAdds, "bound on the adds per window entry");
@@ -401,7 +402,7 @@ __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
     }
     const E *dbase = (const E *)a.D + (((long)nl * (g.Cin / 16) + (c0 >> 4)) * g.taps) * plane_out * 16 + pix * 16 +
                      (c0 & 15);
-    const E *xbase = (const E *)a.xt + (((long)n * (g.Cin / KC) + c0 / KC) * slab_px) * KC + (c0 % KC);
+    const E *xbase = (const E *)a.xt + (((long)n * (g.Cin / RC) + c0 / RC) * slab_px) * RC + (c0 % RC);
     // row of the columns matrix of channel c0 at tap 0 (a chunk stays inside one group)
     const int grp = c0 / g.cin_g;
     E *cbase = (E *)a.col + (((long)nl * g.Cin + (long)grp * g.cin_g) * g.taps + (c0 - grp * g.cin_g)) * a.P_pad + pix;
@@ -427,12 +428,12 @@ __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
           const bool ok00 = y0 >= 0 && x0 >= 0, ok01 = y0 >= 0 && x1 <= g.W - 1;
           const bool ok10 = y1 <= g.H - 1 && x0 >= 0, ok11 = y1 <= g.H - 1 && x1 <= g.W - 1;
           // corners outside the image read the copy's zero border
-          const E *xp = xbase + ((long)(y0 + 1) * g.Wp + (x0 + 1)) * KC;
+          const E *xp = xbase + ((long)(y0 + 1) * g.Wp + (x0 + 1)) * RC;
           VecCh<E, CH> r00, r01, r10, r11;
           r00.load(xp);
-          r01.load(xp + KC);
-          r10.load(xp + (long)g.Wp * KC);
-          r11.load(xp + (long)(g.Wp + 1) * KC);
+          r01.load(xp + RC);
+          r10.load(xp + (long)g.Wp * RC);
+          r11.load(xp + (long)(g.Wp + 1) * RC);
           float v00[CH], v01[CH], v10[CH], v11[CH];
           r00.unpack(v00);
           r01.unpack(v01);

@@ -115,9 +115,14 @@ __global__ __launch_bounds__(256) void relayout_kernel(Geom g, const E *__restri
 // instruction reads 128 contiguous bytes per channel and a store instruction
 // writes whole 128-byte pixels.  One block = 32 pixel runs x 8 channel groups:
 // one slab of 32 * EPV pixels.  Borders as in relayout_kernel.
-template <typename E, bool BORDER>
+// REC = 32 writes the copy in records of 32 bytes instead of 128: [N][Cin/RC][H+2][W+2][RC] with RC = 32 bytes
+// of channels, i.e. each 128-byte slab as four planes -- for a reader that takes 32 bytes of a pixel at a
+// time and whose neighbouring lanes read neighbouring pixels (the backward's scatter kernel): four pixels
+// share a cache line there, where the 128-byte records give every lane a line of its own.
+template <typename E, bool BORDER, int REC = 128>
 __device__ __forceinline__ void relayout_vec_block(const Geom &g, const E *__restrict__ in, E *__restrict__ xt,
                                                    int n_pchunks, int b) {
+  static_assert(REC == 128 || REC == 32, "whole slabs or quarters of them");
   constexpr int EPV = 16 / (int)sizeof(E);
   constexpr int KC = 128 / (int)sizeof(E);
   constexpr int PXB = 32 * EPV;  // pixels per block
@@ -130,8 +135,10 @@ __device__ __forceinline__ void relayout_vec_block(const Geom &g, const E *__res
   const int cg = tid & 7, pg = tid >> 3;
   const int plane = g.H * g.W;
   const int p0 = pc * PXB + pg * EPV;
-  unsigned char *dst_slab =
-      (unsigned char *)xt + (((long)n * slabs_total + slab) * (BORDER ? (long)g.Hp * g.Wp : (long)plane)) * 128;
+  const long plane_px = BORDER ? (long)g.Hp * g.Wp : (long)plane;   // pixels of a plane of the copy
+  unsigned char *dst_slab = (unsigned char *)xt + (((long)n * slabs_total + slab) * plane_px) * 128;
+  // where this thread's 16 bytes of pixel 0 go
+  unsigned char *dst_cg = REC == 128 ? dst_slab + cg * 16 : dst_slab + (long)(cg >> 1) * plane_px * 32 + (cg & 1) * 16;
   const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
   if (p0 < plane) {
     const int np = min(EPV, plane - p0);  // pixels of the run that exist
@@ -176,11 +183,11 @@ __device__ __forceinline__ void relayout_vec_block(const Geom &g, const E *__res
 #pragma unroll
     for (int i = 0; i < EPV; ++i) {
       if (i >= np) break;
-      unsigned char *d = dst_slab + (BORDER ? (long)(y + 1) * g.Wp + (x + 1) : (long)(p0 + i)) * 128 + cg * 16;
+      unsigned char *d = dst_cg + (BORDER ? (long)(y + 1) * g.Wp + (x + 1) : (long)(p0 + i)) * REC;
       *(uint4 *)d = o[i];
       if (BORDER && x == g.W - 1) {
-        *(uint4 *)(d + 128) = zero;
-        *(uint4 *)(d + 256) = zero;
+        *(uint4 *)(d + REC) = zero;
+        *(uint4 *)(d + 2 * REC) = zero;
       }
       if (++x == g.W) {
         x = 0;
@@ -189,17 +196,24 @@ __device__ __forceinline__ void relayout_vec_block(const Geom &g, const E *__res
     }
   }
   if (!BORDER) return;
-  if (pc == 0)  // top border row and the left border pixel of the first image row
-    for (int i = tid; i < (g.Wp + 1) * 8; i += 256) *(uint4 *)(dst_slab + (long)i * 16) = zero;
-  if (pc == n_pchunks - 1)  // bottom border row
-    for (int i = tid; i < g.Wp * 8; i += 256)
-      *(uint4 *)(dst_slab + ((long)(g.Hp - 1) * g.Wp) * 128 + (long)i * 16) = zero;
+  constexpr int NPL = 128 / REC;       // planes of the copy per slab
+  constexpr int QPP = REC / 16;        // 16-byte pieces per pixel of a plane
+  if (pc == 0) {  // top border row and the left border pixel of the first image row
+    const int per = (g.Wp + 1) * QPP;
+    for (int i = tid; i < per * NPL; i += 256)
+      *(uint4 *)(dst_slab + (long)(i / per) * plane_px * REC + (long)(i % per) * 16) = zero;
+  }
+  if (pc == n_pchunks - 1) {  // bottom border row
+    const int per = g.Wp * QPP;
+    for (int i = tid; i < per * NPL; i += 256)
+      *(uint4 *)(dst_slab + (long)(i / per) * plane_px * REC + ((long)(g.Hp - 1) * g.Wp) * REC + (long)(i % per) * 16) = zero;
+  }
 }
 
-template <typename E, bool BORDER = true>
+template <typename E, bool BORDER = true, int REC = 128>
 __global__ __launch_bounds__(256) void relayout_vec_kernel(Geom g, const E *__restrict__ in, E *__restrict__ xt,
                                                            int n_pchunks) {
-  relayout_vec_block<E, BORDER>(g, in, xt, n_pchunks, (int)blockIdx.x);
+  relayout_vec_block<E, BORDER, REC>(g, in, xt, n_pchunks, (int)blockIdx.x);
 }
 
 // weight[Cout][Cin/G][kh][kw] -> wp[G][n_ctiles][nk][CT][KC]: for every
