@@ -332,7 +332,12 @@ __global__ __launch_bounds__(256) void combine_parts_kernel(const float *__restr
 // cannot overflow, and one contribution is rounded to B * 2^-19 at worst -- two
 // thousand times finer than the bf16/fp16 rounding of the result.  Integer sums
 // are exact, so the window part of grad_input does not depend on the order of
-// the adds.
+// the adds.  Two channels share one 64-bit entry (ds_add_u64 costs 14 clocks
+// where two ds_add_u32 cost 22): the even channel's value sign-extended plus the
+// odd channel's shifted up by 32 bits; the low half's borrows and carries into
+// the high half cancel when the entry is taken apart again (low = the entry's low
+// word as a signed number, high = (entry - low) >> 32), since neither sum leaves
+// 32 bits.
 // With a.col the kernel also stores the forward's columns (mask * bilinear
 // sample, rounded to E as the reference's columns tensor is) for the
 // weight-gradient product; with a.D == null that is all it does.
@@ -340,10 +345,11 @@ template <typename E, int CH, typename WT>
 __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
   constexpr int RC = 32 / (int)sizeof(E);   // channels per record of the input copy
   static_assert(CH <= RC && RC % CH == 0, "a pass reads a record or a whole fraction of one");
+  static_assert(CH % 2 == 0, "fixed-point window entries hold two channels");
   constexpr bool kFixed = sizeof(WT) == 4;
   static_assert(kScTH * kScTW == 256, "one thread per pixel of the tile");
   static_assert(kScTH * kScTW * kBwdTapsMax <= kScMaxAdds, "bound on the adds per window entry");
-  __shared__ WT win[kScWindowBytes / sizeof(WT)];
+  __shared__ __align__(16) WT win[kScWindowBytes / sizeof(WT)];
   float fx_scale = 1.0f, fx_inv = 1.0f;
   if (kFixed && a.D != nullptr) {
     const float bound = __uint_as_float(*a.dmax) * (a.mmax ? __uint_as_float(*a.mmax) : 1.0f) * (float)kScMaxAdds;
@@ -397,7 +403,7 @@ __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
   for (int c0 = c_begin; c0 < c_end; c0 += CH) {
     if (data) {
       __syncthreads();  // the previous chunk's flush is done
-      for (int i = tid; i < win_px * CH; i += 256) win[i] = (WT)0;
+      for (int i = tid; i < win_px * CH; i += 256) win[i] = (WT)0;   // (fixed point: CH / 2 entries of 64 bits per pixel)
       __syncthreads();
     }
     const E *dbase = (const E *)a.D + (((long)nl * (g.Cin / 16) + (c0 >> 4)) * g.taps) * plane_out * 16 + pix * 16 +
@@ -456,6 +462,8 @@ __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
             const int wbase = ry * a.WW + rx;  // window is [channel][WH][WW]: neighbouring pixels, neighbouring banks
             const long o00 = (long)y0 * g.W + x0, o01 = o00 + 1, o10 = o00 + g.W, o11 = o10 + 1;
             float am = 0.0f, ay = 0.0f, ax = 0.0f;
+            // fixed point: the even channel's four contributions wait here for the odd channel's
+            int q00 = 0, q01 = 0, q10 = 0, q11 = 0;
 #pragma unroll
             for (int cc = 0; cc < CH; ++cc) {
               const float dc = d[cc];
@@ -464,14 +472,24 @@ __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
               ax += dc * (hy * (v01[cc] - v00[cc]) + ly * (v11[cc] - v10[cc]));
               const float t = dc * m;
               if (in_win) {
-                WT *wp = win + cc * win_px + wbase;
                 if constexpr (kFixed) {
                   const float ts = t * fx_scale;
-                  if (ok00) atomicAdd(wp, __float2int_rn(w00 * ts));
-                  if (ok01) atomicAdd(wp + 1, __float2int_rn(w01 * ts));
-                  if (ok10) atomicAdd(wp + a.WW, __float2int_rn(w10 * ts));
-                  if (ok11) atomicAdd(wp + a.WW + 1, __float2int_rn(w11 * ts));
+                  const int r00 = __float2int_rn(w00 * ts), r01 = __float2int_rn(w01 * ts);
+                  const int r10 = __float2int_rn(w10 * ts), r11 = __float2int_rn(w11 * ts);
+                  if ((cc & 1) == 0) {
+                    q00 = r00, q01 = r01, q10 = r10, q11 = r11;
+                  } else {
+                    unsigned long long *wp = (unsigned long long *)win + (cc >> 1) * win_px + wbase;
+                    auto both = [](int lo, int hi) {
+                      return (unsigned long long)((long long)lo + (long long)((unsigned long long)(unsigned)hi << 32));
+                    };
+                    if (ok00) atomicAdd(wp, both(q00, r00));
+                    if (ok01) atomicAdd(wp + 1, both(q01, r01));
+                    if (ok10) atomicAdd(wp + a.WW, both(q10, r10));
+                    if (ok11) atomicAdd(wp + a.WW + 1, both(q11, r11));
+                  }
                 } else {
+                  WT *wp = win + cc * win_px + wbase;
                   if (ok00) atomicAdd(wp, (WT)(w00 * t));
                   if (ok01) atomicAdd(wp + 1, (WT)(w01 * t));
                   if (ok10) atomicAdd(wp + a.WW, (WT)(w10 * t));
@@ -497,12 +515,28 @@ __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
     }
     if (data) {
       __syncthreads();  // every add into the window has landed
-      for (int i = tid; i < win_px * CH; i += 256) {
-        const float v = kFixed ? (float)win[i] * fx_inv : (float)win[i];
-        if (v != 0.0f) {
-          const int cc = i / win_px, q = i - cc * win_px;
-          const int y = wy0 + q / a.WW, x = wx0 + q % a.WW;  // in the image: only valid corners were added
-          unsafeAtomicAdd(a.gin32 + ((long)n * g.Cin + c0 + cc) * plane_in + (long)y * g.W + x, v);
+      if constexpr (kFixed) {
+        const long long *w64 = (const long long *)win;
+        for (int i = tid; i < win_px * (CH / 2); i += 256) {
+          const long long e = w64[i];
+          if (e != 0) {
+            const int lo = (int)(unsigned)(unsigned long long)e;
+            const int hi = (int)((e - (long long)lo) >> 32);
+            const int cp = i / win_px, q = i - cp * win_px;
+            const int y = wy0 + q / a.WW, x = wx0 + q % a.WW;  // in the image: only valid corners were added
+            float *gi = a.gin32 + ((long)n * g.Cin + c0 + 2 * cp) * plane_in + (long)y * g.W + x;
+            if (lo != 0) unsafeAtomicAdd(gi, (float)lo * fx_inv);
+            if (hi != 0) unsafeAtomicAdd(gi + plane_in, (float)hi * fx_inv);
+          }
+        }
+      } else {
+        for (int i = tid; i < win_px * CH; i += 256) {
+          const float v = (float)win[i];
+          if (v != 0.0f) {
+            const int cc = i / win_px, q = i - cc * win_px;
+            const int y = wy0 + q / a.WW, x = wx0 + q % a.WW;  // in the image: only valid corners were added
+            unsafeAtomicAdd(a.gin32 + ((long)n * g.Cin + c0 + cc) * plane_in + (long)y * g.W + x, v);
+          }
         }
       }
     }
