@@ -915,10 +915,10 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
       gg.Cin = g.Cout;
       gg.H = g.Ho;
       gg.W = g.Wo;
-      const int o_pchunks = (int)((plane_out + 127) / 128);
-      const int o_words_ok = (plane_out % 2 == 0) && (((uintptr_t)bp->grad_output % 4) == 0);
-      hipLaunchKernelGGL((relayout_kernel<E, false>), dim3((unsigned)((long)g.N * (g.Cout / KC) * o_pchunks)),
-                         dim3(256), 0, st, gg, (const E *)bp->grad_output, (E *)gT, o_pchunks, o_words_ok);
+      constexpr int EPV = 16 / (int)sizeof(E);
+      const int o_pchunks = (int)((plane_out + 32 * EPV - 1) / (32 * EPV));
+      hipLaunchKernelGGL((relayout_vec_kernel<E, false>), dim3((unsigned)((long)g.N * (g.Cout / KC) * o_pchunks)),
+                         dim3(256), 0, st, gg, (const E *)bp->grad_output, (E *)gT, o_pchunks);
       check();
       if (pl.mx_bytes) {
         hipLaunchKernelGGL(fill_zero_kernel<uint32_t>, dim3(1), dim3(256), 0, st, maxima, 2L);

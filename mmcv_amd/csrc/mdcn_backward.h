@@ -25,15 +25,32 @@ namespace mdcn {
 
 template <typename T>
 __global__ __launch_bounds__(256) void fill_zero_kernel(T *p, long n) {
-  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
-    p[i] = (T)0;
+  // 16 bytes per thread and step where the buffer starts aligned (workspace regions do), the rest one by one
+  const long first = (long)blockIdx.x * blockDim.x + threadIdx.x, stride = (long)gridDim.x * blockDim.x;
+  constexpr long PER = 16 / (long)sizeof(T);
+  const long nv = ((uintptr_t)p % 16 == 0) ? n / PER : 0;
+  for (long i = first; i < nv; i += stride) ((uint4 *)p)[i] = make_uint4(0u, 0u, 0u, 0u);
+  for (long i = nv * PER + first; i < n; i += stride) p[i] = (T)0;
 }
 
 template <typename E>
 __global__ __launch_bounds__(256) void round_kernel(const float *__restrict__ src, E *__restrict__ dst,
                                                     long n) {
-  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
-    dst[i] = from_f32<E>(src[i]);
+  // eight elements per thread and step (two 16-byte loads; the store lands wherever the caller's tensor
+  // starts: global memory takes unaligned accesses), the rest one by one
+  const long first = (long)blockIdx.x * blockDim.x + threadIdx.x, stride = (long)gridDim.x * blockDim.x;
+  typedef float4 float4_a4 __attribute__((aligned(4)));
+  struct Out8 { E v[8]; };
+  typedef Out8 Out8_any __attribute__((aligned(2)));
+  const long nv = n / 8;
+  for (long i = first; i < nv; i += stride) {
+    const float4 a = ((const float4_a4 *)src)[2 * i], b = ((const float4_a4 *)src)[2 * i + 1];
+    Out8 o;
+    o.v[0] = from_f32<E>(a.x); o.v[1] = from_f32<E>(a.y); o.v[2] = from_f32<E>(a.z); o.v[3] = from_f32<E>(a.w);
+    o.v[4] = from_f32<E>(b.x); o.v[5] = from_f32<E>(b.y); o.v[6] = from_f32<E>(b.z); o.v[7] = from_f32<E>(b.w);
+    ((Out8_any *)dst)[i] = o;
+  }
+  for (long i = nv * 8 + first; i < n; i += stride) dst[i] = from_f32<E>(src[i]);
 }
 
 // Pixels of one image a block of bwd_bias_kernel sums.

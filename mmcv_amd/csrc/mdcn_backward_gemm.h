@@ -14,7 +14,7 @@
 // store the forward's columns, from which grad_weight is a second plain product
 // (bwd_wgrad_kernel).
 // Both operands of the product are pixel-major / K-contiguous copies written by
-// small pre-passes (relayout_kernel<E, false> for grad_output,
+// small pre-passes (relayout_vec_kernel<E, false> for grad_output,
 // pack_weight_t_kernel for the weights).
 #pragma once
 

@@ -10,100 +10,15 @@ namespace mdcn {
 // every bilinear corner of an in-range position a plain load: a corner outside
 // the image reads a stored zero, which is exactly the per-corner rule of the
 // reference sampler (mmcv/ops/csrc/pytorch/cpu/modulated_deform_conv.cpp:17-27).
-//
-// One block moves one slab of 128 consecutive pixels of the image plane (rows
-// run on into each other, so every block but the last of a plane is full
-// whatever W is) through LDS.  Reads run along the plane in 32-bit words (two
-// 16-bit pixels or one fp32 pixel; a wave takes 256 contiguous bytes of one
-// channel), writes are 16 bytes per lane, 128 per pixel.  The pixel that ends an
-// image row also zeroes the two border pixels that follow it in the copy (right
-// border of its row, left border of the next); the first block of a plane
-// zeroes the top border row and the pixel after it, the last one the bottom row.
+// Image rows run on into each other in the flattened plane, so every block but
+// the last of a plane is full whatever W is.  The pixel that ends an image row
+// also zeroes the two border pixels that follow it in the copy (right border of
+// its row, left border of the next); the first block of a plane zeroes the top
+// border row and the pixel after it, the last one the bottom row.
 // BORDER = false writes the plain pixel-major copy [N][Cin/KC][H*W][KC] instead
 // (the backward's pixel-major grad_output).
-template <typename E, bool BORDER = true>
-__global__ __launch_bounds__(256) void relayout_kernel(Geom g, const E *__restrict__ in,
-                                                       E *__restrict__ xt, int n_pchunks,
-                                                       int words_ok) {
-  constexpr int KC = 128 / (int)sizeof(E);
-  constexpr int EPW = 4 / (int)sizeof(E);   // elements per 32-bit word
-  constexpr int ROWW = 33;                  // LDS words per pixel: 128 bytes + 4 of padding
-  __shared__ uint32_t tile[128 * ROWW];
-
-  int b = blockIdx.x;
-  const int pc = b % n_pchunks;
-  b /= n_pchunks;
-  const int slabs_total = g.Cin / KC;
-  const int slab = b % slabs_total;
-  const int n = b / slabs_total;
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int plane = g.H * g.W;
-  const int p0 = pc * 128;
-
-  {
-    const E *src_slab = in + ((long)n * g.Cin + slab * KC) * plane;
-    // 64 segments (KC channels x 128/(64*EPW) parts of the pixel run), 16 per wave
-#pragma unroll 4
-    for (int it = 0; it < 16; ++it) {
-      const int seg = wave + 4 * it;
-      const int c = seg % KC;
-      const int part = seg / KC;                      // fp32: two halves of 64 pixels
-      const int lp = (part * 64 + lane) * EPW;        // first local pixel of the word
-      const int p = p0 + lp;
-      const E *src = src_slab + (long)c * plane + p;
-      if (EPW == 2) {
-        uint32_t word = 0;
-        if (words_ok) {
-          if (p < plane) word = *(const uint32_t *)src;  // plane even: p + 1 < plane too
-        } else {
-          uint32_t lo = 0, hi = 0;
-          if (p < plane) lo = *(const uint16_t *)src;
-          if (p + 1 < plane) hi = *((const uint16_t *)src + 1);
-          word = lo | (hi << 16);
-        }
-        uint16_t *t16 = (uint16_t *)tile;
-        t16[lp * (ROWW * 2) + c] = (uint16_t)(word & 0xffffu);
-        t16[(lp + 1) * (ROWW * 2) + c] = (uint16_t)(word >> 16);
-      } else {
-        uint32_t word = 0;
-        if (p < plane) word = *(const uint32_t *)src;
-        tile[lp * ROWW + c] = word;
-      }
-    }
-  }
-  __syncthreads();
-  unsigned char *dst_slab =
-      (unsigned char *)xt + (((long)n * slabs_total + slab) * (BORDER ? (long)g.Hp * g.Wp : (long)plane)) * 128;
-  const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
-#pragma unroll
-  for (int it = 0; it < 4; ++it) {
-    const int u = tid + 256 * it;
-    const int lp = u >> 3, q = u & 7;
-    const int p = p0 + lp;
-    if (p < plane) {
-      const int y = p / g.W;
-      const int x = p - y * g.W;
-      const uint32_t *t = tile + lp * ROWW + q * 4;
-      unsigned char *d = dst_slab + (BORDER ? (long)(y + 1) * g.Wp + (x + 1) : (long)p) * 128 + q * 16;
-      *(uint4 *)d = make_uint4(t[0], t[1], t[2], t[3]);
-      if (BORDER && x == g.W - 1) {
-        *(uint4 *)(d + 128) = zero;
-        *(uint4 *)(d + 256) = zero;
-      }
-    }
-  }
-  if (!BORDER) return;
-  if (pc == 0)  // top border row and the left border pixel of the first image row
-    for (int i = tid; i < (g.Wp + 1) * 8; i += 256) *(uint4 *)(dst_slab + (long)i * 16) = zero;
-  if (pc == n_pchunks - 1)  // bottom border row
-    for (int i = tid; i < g.Wp * 8; i += 256)
-      *(uint4 *)(dst_slab + ((long)(g.Hp - 1) * g.Wp) * 128 + (long)i * 16) = zero;
-}
-
-// The same re-layout without LDS: channel rows are read 16 bytes at a time, at
+//
+// No LDS: channel rows are read 16 bytes at a time, at
 // whatever alignment the plane size and the tensor give them (global memory takes
 // unaligned accesses; only the last, partial run of a plane whose size is not a
 // multiple of the run is read element by element, so that nothing past the
@@ -114,7 +29,7 @@ __global__ __launch_bounds__(256) void relayout_kernel(Geom g, const E *__restri
 // neighbouring lanes hold the eight channel groups of a pixel run, so a load
 // instruction reads 128 contiguous bytes per channel and a store instruction
 // writes whole 128-byte pixels.  One block = 32 pixel runs x 8 channel groups:
-// one slab of 32 * EPV pixels.  Borders as in relayout_kernel.
+// one slab of 32 * EPV pixels.
 // REC = 32 writes the copy in records of 32 bytes instead of 128: [N][Cin/RC][H+2][W+2][RC] with RC = 32 bytes
 // of channels, i.e. each 128-byte slab as four planes -- for a reader that takes 32 bytes of a pixel at a
 // time and whose neighbouring lanes read neighbouring pixels (the backward's scatter kernel): four pixels
