@@ -201,12 +201,30 @@ __global__ __launch_bounds__(TILE * 2, TILE == 128 ? 2 : 1) void bwd_colgrad_ker
     for (int nb = 0; nb < 2; ++nb) {
       const int px = pt * TILE + wn * 64 + nb * 32 + frow;
       if (px >= a.P) continue;
+      // The two halves of the wave exchange their 4-channel groups so that a lane holds 8 consecutive
+      // channels: one 16-byte store per lane and 16 channels, 32 pixels x 32 bytes contiguous per instruction
+      // (the lower half takes the first 8 channels of a 16-channel chunk, the upper half the second 8).
+      if constexpr (sizeof(E) == 2) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int c = cb + j * 8 + fhalf * 4;
-        E *dst = D + ((((long)nl * chunks + (c >> 4)) * a.taps + tap) * a.P + px) * 16 + (c & 15);
-        TR::store4((unsigned char *)dst, acc[mb][nb][4 * j], acc[mb][nb][4 * j + 1],
-                   acc[mb][nb][4 * j + 2], acc[mb][nb][4 * j + 3]);
+        for (int jp = 0; jp < 2; ++jp) {
+          const f32x16 &c16 = acc[mb][nb];
+          const int ja = 2 * jp, jb = 2 * jp + 1;
+          const uint32_t a0 = TR::pack2(c16[4 * ja], c16[4 * ja + 1]), a1 = TR::pack2(c16[4 * ja + 2], c16[4 * ja + 3]);
+          const uint32_t b0 = TR::pack2(c16[4 * jb], c16[4 * jb + 1]), b1 = TR::pack2(c16[4 * jb + 2], c16[4 * jb + 3]);
+          const auto s0 = __builtin_amdgcn_permlane32_swap(a0, b0, false, false);
+          const auto s1 = __builtin_amdgcn_permlane32_swap(a1, b1, false, false);
+          const int c = cb + jp * 16 + fhalf * 8;
+          E *dst = D + ((((long)nl * chunks + (c >> 4)) * a.taps + tap) * a.P + px) * 16 + (c & 15);
+          *(uint4 *)dst = make_uint4(s0[0], s1[0], s0[1], s1[1]);
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int c = cb + j * 8 + fhalf * 4;
+          E *dst = D + ((((long)nl * chunks + (c >> 4)) * a.taps + tap) * a.P + px) * 16 + (c & 15);
+          TR::store4((unsigned char *)dst, acc[mb][nb][4 * j], acc[mb][nb][4 * j + 1],
+                     acc[mb][nb][4 * j + 2], acc[mb][nb][4 * j + 3]);
+        }
       }
     }
   }
