@@ -894,11 +894,11 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
   const bool gemm = pl.gemm;
 
   if (bp->grad_input) {
-    hipLaunchKernelGGL(fill_zero_kernel<float>, dim3(blocks_for(n_in)), dim3(256), 0, st, gin32, n_in);
+    hipLaunchKernelGGL(fill_zero_kernel<float>, dim3(blocks_for(n_in / 4 + 1)), dim3(256), 0, st, gin32, n_in);  // (16 bytes per thread)
     check();
   }
   if (bp->grad_weight) {
-    hipLaunchKernelGGL(fill_zero_kernel<float>, dim3(blocks_for(n_w)), dim3(256), 0, st, gw32, n_w);
+    hipLaunchKernelGGL(fill_zero_kernel<float>, dim3(blocks_for(n_w / 4 + 1)), dim3(256), 0, st, gw32, n_w);
     check();
   }
 
@@ -1091,7 +1091,7 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
       check();
     }
     if (pl.gin_bytes) {
-      hipLaunchKernelGGL(round_kernel<E>, dim3(blocks_for(n_in)), dim3(256), 0, st, gin32,
+      hipLaunchKernelGGL(round_kernel<E>, dim3(blocks_for(n_in / 8 + 1)), dim3(256), 0, st, gin32,  // (8 elements per thread)
                          (E *)bp->grad_input, n_in);
       check();
     }
@@ -1116,7 +1116,7 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
       check();
     }
     if (pl.gw_bytes) {
-      hipLaunchKernelGGL(round_kernel<E>, dim3(blocks_for(n_w)), dim3(256), 0, st, gw32,
+      hipLaunchKernelGGL(round_kernel<E>, dim3(blocks_for(n_w / 8 + 1)), dim3(256), 0, st, gw32,
                          (E *)bp->grad_weight, n_w);
       check();
     }
