@@ -55,8 +55,11 @@ __device__ __forceinline__ void relayout_vec_block(const Geom &g, const E *__res
   // where this thread's 16 bytes of pixel 0 go
   unsigned char *dst_cg = REC == 128 ? dst_slab + cg * 16 : dst_slab + (long)(cg >> 1) * plane_px * 32 + (cg & 1) * 16;
   const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+  uint4 o[EPV];    // o[i] = this thread's EPV channels of pixel p0 + i
+#pragma unroll
+  for (int i = 0; i < EPV; ++i) o[i] = zero;
+  const int np = max(0, min(EPV, plane - p0));  // pixels of the run that exist
   if (p0 < plane) {
-    const int np = min(EPV, plane - p0);  // pixels of the run that exist
     const E *src = in + ((long)n * g.Cin + slab * KC + cg * EPV) * plane + p0;
     typedef uint4 uint4_any __attribute__((aligned(2)));  // (2: the smallest element)
     uint4 r[EPV];
@@ -72,7 +75,6 @@ __device__ __forceinline__ void relayout_vec_block(const Geom &g, const E *__res
         __builtin_memcpy(&r[j], e, 16);
       }
     }
-    uint4 o[EPV];
     if constexpr (sizeof(E) == 2) {
       // r[j] = 8 pixels of channel j; o[i] = 8 channels of pixel i
       const uint32_t *rw = (const uint32_t *)r;
@@ -93,6 +95,8 @@ __device__ __forceinline__ void relayout_vec_block(const Geom &g, const E *__res
 #pragma unroll
         for (int i = 0; i < 4; ++i) ow[i * 4 + j] = rw[j * 4 + i];
     }
+  }
+  if constexpr (REC == 128) {
     int y = p0 / g.W;
     int x = p0 - y * g.W;
 #pragma unroll
@@ -107,6 +111,52 @@ __device__ __forceinline__ void relayout_vec_block(const Geom &g, const E *__res
       if (++x == g.W) {
         x = 0;
         ++y;
+      }
+    }
+  } else {
+    // 32-byte records: a store instruction of the wave would write its eight runs' pixel i, 256 bytes apart
+    // each.  The runs of four neighbouring lanes groups (lane bits 4 and 5) first trade pixels with each
+    // other (register bits 0 and 1 against those lane bits), after which register i holds, across these
+    // lanes, four consecutive pixels: 128 contiguous bytes per plane and instruction.
+#pragma unroll
+    for (int i = 0; i < EPV; ++i) {
+      if ((i & 2) == 0) {
+        uint32_t *lo = (uint32_t *)&o[i], *hi = (uint32_t *)&o[i | 2];
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          const auto sw = __builtin_amdgcn_permlane32_swap(lo[w], hi[w], false, false);
+          lo[w] = sw[0];
+          hi[w] = sw[1];
+        }
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < EPV; ++i) {
+      if ((i & 1) == 0) {
+        uint32_t *lo = (uint32_t *)&o[i], *hi = (uint32_t *)&o[i | 1];
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          const auto sw = __builtin_amdgcn_permlane16_swap(lo[w], hi[w], false, false);
+          lo[w] = sw[0];
+          hi[w] = sw[1];
+        }
+      }
+    }
+    // register i now holds pixel src_i of the run of lane group src_pg
+    const int b5 = (pg >> 2) & 1, b4 = (pg >> 1) & 1;
+#pragma unroll
+    for (int i = 0; i < EPV; ++i) {
+      const int src_pg = (pg & ~6) | (((i >> 1) & 1) << 2) | ((i & 1) << 1);
+      const int src_i = (i & ~3) | (b5 << 1) | b4;
+      const int q = pc * PXB + src_pg * EPV + src_i;
+      if (q < plane) {
+        const int y = q / g.W, x = q - y * g.W;
+        unsigned char *d = dst_cg + (BORDER ? (long)(y + 1) * g.Wp + (x + 1) : (long)q) * REC;
+        *(uint4 *)d = o[i];
+        if (BORDER && x == g.W - 1) {
+          *(uint4 *)(d + REC) = zero;
+          *(uint4 *)(d + 2 * REC) = zero;
+        }
       }
     }
   }
