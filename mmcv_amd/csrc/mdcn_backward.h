@@ -39,16 +39,15 @@ __global__ __launch_bounds__(256) void round_kernel(const float *__restrict__ sr
   // eight elements per thread and step (two 16-byte loads; the store lands wherever the caller's tensor
   // starts: global memory takes unaligned accesses), the rest one by one
   const long first = (long)blockIdx.x * blockDim.x + threadIdx.x, stride = (long)gridDim.x * blockDim.x;
-  typedef float4 float4_a4 __attribute__((aligned(4)));
+  struct In4 { float x, y, z, w; };   // (four floats with the alignment of one)
   struct Out8 { E v[8]; };
-  typedef Out8 Out8_any __attribute__((aligned(2)));
   const long nv = n / 8;
   for (long i = first; i < nv; i += stride) {
-    const float4 a = ((const float4_a4 *)src)[2 * i], b = ((const float4_a4 *)src)[2 * i + 1];
+    const In4 a = ((const In4 *)src)[2 * i], b = ((const In4 *)src)[2 * i + 1];
     Out8 o;
     o.v[0] = from_f32<E>(a.x); o.v[1] = from_f32<E>(a.y); o.v[2] = from_f32<E>(a.z); o.v[3] = from_f32<E>(a.w);
     o.v[4] = from_f32<E>(b.x); o.v[5] = from_f32<E>(b.y); o.v[6] = from_f32<E>(b.z); o.v[7] = from_f32<E>(b.w);
-    ((Out8_any *)dst)[i] = o;
+    __builtin_memcpy(dst + 8 * i, &o, sizeof(o));
   }
   for (long i = nv * 8 + first; i < n; i += stride) dst[i] = from_f32<E>(src[i]);
 }

@@ -770,7 +770,6 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
       // A run of 8 pixels of one channel is one 16-byte store wherever it lies in one image; planes that are
       // not whole 16-byte runs (25 x 42 pixels, say) make such a store start at any even or odd pixel, which
       // global memory takes (unaligned access mode).  Only runs across the end of an image go pixel by pixel.
-      typedef u32x4 u32x4_any __attribute__((aligned(2)));
       const int pw0 = p0 + wave_p * 64;
       // image and pixel-in-image of the wave's first pixel; the runs below step on from there
       const int n0 = pw0 / plane_out;
@@ -785,7 +784,7 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
         }
         E *dst = out + ((long)n * g.Cout + cbase) * plane_out + rem;
         if (p + 8 <= total_px && rem + 8 <= plane_out) {
-          *(u32x4_any *)dst = val;
+          __builtin_memcpy(dst, &val, 16);
         } else {
 #pragma unroll
           for (int i = 0; i < 8; ++i) {
@@ -827,7 +826,7 @@ __global__ __launch_bounds__(kF2Threads) void fused2_kernel(FusedArgs a) {
             u32x4 val;
             val.x = s0[0]; val.y = s1[0]; val.z = s0[1]; val.w = s1[1];
             if (plain) {
-              if (col_ok) *(u32x4_any *)(row + nb * 32 + 16 * g2) = val;
+              if (col_ok) __builtin_memcpy(row + nb * 32 + 16 * g2, &val, 16);
             } else if (col_ok) {
               store_run(cbase, nb * 32 + 8 * (fhalf ? gb : ga), val);
             }

@@ -61,11 +61,10 @@ __device__ __forceinline__ void relayout_vec_block(const Geom &g, const E *__res
   const int np = max(0, min(EPV, plane - p0));  // pixels of the run that exist
   if (p0 < plane) {
     const E *src = in + ((long)n * g.Cin + slab * KC + cg * EPV) * plane + p0;
-    typedef uint4 uint4_any __attribute__((aligned(2)));  // (2: the smallest element)
     uint4 r[EPV];
-    if (np == EPV) {
+    if (np == EPV) {  // (16 bytes at the alignment of an element: one load instruction all the same)
 #pragma unroll
-      for (int j = 0; j < EPV; ++j) r[j] = *(const uint4_any *)(src + (long)j * plane);
+      for (int j = 0; j < EPV; ++j) __builtin_memcpy(&r[j], src + (long)j * plane, 16);
     } else {
 #pragma unroll
       for (int j = 0; j < EPV; ++j) {
