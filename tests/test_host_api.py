@@ -483,3 +483,17 @@ def test_built_library_passes_the_assembly_scans():
     assert m
     shifted = text[:m.start(1)] + str(int(m.group(1)) + 1) + text[m.end(1):]
     assert len(asm_check.wait_count_findings(shifted)) >= 1
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU: --gpus above 1 ends with a message and exit status 2 before anything
+    touches a device."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, 'bench.py'), '--gpus', '2'], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode == 2
+    assert 'ONE GPU' in r.stderr
+    assert r.stdout.strip() == ''
