@@ -818,7 +818,8 @@ void make_bwd_plan(const mdcn_bwd_params *bp, const Geom &g, BwdPlan *pl) {
   const long s_tiles = (long)g.N * g.DG * ((g.Ho + kScTH - 1) / kScTH) * ((g.Wo + kScTW - 1) / kScTW);
   const bool mfma_ok = g.Cin % KC == 0 && g.cout_g % KC == 0 && g.cin_g % 32 == 0 &&
                        g.ch_per_dg % pl->sCH == 0 && pl->sR >= 1 && (s_tiles >= 64 || forced) &&
-                       d_img <= kBwdColGradCap && plane_out <= ((size_t)1 << 30);
+                       d_img <= kBwdColGradCap && plane_out <= ((size_t)1 << 30) &&
+                       (size_t)g.H * g.W <= ((size_t)1 << 30);  // (plane offsets held in 32 bits)
   if (mfma_ok) {
     pl->gemm = bp->grad_input != nullptr;
     pl->wgemm = bp->grad_weight != nullptr;
@@ -1055,11 +1056,11 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
   if (bp->grad_input) {
     if (gemm) {
       if (pl.parts > 1) {
-        hipLaunchKernelGGL(combine_parts_kernel<E>, dim3(blocks_for(off_total)), dim3(256), 0, st, poff,
+        hipLaunchKernelGGL(combine_parts_kernel<E>, dim3(blocks_for(off_total / 4 + 1)), dim3(256), 0, st, poff,
                            (E *)bp->grad_offset, off_total, pl.parts);
         check();
         if (bp->grad_mask) {
-          hipLaunchKernelGGL(combine_parts_kernel<E>, dim3(blocks_for(mask_total)), dim3(256), 0, st, pmask,
+          hipLaunchKernelGGL(combine_parts_kernel<E>, dim3(blocks_for(mask_total / 4 + 1)), dim3(256), 0, st, pmask,
                              (E *)bp->grad_mask, mask_total, pl.parts);
           check();
         }

@@ -62,7 +62,7 @@ template <typename E>
 __global__ __launch_bounds__(256) void bwd_bias_kernel(Geom g, const E *__restrict__ gout,
                                                        float *__restrict__ gbias32, int runs_per_image,
                                                        int splits) {
-  __shared__ float part[256];
+  __shared__ float part[4];
   const int co = blockIdx.x;
   const long plane = (long)g.Ho * g.Wo;
   const long work = (long)g.N * runs_per_image;
@@ -75,24 +75,32 @@ __global__ __launch_bounds__(256) void bwd_bias_kernel(Geom g, const E *__restri
     constexpr int EPV = 16 / (int)sizeof(E);  // elements per 16-byte load
     if (plane % EPV == 0 && ((uintptr_t)gout % 16) == 0) {  // (runs start at multiples of kBiasRun)
       const long nv = (p1 - p0) / EPV;
-      for (long v = threadIdx.x; v < nv; v += 256) {
-        const uint4 q = *(const uint4 *)(row + p0 + v * EPV);
-        const E *e = (const E *)&q;
+      const uint4 *src = (const uint4 *)(row + p0);
+      // four loads in flight per thread: a run is a handful of loads deep, so their latency is the cost
+      for (long v0 = 0; v0 < nv; v0 += 4 * 256) {
+        uint4 q[4];
 #pragma unroll
-        for (int i = 0; i < EPV; ++i) s += to_f32(e[i]);
+        for (int u = 0; u < 4; ++u) {
+          const long v = v0 + u * 256 + threadIdx.x;
+          q[u] = v < nv ? src[v] : make_uint4(0u, 0u, 0u, 0u);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const E *e = (const E *)&q[u];
+#pragma unroll
+          for (int i = 0; i < EPV; ++i) s += to_f32(e[i]);
+        }
       }
       for (long p = p0 + nv * EPV + threadIdx.x; p < p1; p += 256) s += to_f32(row[p]);
     } else {
       for (long p = p0 + threadIdx.x; p < p1; p += 256) s += to_f32(row[p]);
     }
   }
-  part[threadIdx.x] = s;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
   __syncthreads();
-  for (int w = 128; w > 0; w >>= 1) {
-    if ((int)threadIdx.x < w) part[threadIdx.x] += part[threadIdx.x + w];
-    __syncthreads();
-  }
-  if (threadIdx.x == 0) unsafeAtomicAdd(gbias32 + co, part[0]);
+  if (threadIdx.x == 0) unsafeAtomicAdd(gbias32 + co, (part[0] + part[1]) + (part[2] + part[3]));
 }
 
 // Channels whose column gradient a thread of bwd_data_kernel holds at a time.

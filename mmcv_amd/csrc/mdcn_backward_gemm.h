@@ -330,11 +330,25 @@ struct BwdScatterArgs {
   const uint32_t *dmax, *mmax;
 };
 
-// out[i] = sum over parts of part[p][i], rounded once.
+// out[i] = sum over parts of part[p][i], rounded once.  Four elements per thread
+// and step where the parts start at multiples of 16 bytes (total a multiple of 4).
 template <typename E>
 __global__ __launch_bounds__(256) void combine_parts_kernel(const float *__restrict__ part, E *__restrict__ out,
                                                             long total, int parts) {
-  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+  const long first = (long)blockIdx.x * blockDim.x + threadIdx.x, stride = (long)gridDim.x * blockDim.x;
+  const long nv = (total % 4 == 0 && (uintptr_t)part % 16 == 0) ? total / 4 : 0;
+  struct Out4 { E v[4]; };
+  for (long i = first; i < nv; i += stride) {
+    float4 s = ((const float4 *)part)[i];
+    for (int p = 1; p < parts; ++p) {
+      const float4 t = ((const float4 *)(part + (long)p * total))[i];
+      s.x += t.x; s.y += t.y; s.z += t.z; s.w += t.w;
+    }
+    Out4 o;
+    o.v[0] = from_f32<E>(s.x); o.v[1] = from_f32<E>(s.y); o.v[2] = from_f32<E>(s.z); o.v[3] = from_f32<E>(s.w);
+    __builtin_memcpy(out + 4 * i, &o, sizeof(o));
+  }
+  for (long i = nv * 4 + first; i < total; i += stride) {
     float s = 0.0f;
     for (int p = 0; p < parts; ++p) s += part[(long)p * total + i];
     out[i] = from_f32<E>(s);
@@ -418,12 +432,23 @@ __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
   const int part = blockIdx.y;
   const int ch_per_part = g.ch_per_dg / a.parts;
   const int c_begin = dgi * g.ch_per_dg + part * ch_per_part, c_end = c_begin + ch_per_part;
+
+  // Window pixels this thread flushes (tid, tid + 256, ...) as offsets into an image plane, the same
+  // in every pass; -1 for one outside the image or past the window (it only ever receives zeros).
+  constexpr int NE = kFixed ? CH / 2 : CH;  // window entries per pixel
+  constexpr int kSlots = (kScWindowBytes / (NE * 8) + 255) / 256;
+  int flush_at[kSlots];
+#pragma unroll
+  for (int j = 0; j < kSlots; ++j) {
+    const int q = tid + 256 * j;
+    const int y = wy0 + q / a.WW, x = wx0 + q % a.WW;
+    flush_at[j] = (q < win_px && y >= 0 && y < g.H && x >= 0 && x < g.W) ? y * g.W + x : -1;
+  }
+  if (data)  // the flush leaves the window zeroed for the next pass
+    for (int i = tid; i < kScWindowBytes / 16; i += 256) ((uint4 *)win)[i] = make_uint4(0u, 0u, 0u, 0u);
+
   for (int c0 = c_begin; c0 < c_end; c0 += CH) {
-    if (data) {
-      __syncthreads();  // the previous chunk's flush is done
-      for (int i = tid; i < win_px * CH; i += 256) win[i] = (WT)0;   // (fixed point: CH / 2 entries of 64 bits per pixel)
-      __syncthreads();
-    }
+    if (data) __syncthreads();  // the window is zero: first fill or the previous pass's flush
     const E *dbase = (const E *)a.D + (((long)nl * (g.Cin / 16) + (c0 >> 4)) * g.taps) * plane_out * 16 + pix * 16 +
                      (c0 & 15);
     const E *xbase = (const E *)a.xt + (((long)n * (g.Cin / RC) + c0 / RC) * slab_px) * RC + (c0 % RC);
@@ -439,121 +464,146 @@ __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
         // (opaque to the optimiser: it would otherwise move the position arithmetic of all taps
         // out of the channel loop and spill what that keeps alive)
         asm volatile("" : "+v"(dy), "+v"(dx));
-        const float m = mask_value<E>(t_m[tap], a.om.logit);
         const float py = (float)(ho * g.sh - g.ph + ti * g.dh) + dy;
         const float px = (float)(wo * g.sw - g.pw + tj * g.dw) + dx;
         const bool inside =
             valid && (py > -1.0f) && (px > -1.0f) && (py < (float)g.H) && (px < (float)g.W);
-        E *crow = cbase + (long)tap * g.cin_g * a.P_pad;
-        if (inside) {
-          const float fy = floorf(py), fx = floorf(px);
-          const int y0 = (int)fy, x0 = (int)fx, y1 = y0 + 1, x1 = x0 + 1;
-          const float ly = py - fy, lx = px - fx, hy = 1.0f - ly, hx = 1.0f - lx;
-          const bool ok00 = y0 >= 0 && x0 >= 0, ok01 = y0 >= 0 && x1 <= g.W - 1;
-          const bool ok10 = y1 <= g.H - 1 && x0 >= 0, ok11 = y1 <= g.H - 1 && x1 <= g.W - 1;
-          // corners outside the image read the copy's zero border
-          const E *xp = xbase + ((long)(y0 + 1) * g.Wp + (x0 + 1)) * RC;
-          VecCh<E, CH> r00, r01, r10, r11;
-          r00.load(xp);
-          r01.load(xp + RC);
-          r10.load(xp + (long)g.Wp * RC);
-          r11.load(xp + (long)(g.Wp + 1) * RC);
-          float v00[CH], v01[CH], v10[CH], v11[CH];
-          r00.unpack(v00);
-          r01.unpack(v01);
-          r10.unpack(v10);
-          r11.unpack(v11);
-          const float w00 = hy * hx, w01 = hy * lx, w10 = ly * hx, w11 = ly * lx;
-          if (a.col) {
+        // No branch around the body: a position outside the sampling range (or a lane past the
+        // image) samples the border's corner pixel with weights, mask and d of zero, so it stores
+        // a column of zeros and adds zeros.  Per-corner conditions become weights of zero too: a
+        // wavefront pays for an LDS atomic whether or not a lane sits it out, and a branch per
+        // corner and channel was most of the instructions this kernel issued.
+        const float fy = floorf(py), fx = floorf(px);
+        const int y0 = inside ? (int)fy : -1, x0 = inside ? (int)fx : -1, y1 = y0 + 1, x1 = x0 + 1;
+        const float ly = inside ? py - fy : 0.0f, lx = inside ? px - fx : 0.0f, hy = 1.0f - ly, hx = 1.0f - lx;
+        const float m = inside ? mask_value<E>(t_m[tap], a.om.logit) : 0.0f;
+        const bool ok00 = y0 >= 0 && x0 >= 0, ok01 = y0 >= 0 && x1 <= g.W - 1;
+        const bool ok10 = y1 <= g.H - 1 && x0 >= 0, ok11 = y1 <= g.H - 1 && x1 <= g.W - 1;
+        // corners outside the image read the copy's zero border
+        const E *xp = xbase + ((long)(y0 + 1) * g.Wp + (x0 + 1)) * RC;
+        VecCh<E, CH> r00, r01, r10, r11;
+        r00.load(xp);
+        r01.load(xp + RC);
+        r10.load(xp + (long)g.Wp * RC);
+        r11.load(xp + (long)(g.Wp + 1) * RC);
+        VecCh<E, CH> rd;
+        if (data) rd.load(dbase + (long)tap * plane_out * 16);
+        float v00[CH], v01[CH], v10[CH], v11[CH];
+        r00.unpack(v00);
+        r01.unpack(v01);
+        r10.unpack(v10);
+        r11.unpack(v11);
+        const float w00 = hy * hx, w01 = hy * lx, w10 = ly * hx, w11 = ly * lx;
+        if (a.col) {
+          E cv[CH];
 #pragma unroll
-            for (int cc = 0; cc < CH; ++cc)
-              crow[(long)cc * a.P_pad] =
-                  from_f32<E>(m * (w00 * v00[cc] + w01 * v01[cc] + w10 * v10[cc] + w11 * v11[cc]));
+          for (int cc = 0; cc < CH; ++cc)
+            cv[cc] = from_f32<E>(m * (w00 * v00[cc] + w01 * v01[cc] + w10 * v10[cc] + w11 * v11[cc]));
+          if (valid) {
+            E *crow = cbase + (long)tap * g.cin_g * a.P_pad;
+#pragma unroll
+            for (int cc = 0; cc < CH; ++cc) crow[(long)cc * a.P_pad] = cv[cc];
           }
-          if (data) {
-            VecCh<E, CH> rd;
-            rd.load(dbase + (long)tap * plane_out * 16);
-            float d[CH];
-            rd.unpack(d);
-            const int ry = y0 - wy0, rx = x0 - wx0;
-            const bool in_win = ry >= 0 && ry + 1 < a.WH && rx >= 0 && rx + 1 < a.WW;
-            const int wbase = ry * a.WW + rx;  // window is [channel][WH][WW]: neighbouring pixels, neighbouring banks
+        }
+        if (data) {
+          const uint32_t keep = inside ? ~0u : 0u;  // (whatever d holds where nothing is sampled)
+#pragma unroll
+          for (int i = 0; i < VecCh<E, CH>::NW; ++i) rd.raw[i] &= keep;
+          float d[CH];
+          rd.unpack(d);
+          const int ry = y0 - wy0, rx = x0 - wx0;
+          const bool in_win = ry >= 0 && ry + 1 < a.WH && rx >= 0 && rx + 1 < a.WW;
+          const bool to_win = inside && in_win;
+          // window is [channel][WH][WW]: neighbouring pixels, neighbouring banks; a lane with nothing
+          // for the window adds its zeros at an entry of its own
+          const int wbase = to_win ? ry * a.WW + rx : (tid & 63);
+          const float s00 = (to_win && ok00) ? w00 : 0.0f, s01 = (to_win && ok01) ? w01 : 0.0f;
+          const float s10 = (to_win && ok10) ? w10 : 0.0f, s11 = (to_win && ok11) ? w11 : 0.0f;
+          const float mts = m * fx_scale;
+          float am = 0.0f, ay = 0.0f, ax = 0.0f;
+          // fixed point: the even channel's four contributions wait here for the odd channel's
+          int q00 = 0, q01 = 0, q10 = 0, q11 = 0;
+#pragma unroll
+          for (int cc = 0; cc < CH; ++cc) {
+            const float dc = d[cc];
+            am += dc * (w00 * v00[cc] + w01 * v01[cc] + w10 * v10[cc] + w11 * v11[cc]);
+            ay += dc * (hx * (v10[cc] - v00[cc]) + lx * (v11[cc] - v01[cc]));
+            ax += dc * (hy * (v01[cc] - v00[cc]) + ly * (v11[cc] - v10[cc]));
+            if constexpr (kFixed) {
+              // round(w * ts) to nearest even in one multiply-add: the sum's mantissa holds the integer
+              // (|w * ts| < 2^19 by the choice of the scale)
+              const float ts = dc * mts;
+              auto fix = [](float w, float t) { return __float_as_int(fmaf(w, t, 12582912.0f)) - 0x4B400000; };
+              const int f00 = fix(s00, ts), f01 = fix(s01, ts), f10 = fix(s10, ts), f11 = fix(s11, ts);
+              if ((cc & 1) == 0) {
+                q00 = f00, q01 = f01, q10 = f10, q11 = f11;
+              } else {
+                unsigned long long *wp = (unsigned long long *)win + (cc >> 1) * win_px + wbase;
+                auto both = [](int lo, int hi) {
+                  return (unsigned long long)((long long)lo + (long long)((unsigned long long)(unsigned)hi << 32));
+                };
+                atomicAdd(wp, both(q00, f00));
+                atomicAdd(wp + 1, both(q01, f01));
+                atomicAdd(wp + a.WW, both(q10, f10));
+                atomicAdd(wp + a.WW + 1, both(q11, f11));
+              }
+            } else {
+              const float t = dc * m;
+              WT *wp = win + cc * win_px + wbase;
+              atomicAdd(wp, (WT)(s00 * t));
+              atomicAdd(wp + 1, (WT)(s01 * t));
+              atomicAdd(wp + a.WW, (WT)(s10 * t));
+              atomicAdd(wp + a.WW + 1, (WT)(s11 * t));
+            }
+          }
+          acc_m[tap] += am;
+          acc_y[tap] += ay * m;
+          acc_x[tap] += ax * m;
+          if (inside && !in_win) {  // rare: corners beyond the window go to memory directly
             const long o00 = (long)y0 * g.W + x0, o01 = o00 + 1, o10 = o00 + g.W, o11 = o10 + 1;
-            float am = 0.0f, ay = 0.0f, ax = 0.0f;
-            // fixed point: the even channel's four contributions wait here for the odd channel's
-            int q00 = 0, q01 = 0, q10 = 0, q11 = 0;
 #pragma unroll
             for (int cc = 0; cc < CH; ++cc) {
-              const float dc = d[cc];
-              am += dc * (w00 * v00[cc] + w01 * v01[cc] + w10 * v10[cc] + w11 * v11[cc]);
-              ay += dc * (hx * (v10[cc] - v00[cc]) + lx * (v11[cc] - v01[cc]));
-              ax += dc * (hy * (v01[cc] - v00[cc]) + ly * (v11[cc] - v10[cc]));
-              const float t = dc * m;
-              if (in_win) {
-                if constexpr (kFixed) {
-                  const float ts = t * fx_scale;
-                  const int r00 = __float2int_rn(w00 * ts), r01 = __float2int_rn(w01 * ts);
-                  const int r10 = __float2int_rn(w10 * ts), r11 = __float2int_rn(w11 * ts);
-                  if ((cc & 1) == 0) {
-                    q00 = r00, q01 = r01, q10 = r10, q11 = r11;
-                  } else {
-                    unsigned long long *wp = (unsigned long long *)win + (cc >> 1) * win_px + wbase;
-                    auto both = [](int lo, int hi) {
-                      return (unsigned long long)((long long)lo + (long long)((unsigned long long)(unsigned)hi << 32));
-                    };
-                    if (ok00) atomicAdd(wp, both(q00, r00));
-                    if (ok01) atomicAdd(wp + 1, both(q01, r01));
-                    if (ok10) atomicAdd(wp + a.WW, both(q10, r10));
-                    if (ok11) atomicAdd(wp + a.WW + 1, both(q11, r11));
-                  }
-                } else {
-                  WT *wp = win + cc * win_px + wbase;
-                  if (ok00) atomicAdd(wp, (WT)(w00 * t));
-                  if (ok01) atomicAdd(wp + 1, (WT)(w01 * t));
-                  if (ok10) atomicAdd(wp + a.WW, (WT)(w10 * t));
-                  if (ok11) atomicAdd(wp + a.WW + 1, (WT)(w11 * t));
-                }
-              } else {
-                float *gi = a.gin32 + ((long)n * g.Cin + c0 + cc) * plane_in;
-                if (ok00) unsafeAtomicAdd(gi + o00, w00 * t);
-                if (ok01) unsafeAtomicAdd(gi + o01, w01 * t);
-                if (ok10) unsafeAtomicAdd(gi + o10, w10 * t);
-                if (ok11) unsafeAtomicAdd(gi + o11, w11 * t);
-              }
+              const float t = d[cc] * m;
+              float *gi = a.gin32 + ((long)n * g.Cin + c0 + cc) * plane_in;
+              if (ok00) unsafeAtomicAdd(gi + o00, w00 * t);
+              if (ok01) unsafeAtomicAdd(gi + o01, w01 * t);
+              if (ok10) unsafeAtomicAdd(gi + o10, w10 * t);
+              if (ok11) unsafeAtomicAdd(gi + o11, w11 * t);
             }
-            acc_m[tap] += am;
-            acc_y[tap] += ay * m;
-            acc_x[tap] += ax * m;
           }
-        } else if (valid && a.col) {  // a position outside the sampling range: a column of zeros
-#pragma unroll
-          for (int cc = 0; cc < CH; ++cc) crow[(long)cc * a.P_pad] = from_f32<E>(0.0f);
         }
       }
     }
     if (data) {
       __syncthreads();  // every add into the window has landed
-      if constexpr (kFixed) {
-        const long long *w64 = (const long long *)win;
-        for (int i = tid; i < win_px * (CH / 2); i += 256) {
-          const long long e = w64[i];
-          if (e != 0) {
-            const int lo = (int)(unsigned)(unsigned long long)e;
-            const int hi = (int)((e - (long long)lo) >> 32);
-            const int cp = i / win_px, q = i - cp * win_px;
-            const int y = wy0 + q / a.WW, x = wx0 + q % a.WW;  // in the image: only valid corners were added
-            float *gi = a.gin32 + ((long)n * g.Cin + c0 + 2 * cp) * plane_in + (long)y * g.W + x;
-            if (lo != 0) unsafeAtomicAdd(gi, (float)lo * fx_inv);
-            if (hi != 0) unsafeAtomicAdd(gi + plane_in, (float)hi * fx_inv);
-          }
-        }
-      } else {
-        for (int i = tid; i < win_px * CH; i += 256) {
-          const float v = (float)win[i];
-          if (v != 0.0f) {
-            const int cc = i / win_px, q = i - cc * win_px;
-            const int y = wy0 + q / a.WW, x = wx0 + q % a.WW;  // in the image: only valid corners were added
-            unsafeAtomicAdd(a.gin32 + ((long)n * g.Cin + c0 + cc) * plane_in + (long)y * g.W + x, v);
+      float *gplane = a.gin32 + ((long)n * g.Cin + c0) * plane_in;
+#pragma unroll
+      for (int j = 0; j < kSlots; ++j) {
+        if (flush_at[j] >= 0) {
+          const int q = tid + 256 * j;
+          float *gi = gplane + flush_at[j];
+          if constexpr (kFixed) {
+            long long *w64 = (long long *)win + q;
+#pragma unroll
+            for (int cp = 0; cp < NE; ++cp) {
+              const long long e = w64[cp * win_px];
+              if (e != 0) {
+                w64[cp * win_px] = 0;
+                const int lo = (int)(unsigned)(unsigned long long)e;
+                const int hi = (int)((e - (long long)lo) >> 32);
+                if (lo != 0) unsafeAtomicAdd(gi + (long)(2 * cp) * plane_in, (float)lo * fx_inv);
+                if (hi != 0) unsafeAtomicAdd(gi + (long)(2 * cp + 1) * plane_in, (float)hi * fx_inv);
+              }
+            }
+          } else {
+#pragma unroll
+            for (int cc = 0; cc < NE; ++cc) {
+              const WT v = win[cc * win_px + q];
+              if (v != (WT)0) {
+                win[cc * win_px + q] = (WT)0;
+                unsafeAtomicAdd(gi + (long)cc * plane_in, (float)v);
+              }
+            }
           }
         }
       }
