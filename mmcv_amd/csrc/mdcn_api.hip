@@ -1009,10 +1009,19 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
         using WT = typename std::conditional<k16, int32_t, double>::type;
         constexpr int CHB = k16 ? 16 : 8;
         const dim3 sgrid((unsigned)sblocks, (unsigned)sa.parts);
+        auto launch = [&](auto chv) {
+          constexpr int CHS = decltype(chv)::value;
+          if (gemm && wgemm)
+            hipLaunchKernelGGL((bwd_scatter_kernel<E, CHS, WT, true, true>), sgrid, dim3(256), 0, st, sa);
+          else if (gemm)
+            hipLaunchKernelGGL((bwd_scatter_kernel<E, CHS, WT, true, false>), sgrid, dim3(256), 0, st, sa);
+          else
+            hipLaunchKernelGGL((bwd_scatter_kernel<E, CHS, WT, false, true>), sgrid, dim3(256), 0, st, sa);
+        };
         if (pl.sCH == CHB)
-          hipLaunchKernelGGL((bwd_scatter_kernel<E, CHB, WT>), sgrid, dim3(256), 0, st, sa);
+          launch(std::integral_constant<int, CHB>());
         else
-          hipLaunchKernelGGL((bwd_scatter_kernel<E, CHB / 2, WT>), sgrid, dim3(256), 0, st, sa);
+          launch(std::integral_constant<int, CHB / 2>());
       }
       check();
       if (wgemm) {

@@ -287,6 +287,24 @@ struct VecCh {
       raw[1] = v.y;
     }
   }
+  // channels 2 i and 2 i + 1
+  __device__ __forceinline__ void pair(int i, float &lo, float &hi) const {
+    if constexpr (sizeof(E) == 4) {
+      lo = __uint_as_float(raw[2 * i]);
+      hi = __uint_as_float(raw[2 * i + 1]);
+    } else {
+      ElemTraits<E>::unpack2(raw[i], lo, hi);
+    }
+  }
+  // acc + this's channels 2 i and 2 i + 1 times o's
+  __device__ __forceinline__ float dot_pair(const VecCh &o, int i, float acc) const {
+    if constexpr (sizeof(E) == 4) {
+      acc = fmaf(__uint_as_float(raw[2 * i]), __uint_as_float(o.raw[2 * i]), acc);
+      return fmaf(__uint_as_float(raw[2 * i + 1]), __uint_as_float(o.raw[2 * i + 1]), acc);
+    } else {
+      return ElemTraits<E>::dot2(raw[i], o.raw[i], acc);
+    }
+  }
   __device__ __forceinline__ void unpack(float (&out)[CH]) const {
     if constexpr (sizeof(E) == 4) {
 #pragma unroll
@@ -373,17 +391,20 @@ __global__ __launch_bounds__(256) void combine_parts_kernel(const float *__restr
 // With a.col the kernel also stores the forward's columns (mask * bilinear
 // sample, rounded to E as the reference's columns tensor is) for the
 // weight-gradient product; with a.D == null that is all it does.
-template <typename E, int CH, typename WT>
+// DATA: the gradient part (a.D, window, offset / mask sums); COL: the columns
+// part (a.col).  At least one of them.
+template <typename E, int CH, typename WT, bool DATA, bool COL>
 __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
   constexpr int RC = 32 / (int)sizeof(E);   // channels per record of the input copy
+  static_assert(DATA || COL, "nothing to do");
   static_assert(CH <= RC && RC % CH == 0, "a pass reads a record or a whole fraction of one");
   static_assert(CH % 2 == 0, "fixed-point window entries hold two channels");
   constexpr bool kFixed = sizeof(WT) == 4;
   static_assert(kScTH * kScTW == 256, "one thread per pixel of the tile");
   static_assert(kScTH * kScTW * kBwdTapsMax <= kScMaxAdds, "bound on the adds per window entry");
-  __shared__ __align__(16) WT win[kScWindowBytes / sizeof(WT)];
+  __shared__ __align__(16) WT win[DATA ? kScWindowBytes / sizeof(WT) : 4];
   float fx_scale = 1.0f, fx_inv = 1.0f;
-  if (kFixed && a.D != nullptr) {
+  if (kFixed && DATA) {
     const float bound = __uint_as_float(*a.dmax) * (a.mmax ? __uint_as_float(*a.mmax) : 1.0f) * (float)kScMaxAdds;
     // largest power of two not above 2^30 / bound (any scale will do when everything is zero)
     const int e = (bound > 0.0f && bound < 3.0e38f) ? 29 - ilogbf(bound) : 0;
@@ -408,7 +429,6 @@ __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
   const long pix = valid ? (long)ho * g.Wo + wo : 0;
   const int wy0 = ty * kScTH * g.sh - g.ph - a.R, wx0 = tx * kScTW * g.sw - g.pw - a.R;
   const int win_px = a.WH * a.WW;
-  const bool data = a.D != nullptr;  // workgroup uniform
 
   const E *off = (const E *)a.om.off + (long)n * a.om.off_n + pix * a.om.off_px +
                  (long)(dgi * 2 * g.taps) * a.om.off_ch;
@@ -419,7 +439,7 @@ __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
 #pragma unroll
   for (int t = 0; t < kBwdTapsMax; ++t) acc_m[t] = acc_y[t] = acc_x[t] = 0.0f;
   // this pixel's offsets and mask, fetched once: every channel pass needs them before it can
-  // address its corners, and a load there would also wait for the pass's older stores
+  // address its corners
   E t_dy[kBwdTapsMax], t_dx[kBwdTapsMax], t_m[kBwdTapsMax];
 #pragma unroll
   for (int t = 0; t < kBwdTapsMax; ++t) {
@@ -436,131 +456,170 @@ __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
   // Window pixels this thread flushes (tid, tid + 256, ...) as offsets into an image plane, the same
   // in every pass; -1 for one outside the image or past the window (it only ever receives zeros).
   constexpr int NE = kFixed ? CH / 2 : CH;  // window entries per pixel
-  constexpr int kSlots = (kScWindowBytes / (NE * 8) + 255) / 256;
+  constexpr int kSlots = DATA ? (kScWindowBytes / (NE * 8) + 255) / 256 : 1;
   int flush_at[kSlots];
+  if constexpr (DATA) {
 #pragma unroll
-  for (int j = 0; j < kSlots; ++j) {
-    const int q = tid + 256 * j;
-    const int y = wy0 + q / a.WW, x = wx0 + q % a.WW;
-    flush_at[j] = (q < win_px && y >= 0 && y < g.H && x >= 0 && x < g.W) ? y * g.W + x : -1;
-  }
-  if (data)  // the flush leaves the window zeroed for the next pass
+    for (int j = 0; j < kSlots; ++j) {
+      const int q = tid + 256 * j;
+      const int y = wy0 + q / a.WW, x = wx0 + q % a.WW;
+      flush_at[j] = (q < win_px && y >= 0 && y < g.H && x >= 0 && x < g.W) ? y * g.W + x : -1;
+    }
+    // (the flush leaves the window zeroed for the next pass)
     for (int i = tid; i < kScWindowBytes / 16; i += 256) ((uint4 *)win)[i] = make_uint4(0u, 0u, 0u, 0u);
+  }
+
+  // One tap's sampling position and what was loaded there.  No branch around a tap's body: a
+  // position outside the sampling range (or a lane past the image) samples the border's corner
+  // pixel with weights, mask and d of zero, so it stores a column of zeros and adds zeros.
+  // Per-corner conditions become weights of zero too: a wavefront pays for an LDS atomic
+  // whether or not a lane sits it out, and a branch per corner and channel was most of the
+  // instructions this kernel issued.
+  struct Sample {
+    int y0, x0;
+    float ly, lx, m;
+    bool inside;
+    VecCh<E, CH> r00, r01, r10, r11, rd;
+  };
+  auto fetch = [&](int c0, int tap, E e_dy, E e_dx, E e_m, Sample &s) {
+    const int ti = tap / g.kw, tj = tap - ti * g.kw;
+    float dy = to_f32(e_dy);
+    float dx = to_f32(e_dx);
+    // (opaque to the optimiser: it would otherwise move the position arithmetic of all taps
+    // out of the channel loop and spill what that keeps alive)
+    asm volatile("" : "+v"(dy), "+v"(dx));
+    const float py = (float)(ho * g.sh - g.ph + ti * g.dh) + dy;
+    const float px = (float)(wo * g.sw - g.pw + tj * g.dw) + dx;
+    s.inside = valid && (py > -1.0f) && (px > -1.0f) && (py < (float)g.H) && (px < (float)g.W);
+    const float fy = floorf(py), fx = floorf(px);
+    s.y0 = s.inside ? (int)fy : -1;
+    s.x0 = s.inside ? (int)fx : -1;
+    s.ly = s.inside ? py - fy : 0.0f;
+    s.lx = s.inside ? px - fx : 0.0f;
+    s.m = s.inside ? mask_value<E>(e_m, a.om.logit) : 0.0f;
+    // corners outside the image read the copy's zero border
+    const E *xp = (const E *)a.xt + (((long)n * (g.Cin / RC) + c0 / RC) * slab_px) * RC + (c0 % RC) +
+                  ((long)(s.y0 + 1) * g.Wp + (s.x0 + 1)) * RC;
+    s.r00.load(xp);
+    s.r01.load(xp + RC);
+    s.r10.load(xp + (long)g.Wp * RC);
+    s.r11.load(xp + (long)(g.Wp + 1) * RC);
+    if constexpr (DATA)
+      s.rd.load((const E *)a.D + (((long)nl * (g.Cin / 16) + (c0 >> 4)) * g.taps + tap) * plane_out * 16 + pix * 16 +
+                (c0 & 15));
+  };
+  // A tap's loads are issued one tap ahead, in front of the previous tap's stores and atomics
+  // (a wait for loads also waits for every older store, and the compiler cannot move a load
+  // above a store that might alias it); the last tap of a pass fetches the first of the next.
+  Sample cur;
+  fetch(c_begin, 0, t_dy[0], t_dx[0], t_m[0], cur);
 
   for (int c0 = c_begin; c0 < c_end; c0 += CH) {
-    if (data) __syncthreads();  // the window is zero: first fill or the previous pass's flush
-    const E *dbase = (const E *)a.D + (((long)nl * (g.Cin / 16) + (c0 >> 4)) * g.taps) * plane_out * 16 + pix * 16 +
-                     (c0 & 15);
-    const E *xbase = (const E *)a.xt + (((long)n * (g.Cin / RC) + c0 / RC) * slab_px) * RC + (c0 % RC);
+    if constexpr (DATA) __syncthreads();  // the window is zero: first fill or the previous pass's flush
     // row of the columns matrix of channel c0 at tap 0 (a chunk stays inside one group)
     const int grp = c0 / g.cin_g;
     E *cbase = (E *)a.col + (((long)nl * g.Cin + (long)grp * g.cin_g) * g.taps + (c0 - grp * g.cin_g)) * a.P_pad + pix;
+    const int c_next = min(c0 + CH, c_end - CH);  // (the last pass fetches its own first tap again: unused)
 #pragma unroll
     for (int tap = 0; tap < kBwdTapsMax; ++tap) {
       if (tap < g.taps) {
-        const int ti = tap / g.kw, tj = tap - ti * g.kw;
-        float dy = to_f32(t_dy[tap]);
-        float dx = to_f32(t_dx[tap]);
-        // (opaque to the optimiser: it would otherwise move the position arithmetic of all taps
-        // out of the channel loop and spill what that keeps alive)
-        asm volatile("" : "+v"(dy), "+v"(dx));
-        const float py = (float)(ho * g.sh - g.ph + ti * g.dh) + dy;
-        const float px = (float)(wo * g.sw - g.pw + tj * g.dw) + dx;
-        const bool inside =
-            valid && (py > -1.0f) && (px > -1.0f) && (py < (float)g.H) && (px < (float)g.W);
-        // No branch around the body: a position outside the sampling range (or a lane past the
-        // image) samples the border's corner pixel with weights, mask and d of zero, so it stores
-        // a column of zeros and adds zeros.  Per-corner conditions become weights of zero too: a
-        // wavefront pays for an LDS atomic whether or not a lane sits it out, and a branch per
-        // corner and channel was most of the instructions this kernel issued.
-        const float fy = floorf(py), fx = floorf(px);
-        const int y0 = inside ? (int)fy : -1, x0 = inside ? (int)fx : -1, y1 = y0 + 1, x1 = x0 + 1;
-        const float ly = inside ? py - fy : 0.0f, lx = inside ? px - fx : 0.0f, hy = 1.0f - ly, hx = 1.0f - lx;
-        const float m = inside ? mask_value<E>(t_m[tap], a.om.logit) : 0.0f;
+        Sample nxt;
+        {
+          const bool more = tap + 1 < g.taps;  // workgroup uniform
+          const int tn = tap + 1 < kBwdTapsMax ? tap + 1 : 0;  // (a constant once the loop is unrolled)
+          fetch(more ? c0 : c_next, more ? tn : 0, more ? t_dy[tn] : t_dy[0], more ? t_dx[tn] : t_dx[0],
+                more ? t_m[tn] : t_m[0], nxt);
+        }
+        const bool inside = cur.inside;
+        const int y0 = cur.y0, x0 = cur.x0, y1 = y0 + 1, x1 = x0 + 1;
+        const float ly = cur.ly, lx = cur.lx, hy = 1.0f - ly, hx = 1.0f - lx, m = cur.m;
         const bool ok00 = y0 >= 0 && x0 >= 0, ok01 = y0 >= 0 && x1 <= g.W - 1;
         const bool ok10 = y1 <= g.H - 1 && x0 >= 0, ok11 = y1 <= g.H - 1 && x1 <= g.W - 1;
-        // corners outside the image read the copy's zero border
-        const E *xp = xbase + ((long)(y0 + 1) * g.Wp + (x0 + 1)) * RC;
-        VecCh<E, CH> r00, r01, r10, r11;
-        r00.load(xp);
-        r01.load(xp + RC);
-        r10.load(xp + (long)g.Wp * RC);
-        r11.load(xp + (long)(g.Wp + 1) * RC);
-        VecCh<E, CH> rd;
-        if (data) rd.load(dbase + (long)tap * plane_out * 16);
-        float v00[CH], v01[CH], v10[CH], v11[CH];
-        r00.unpack(v00);
-        r01.unpack(v01);
-        r10.unpack(v10);
-        r11.unpack(v11);
         const float w00 = hy * hx, w01 = hy * lx, w10 = ly * hx, w11 = ly * lx;
-        if (a.col) {
-          E cv[CH];
+        VecCh<E, CH> &rd = cur.rd;
+        if constexpr (DATA) {
+          const uint32_t keep = inside ? ~0u : 0u;  // (whatever d holds where nothing is sampled)
 #pragma unroll
-          for (int cc = 0; cc < CH; ++cc)
-            cv[cc] = from_f32<E>(m * (w00 * v00[cc] + w01 * v01[cc] + w10 * v10[cc] + w11 * v11[cc]));
+          for (int i = 0; i < VecCh<E, CH>::NW; ++i) rd.raw[i] &= keep;
+        }
+        const int ry = y0 - wy0, rx = x0 - wx0;
+        const bool in_win = ry >= 0 && ry + 1 < a.WH && rx >= 0 && rx + 1 < a.WW;
+        const bool to_win = inside && in_win;
+        // window is [channel][WH][WW]: neighbouring pixels, neighbouring banks; a lane with nothing
+        // for the window adds its zeros at an entry of its own
+        const int wbase = to_win ? ry * a.WW + rx : (tid & 63);
+        const float s00 = (to_win && ok00) ? w00 : 0.0f, s01 = (to_win && ok01) ? w01 : 0.0f;
+        const float s10 = (to_win && ok10) ? w10 : 0.0f, s11 = (to_win && ok11) ? w11 : 0.0f;
+        const float mts = m * fx_scale;
+        // sums over the pass's channels of d times each corner's value: the offset and mask
+        // gradients are combinations of these four
+        float S00 = 0.0f, S01 = 0.0f, S10 = 0.0f, S11 = 0.0f;
+        E cv[CH];
+        // two channels at a time, straight from the loaded words
+#pragma unroll
+        for (int cp = 0; cp < CH / 2; ++cp) {
+          if constexpr (DATA) {
+            S00 = cur.r00.dot_pair(rd, cp, S00);
+            S01 = cur.r01.dot_pair(rd, cp, S01);
+            S10 = cur.r10.dot_pair(rd, cp, S10);
+            S11 = cur.r11.dot_pair(rd, cp, S11);
+          }
+          if constexpr (COL) {
+            float v00[2], v01[2], v10[2], v11[2];
+            cur.r00.pair(cp, v00[0], v00[1]);
+            cur.r01.pair(cp, v01[0], v01[1]);
+            cur.r10.pair(cp, v10[0], v10[1]);
+            cur.r11.pair(cp, v11[0], v11[1]);
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+              cv[2 * cp + h] = from_f32<E>(m * (w00 * v00[h] + w01 * v01[h] + w10 * v10[h] + w11 * v11[h]));
+          }
+          if constexpr (DATA) {
+            float d[2];
+            rd.pair(cp, d[0], d[1]);
+            if constexpr (kFixed) {
+              // round(w * ts) to nearest even in one multiply-add: the sum's mantissa holds the
+              // integer (|w * ts| < 2^19 by the choice of the scale).  An entry is the even
+              // channel's value sign-extended plus the odd one's shifted up 32 bits.
+              const float tl = d[0] * mts, th = d[1] * mts;
+              auto entry = [](float w, float tl, float th) {
+                const int lo = __float_as_int(fmaf(w, tl, 12582912.0f)) - 0x4B400000;
+                const uint32_t hi = (uint32_t)__float_as_int(fmaf(w, th, 12582912.0f)) - 0x4B400000u + (uint32_t)(lo >> 31);
+                return (unsigned long long)(uint32_t)lo | ((unsigned long long)hi << 32);
+              };
+              unsigned long long *wp = (unsigned long long *)win + cp * win_px + wbase;
+              atomicAdd(wp, entry(s00, tl, th));
+              atomicAdd(wp + 1, entry(s01, tl, th));
+              atomicAdd(wp + a.WW, entry(s10, tl, th));
+              atomicAdd(wp + a.WW + 1, entry(s11, tl, th));
+            } else {
+#pragma unroll
+              for (int h = 0; h < 2; ++h) {
+                const float t = d[h] * m;
+                WT *wp = win + (2 * cp + h) * win_px + wbase;
+                atomicAdd(wp, (WT)(s00 * t));
+                atomicAdd(wp + 1, (WT)(s01 * t));
+                atomicAdd(wp + a.WW, (WT)(s10 * t));
+                atomicAdd(wp + a.WW + 1, (WT)(s11 * t));
+              }
+            }
+          }
+        }
+        if constexpr (COL) {
           if (valid) {
             E *crow = cbase + (long)tap * g.cin_g * a.P_pad;
 #pragma unroll
             for (int cc = 0; cc < CH; ++cc) crow[(long)cc * a.P_pad] = cv[cc];
           }
         }
-        if (data) {
-          const uint32_t keep = inside ? ~0u : 0u;  // (whatever d holds where nothing is sampled)
-#pragma unroll
-          for (int i = 0; i < VecCh<E, CH>::NW; ++i) rd.raw[i] &= keep;
-          float d[CH];
-          rd.unpack(d);
-          const int ry = y0 - wy0, rx = x0 - wx0;
-          const bool in_win = ry >= 0 && ry + 1 < a.WH && rx >= 0 && rx + 1 < a.WW;
-          const bool to_win = inside && in_win;
-          // window is [channel][WH][WW]: neighbouring pixels, neighbouring banks; a lane with nothing
-          // for the window adds its zeros at an entry of its own
-          const int wbase = to_win ? ry * a.WW + rx : (tid & 63);
-          const float s00 = (to_win && ok00) ? w00 : 0.0f, s01 = (to_win && ok01) ? w01 : 0.0f;
-          const float s10 = (to_win && ok10) ? w10 : 0.0f, s11 = (to_win && ok11) ? w11 : 0.0f;
-          const float mts = m * fx_scale;
-          float am = 0.0f, ay = 0.0f, ax = 0.0f;
-          // fixed point: the even channel's four contributions wait here for the odd channel's
-          int q00 = 0, q01 = 0, q10 = 0, q11 = 0;
-#pragma unroll
-          for (int cc = 0; cc < CH; ++cc) {
-            const float dc = d[cc];
-            am += dc * (w00 * v00[cc] + w01 * v01[cc] + w10 * v10[cc] + w11 * v11[cc]);
-            ay += dc * (hx * (v10[cc] - v00[cc]) + lx * (v11[cc] - v01[cc]));
-            ax += dc * (hy * (v01[cc] - v00[cc]) + ly * (v11[cc] - v10[cc]));
-            if constexpr (kFixed) {
-              // round(w * ts) to nearest even in one multiply-add: the sum's mantissa holds the integer
-              // (|w * ts| < 2^19 by the choice of the scale)
-              const float ts = dc * mts;
-              auto fix = [](float w, float t) { return __float_as_int(fmaf(w, t, 12582912.0f)) - 0x4B400000; };
-              const int f00 = fix(s00, ts), f01 = fix(s01, ts), f10 = fix(s10, ts), f11 = fix(s11, ts);
-              if ((cc & 1) == 0) {
-                q00 = f00, q01 = f01, q10 = f10, q11 = f11;
-              } else {
-                unsigned long long *wp = (unsigned long long *)win + (cc >> 1) * win_px + wbase;
-                auto both = [](int lo, int hi) {
-                  return (unsigned long long)((long long)lo + (long long)((unsigned long long)(unsigned)hi << 32));
-                };
-                atomicAdd(wp, both(q00, f00));
-                atomicAdd(wp + 1, both(q01, f01));
-                atomicAdd(wp + a.WW, both(q10, f10));
-                atomicAdd(wp + a.WW + 1, both(q11, f11));
-              }
-            } else {
-              const float t = dc * m;
-              WT *wp = win + cc * win_px + wbase;
-              atomicAdd(wp, (WT)(s00 * t));
-              atomicAdd(wp + 1, (WT)(s01 * t));
-              atomicAdd(wp + a.WW, (WT)(s10 * t));
-              atomicAdd(wp + a.WW + 1, (WT)(s11 * t));
-            }
-          }
-          acc_m[tap] += am;
-          acc_y[tap] += ay * m;
-          acc_x[tap] += ax * m;
+        if constexpr (DATA) {
+          acc_m[tap] += w00 * S00 + w01 * S01 + w10 * S10 + w11 * S11;
+          acc_y[tap] += m * (hx * (S10 - S00) + lx * (S11 - S01));
+          acc_x[tap] += m * (hy * (S01 - S00) + ly * (S11 - S10));
           if (inside && !in_win) {  // rare: corners beyond the window go to memory directly
             const long o00 = (long)y0 * g.W + x0, o01 = o00 + 1, o10 = o00 + g.W, o11 = o10 + 1;
+            float d[CH];
+            rd.unpack(d);
 #pragma unroll
             for (int cc = 0; cc < CH; ++cc) {
               const float t = d[cc] * m;
@@ -572,9 +631,10 @@ __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
             }
           }
         }
+        cur = nxt;
       }
     }
-    if (data) {
+    if constexpr (DATA) {
       __syncthreads();  // every add into the window has landed
       float *gplane = a.gin32 + ((long)n * g.Cin + c0) * plane_in;
 #pragma unroll
@@ -609,28 +669,30 @@ __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
       }
     }
   }
-  if (valid && data) {
-    const long ob = ((long)n * g.DG + dgi) * 2 * g.taps;
-    const long mb = ((long)n * g.DG + dgi) * g.taps;
-    if (a.parts == 1) {
-      E *goff = (E *)a.goff, *gmask = (E *)a.gmask;
+  if constexpr (DATA) {
+    if (valid) {
+      const long ob = ((long)n * g.DG + dgi) * 2 * g.taps;
+      const long mb = ((long)n * g.DG + dgi) * g.taps;
+      if (a.parts == 1) {
+        E *goff = (E *)a.goff, *gmask = (E *)a.gmask;
 #pragma unroll
-      for (int tap = 0; tap < kBwdTapsMax; ++tap) {
-        if (tap < g.taps) {
-          goff[(ob + 2 * tap) * plane_out + pix] = from_f32<E>(acc_y[tap]);
-          goff[(ob + 2 * tap + 1) * plane_out + pix] = from_f32<E>(acc_x[tap]);
-          if (gmask) gmask[(mb + tap) * plane_out + pix] = from_f32<E>(acc_m[tap]);
+        for (int tap = 0; tap < kBwdTapsMax; ++tap) {
+          if (tap < g.taps) {
+            goff[(ob + 2 * tap) * plane_out + pix] = from_f32<E>(acc_y[tap]);
+            goff[(ob + 2 * tap + 1) * plane_out + pix] = from_f32<E>(acc_x[tap]);
+            if (gmask) gmask[(mb + tap) * plane_out + pix] = from_f32<E>(acc_m[tap]);
+          }
         }
-      }
-    } else {
-      float *poff = a.poff + (long)part * a.off_total;
-      float *pmask = a.gmask ? a.pmask + (long)part * a.mask_total : nullptr;
+      } else {
+        float *poff = a.poff + (long)part * a.off_total;
+        float *pmask = a.gmask ? a.pmask + (long)part * a.mask_total : nullptr;
 #pragma unroll
-      for (int tap = 0; tap < kBwdTapsMax; ++tap) {
-        if (tap < g.taps) {
-          poff[(ob + 2 * tap) * plane_out + pix] = acc_y[tap];
-          poff[(ob + 2 * tap + 1) * plane_out + pix] = acc_x[tap];
-          if (pmask) pmask[(mb + tap) * plane_out + pix] = acc_m[tap];
+        for (int tap = 0; tap < kBwdTapsMax; ++tap) {
+          if (tap < g.taps) {
+            poff[(ob + 2 * tap) * plane_out + pix] = acc_y[tap];
+            poff[(ob + 2 * tap + 1) * plane_out + pix] = acc_x[tap];
+            if (pmask) pmask[(mb + tap) * plane_out + pix] = acc_m[tap];
+          }
         }
       }
     }
