@@ -6,11 +6,12 @@
 // layout made for that kernel: d[image][16-channel chunk][tap][pixel][16].  The
 // scatter kernel (bwd_scatter_kernel) then is the reference's three element-wise
 // kernels in one pass (cpu/modulated_deform_conv.cpp:34-107,170-320): a thread
-// owns an output pixel, reads 8 channels of d and of the four corners (from the
-// zero-bordered pixel-major input copy, 16 or 32 contiguous bytes per corner),
-// forms its share of grad_offset / grad_mask in registers, and adds the
-// grad_input contributions into an LDS window around its 8 x 32 pixel tile,
-// which is flushed with one global atomic per non-zero entry.  On the way it can
+// owns an output pixel, reads 4 to 16 channels of d and of the four corners (from
+// the zero-bordered pixel-major input copy, 16 or 32 contiguous bytes per corner,
+// one tap ahead of their use), forms its share of grad_offset / grad_mask from
+// the four sums of d times a corner's values, and adds the grad_input
+// contributions into an LDS window around its 8 x 32 pixel tile, which is flushed
+// with one global atomic per non-zero entry.  On the way it can
 // store the forward's columns, from which grad_weight is a second plain product
 // (bwd_wgrad_kernel).
 // Both operands of the product are pixel-major / K-contiguous copies written by
@@ -388,11 +389,10 @@ __global__ __launch_bounds__(256) void combine_parts_kernel(const float *__restr
 // the high half cancel when the entry is taken apart again (low = the entry's low
 // word as a signed number, high = (entry - low) >> 32), since neither sum leaves
 // 32 bits.
-// With a.col the kernel also stores the forward's columns (mask * bilinear
-// sample, rounded to E as the reference's columns tensor is) for the
-// weight-gradient product; with a.D == null that is all it does.
-// DATA: the gradient part (a.D, window, offset / mask sums); COL: the columns
-// part (a.col).  At least one of them.
+// DATA: the gradient part (a.D, window, offset / mask sums).  COL: the kernel
+// stores the forward's columns (mask * bilinear sample, rounded to E as the
+// reference's columns tensor is) to a.col for the weight-gradient product.  At
+// least one of the two.
 template <typename E, int CH, typename WT, bool DATA, bool COL>
 __global__ __launch_bounds__(256, 2) void bwd_scatter_kernel(BwdScatterArgs a) {
   constexpr int RC = 32 / (int)sizeof(E);   // channels per record of the input copy
