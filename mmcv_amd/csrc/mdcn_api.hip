@@ -1055,7 +1055,7 @@ int run_backward_typed(const mdcn_bwd_params *bp, const Geom &g, const BwdPlan &
           hipLaunchKernelGGL((bwd_wgrad_kernel<E, kCgTile>), dim3((unsigned)((wa.total + 7) / 8 * 8)),
                              dim3(2 * kCgTile), 0, st, wa);
         check();
-        hipLaunchKernelGGL(wgrad_reduce_kernel, dim3(blocks_for(n_w)), dim3(256), 0, st, wpart, gw32, wa.splits,
+        hipLaunchKernelGGL(wgrad_reduce_kernel, dim3(blocks_for(n_w / 4 + 1)), dim3(256), 0, st, wpart, gw32, wa.splits,
                            g.cin_g, g.taps, n_w);
         check();
       }

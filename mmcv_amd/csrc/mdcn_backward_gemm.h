@@ -871,13 +871,30 @@ __global__ __launch_bounds__(TILE * 2, TILE == 128 ? 2 : 1) void bwd_wgrad_kerne
 __global__ __launch_bounds__(256) void wgrad_reduce_kernel(const float *__restrict__ part, float *__restrict__ gw32,
                                                            int splits, int cin_g, int taps, long n_w) {
   const int M = cin_g * taps;
-  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n_w; i += (long)gridDim.x * blockDim.x) {
+  // four consecutive elements per thread (M is a multiple of 32 here: they share a row and a tap), the shares
+  // in a fixed order with four loads in flight
+  for (long i = 4 * ((long)blockIdx.x * blockDim.x + threadIdx.x); i < n_w; i += 4 * (long)gridDim.x * blockDim.x) {
     const long row = i / M;  // (grp, co)
     const int m = (int)(i - row * M);
-    float sum = 0.0f;
-    for (int sp = 0; sp < splits; ++sp) sum += part[(long)sp * n_w + i];
+    float4 sum = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    int sp = 0;
+    for (; sp + 4 <= splits; sp += 4) {
+      float4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) v[u] = *(const float4 *)(part + (long)(sp + u) * n_w + i);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) sum.x += v[u].x, sum.y += v[u].y, sum.z += v[u].z, sum.w += v[u].w;
+    }
+    for (; sp < splits; ++sp) {
+      const float4 v = *(const float4 *)(part + (long)sp * n_w + i);
+      sum.x += v.x, sum.y += v.y, sum.z += v.z, sum.w += v.w;
+    }
     const int tap = m / cin_g, cl = m - tap * cin_g;
-    gw32[row * M + (long)cl * taps + tap] += sum;
+    float *dst = gw32 + row * M + (long)cl * taps + tap;
+    dst[0] += sum.x;
+    dst[taps] += sum.y;
+    dst[2 * taps] += sum.z;
+    dst[3 * taps] += sum.w;
   }
 }
 
